@@ -1,0 +1,77 @@
+// The C interface of the kernel library (one build per compute dtype, same symbols).
+//
+// Conventions: `elem` pointers hold the build's compute dtype (bfloat16 or float32); the
+// residual stream, logits and rotary tables are always float32; `*_is_f32` says how a gain
+// or bias vector is stored; `stream` is a hipStream_t.  Every function checks its shapes on
+// the host, launches on `stream` and returns 0, or a negative code with a message in
+// axk_last_error().  Nothing here allocates device memory.
+#pragma once
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* axk_last_error(void);
+// 1 for the bfloat16 build, 0 for float32; bytes of one element.
+int axk_is_bf16(void);
+int axk_elem_size(void);
+
+// x[t, :] = table[tokens[t], :] widened to float32.  A token outside [0, vocab) is an error
+// raised by the caller; the kernel clamps nothing.
+int axk_embed(const int32_t* tokens, const void* table, float* x, int n_tokens, int dim, int vocab,
+              void* stream);
+
+// out[r, :] = (x[row(r), :] * inv_rms) * gain, row(r) = rows ? rows[r] : r.
+// The sum of squares runs in 32-bit in an order that depends on `dim` alone.
+int axk_rmsnorm(const float* x, const int32_t* rows, const void* gain, int gain_is_f32, void* out,
+                int n_rows, int dim, float eps, void* stream);
+
+// table[t, i] = (sin, cos)(positions[t] * freqs[i]) computed in float64, stored float32.
+int axk_rope_table(const int32_t* positions, const double* freqs, float* table, int n_tokens,
+                   int n_pairs, void* stream);
+
+// Rotate-half on the first `rotary_dim` dims of each q and k head of qkv [T, (nh + 2 nkv) hd]
+// (q in place), and store k and v rows into the paged cache at each token's position.
+// write_kv = 0 rotates q only.  Cache layout per array: [page][kv head][slot in page][hd].
+int axk_rope_kv_write(void* qkv, const float* table, const int32_t* positions, const int32_t* seq_rows,
+                      const int32_t* block_table, int table_stride, void* k_cache, void* v_cache,
+                      int n_tokens, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
+                      int page_size, int write_kv, void* stream);
+
+// Causal attention of every token of the step over its request's cached positions
+// lo..=pos, lo = window > 0 ? max(0, pos + 1 - window) : 0.  q rows are `q_stride` elements
+// apart; out is [T, nh * hd].  Positions are folded in blocks of 64 in ascending order.
+int axk_attention(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                  const int32_t* block_table, int table_stride, const int32_t* positions,
+                  const int32_t* seq_rows, void* out, int n_tokens, int n_heads, int n_kv_heads,
+                  int head_dim, int page_size, int window, float scale, void* stream);
+
+// out = epilogue(X [M, K] . W [N, K]^T + bias).  mode 0: store elem [M, N]; 1: add into
+// float32 [M, N] (the residual stream); 2: store float32 [M, N] (logits).
+// x_stride / out_stride: elements between rows.
+int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
+             int out_stride, int m, int n, int k, int mode, void* stream);
+
+// out[t, f] = silu(gu[t, f]) * gu[t, F + f]: gate in the first F columns, up in the last.
+int axk_swiglu(const void* gate_up, void* out, int n_tokens, int n_ffn, void* stream);
+
+// picks[r] = index of the largest logit of row r; of equal maxima the last; NaN never
+// (all NaN: n - 1).
+int axk_argmax(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n, void* stream);
+
+// Repeat penalty on `recent` ids, then the k best as 64-bit keys (order key of the logit <<
+// 32 | id), unsorted, into cands[r, 0..k); the penalty is applied to `logits` in place.  recent is [n_rows, recent_stride] with
+// n_recent[r] valid ids each; penalty 1 or n_recent 0: off.  k <= 1024.
+int axk_topk(float* logits, int logits_stride, const int32_t* recent, int recent_stride,
+             const int32_t* n_recent, const float* penalty, const int32_t* k_of_row, uint64_t* cands,
+             int cands_stride, int n_rows, int n, void* stream);
+
+// dst[i] = value for i < n (a fill that may be captured into a graph).
+int axk_fill_i32(int32_t* dst, int32_t value, int n, void* stream);
+int axk_fill_f32(float* dst, float value, int n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

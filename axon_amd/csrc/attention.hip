@@ -1,0 +1,119 @@
+// Paged causal attention over the cache.
+//
+// The order every variant keeps (the reference's rule for its attention kernels,
+// src/cuda/decode.cu:1371-1400, 1650-1670): a token's positions are taken in blocks of 64
+// aligned to absolute position (block b = positions 64b .. 64b+63), each block gives
+// (m_b, l_b, o_b) = (max score, sum of exp(s - m_b), sum of exp(s - m_b) v), and blocks are
+// folded in ascending order into running (M, L, O):
+//     mn = max(M, m_b); alpha = exp(M - mn); w = exp(m_b - mn);
+//     L = l_b w + L alpha;  O = o_b w + O alpha;  out = O / L.
+// The block size does not depend on the page size, the batch or the context length, so a
+// token's result is the same however the step was cut.
+//
+// attention_rows: one wave per (token, query head), any head_dim that is a multiple of 16 up
+// to 256, any page size, any window.  Prefill portions and decode tokens alike.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+#define ATT_BLOCK 64
+#define ATT_MAX_HD 256
+
+__device__ inline const elem_t* cache_row(const elem_t* base, const int32_t* table_row, int pos, int page_size,
+                                          int n_kv_heads, int kvh, int head_dim) {
+  const int page = table_row[pos / page_size];
+  return base + (((size_t)page * n_kv_heads + kvh) * page_size + (pos % page_size)) * head_dim;
+}
+
+__global__ void __launch_bounds__(AXON_WAVE)
+attention_rows_kernel(const elem_t* __restrict__ q, int q_stride, const elem_t* __restrict__ k_cache,
+                      const elem_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
+                      const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
+                      elem_t* __restrict__ out, int n_heads, int n_kv_heads, int head_dim, int page_size, int window,
+                      float scale) {
+  __shared__ float qs[ATT_MAX_HD];
+  __shared__ float es[ATT_BLOCK];
+  __shared__ const elem_t* vrow[ATT_BLOCK];
+  const int t = blockIdx.x, qh = blockIdx.y, lane = threadIdx.x;
+  const int kvh = qh / (n_heads / n_kv_heads);
+  const int pos = positions[t];
+  const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int32_t* table_row = block_table + (size_t)seq_rows[t] * table_stride;
+
+  const elem_t* qrow = q + (size_t)t * q_stride + (size_t)qh * head_dim;
+  for (int d = lane; d < head_dim; d += AXON_WAVE) qs[d] = to_float(qrow[d]);
+  __syncthreads();
+
+  constexpr int DPL = ATT_MAX_HD / AXON_WAVE;  // output dims per lane at most
+  float M = -INFINITY, L = 0.0f, O[DPL];
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) O[i] = 0.0f;
+
+  for (int b0 = (lo / ATT_BLOCK) * ATT_BLOCK; b0 <= pos; b0 += ATT_BLOCK) {
+    const int p = b0 + lane;
+    const bool live = p >= lo && p <= pos;
+    float s = -INFINITY;
+    if (live) {
+      const elem_t* kr = cache_row(k_cache, table_row, p, page_size, n_kv_heads, kvh, head_dim);
+      float dot = 0.0f;
+      for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
+      s = dot * scale;
+      vrow[lane] = cache_row(v_cache, table_row, p, page_size, n_kv_heads, kvh, head_dim);
+    }
+    const float mb = wave_max(s);
+    const float e = live ? expf(s - mb) : 0.0f;
+    const float lb = wave_sum(e);
+    es[lane] = e;
+    __syncthreads();
+    float ob[DPL];
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) ob[i] = 0.0f;
+    const int first = max(lo - b0, 0), last = min(pos - b0, ATT_BLOCK - 1);
+    for (int j = first; j <= last; ++j) {
+      const float ej = es[j];
+      const elem_t* vr = vrow[j];
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const int d = lane + i * AXON_WAVE;
+        if (d < head_dim) ob[i] = fmaf(ej, to_float(vr[d]), ob[i]);
+      }
+    }
+    __syncthreads();
+    const float mn = fmaxf(M, mb);
+    const float alpha = expf(M - mn);
+    const float wgt = expf(mb - mn);
+    L = fmaf(lb, wgt, L * alpha);
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) O[i] = fmaf(ob[i], wgt, O[i] * alpha);
+    M = mn;
+  }
+
+  elem_t* orow = out + ((size_t)t * n_heads + qh) * head_dim;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) {
+    const int d = lane + i * AXON_WAVE;
+    if (d < head_dim) orow[d] = from_float(O[i] / L);
+  }
+}
+
+extern "C" int axk_attention(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                             const int32_t* block_table, int table_stride, const int32_t* positions,
+                             const int32_t* seq_rows, void* out, int n_tokens, int n_heads, int n_kv_heads,
+                             int head_dim, int page_size, int window, float scale, void* stream) {
+  AXK_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && page_size > 0,
+              "attention: bad sizes T=%d nh=%d nkv=%d page=%d", n_tokens, n_heads, n_kv_heads, page_size);
+  AXK_REQUIRE(n_heads % n_kv_heads == 0, "attention: %d query heads are not a multiple of %d kv heads", n_heads,
+              n_kv_heads);
+  AXK_REQUIRE(head_dim > 0 && head_dim % 16 == 0 && head_dim <= ATT_MAX_HD,
+              "attention: head_dim %d is not a multiple of 16 up to %d", head_dim, ATT_MAX_HD);
+  AXK_REQUIRE(n_heads <= 65535, "attention: %d heads (at most 65535)", n_heads);
+  AXK_REQUIRE(window >= 0, "attention: window %d is negative", window);
+  if (n_tokens == 0) return 0;
+  dim3 grid(n_tokens, n_heads);
+  attention_rows_kernel<<<grid, AXON_WAVE, 0, (hipStream_t)stream>>>(
+      (const elem_t*)q, q_stride, (const elem_t*)k_cache, (const elem_t*)v_cache, block_table, table_stride, positions,
+      seq_rows, (elem_t*)out, n_heads, n_kv_heads, head_dim, page_size, window, scale);
+  AXK_LAUNCH_CHECK("attention_rows");
+  return 0;
+}

@@ -1,0 +1,96 @@
+// Shared by every kernel file: the element type of this build, conversions, wave-level
+// reductions with a fixed order, and the error channel of the C interface.
+//
+// The library is compiled once per compute dtype: -DAXON_BF16=1 gives the bfloat16 build
+// (what serving uses: bf16 operands, every sum in 32-bit), -DAXON_BF16=0 the float32 build
+// (true 32-bit products and sums everywhere).  Both export the same C symbols.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#ifndef AXON_BF16
+#error "compile with -DAXON_BF16=0 or -DAXON_BF16=1"
+#endif
+
+#define AXON_WAVE 64
+
+// ---------------------------------------------------------------------------- bf16
+struct bf16_t {
+  uint16_t bits;
+};
+
+__host__ __device__ inline float bf16_to_float(bf16_t v) {
+  union { uint32_t u; float f; } c;
+  c.u = ((uint32_t)v.bits) << 16;
+  return c.f;
+}
+
+// Round to nearest, ties to even; NaN stays NaN (quiet).
+__host__ __device__ inline bf16_t float_to_bf16(float f) {
+  union { uint32_t u; float f; } c;
+  c.f = f;
+  bf16_t r;
+  if ((c.u & 0x7fffffffu) > 0x7f800000u) {
+    r.bits = (uint16_t)((c.u >> 16) | 0x0040u);
+    return r;
+  }
+  uint32_t lsb = (c.u >> 16) & 1u;
+  c.u += 0x7fffu + lsb;
+  r.bits = (uint16_t)(c.u >> 16);
+  return r;
+}
+
+#if AXON_BF16
+typedef bf16_t elem_t;
+__host__ __device__ inline float to_float(elem_t v) { return bf16_to_float(v); }
+__host__ __device__ inline elem_t from_float(float f) { return float_to_bf16(f); }
+#else
+typedef float elem_t;
+__host__ __device__ inline float to_float(elem_t v) { return v; }
+__host__ __device__ inline elem_t from_float(float f) { return f; }
+#endif
+
+// A vector (gain or bias) keeps the precision it was stored in: the caller says which.
+__device__ inline float load_vec(const void* p, int is_f32, int i) {
+  return is_f32 ? ((const float*)p)[i] : bf16_to_float(((const bf16_t*)p)[i]);
+}
+
+// ---------------------------------------------------------------------------- reductions
+// Butterfly over the 64 lanes of a wave: every lane ends with the same value, and the order
+// of the additions is fixed by the lane numbers alone.
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, AXON_WAVE);
+  return v;
+}
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, AXON_WAVE));
+  return v;
+}
+
+// ---------------------------------------------------------------------------- errors
+// Every entry point returns 0, or a negative code after recording a message that
+// axk_last_error() returns.  Shapes are checked on the host before anything is launched.
+void axk_set_error(const char* fmt, ...);
+
+#define AXK_REQUIRE(cond, ...)        \
+  do {                                \
+    if (!(cond)) {                    \
+      axk_set_error(__VA_ARGS__);     \
+      return -1;                      \
+    }                                 \
+  } while (0)
+
+#define AXK_LAUNCH_CHECK(name)                                              \
+  do {                                                                      \
+    hipError_t e_ = hipGetLastError();                                      \
+    if (e_ != hipSuccess) {                                                 \
+      axk_set_error("%s: launch failed: %s", name, hipGetErrorString(e_));  \
+      return -2;                                                            \
+    }                                                                       \
+  } while (0)
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

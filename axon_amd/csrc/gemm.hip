@@ -1,0 +1,150 @@
+// Matrix products out = X [M, K] . W [N, K]^T with a bias / residual epilogue.
+//
+// The rule every variant keeps: the K-reduction of one output element is one chain in
+// ascending k that does not depend on M, on the tile shape or on what else is in the batch
+// (the reference states the rule for its own kernels: src/cuda/decode.cu:352-369,
+// src/cuda/prefill.cu:6-16).  Rows only ride along.
+//
+// gemm_fma: any M, N, K and strides, 32-bit FMA, one chain per output: the float32 build's
+// product (true 32-bit), and the bfloat16 build's fallback for shapes the MFMA kernels refuse.
+#include "api.h"
+#include "common.h"
+
+enum { MODE_STORE = 0, MODE_ADD_F32 = 1, MODE_STORE_F32 = 2 };
+
+#define FMA_BN 64
+#define FMA_BK 16
+#define FMA_THREADS 256
+
+__device__ inline void load4_guarded(const elem_t* __restrict__ p, int valid, bool vec, float out[4]) {
+  if (vec && valid >= 4) {
+#if AXON_BF16
+    const uint2 raw = *reinterpret_cast<const uint2*>(p);
+    union { uint32_t u; float f; } c;
+    c.u = raw.x << 16; out[0] = c.f;
+    c.u = raw.x & 0xffff0000u; out[1] = c.f;
+    c.u = raw.y << 16; out[2] = c.f;
+    c.u = raw.y & 0xffff0000u; out[3] = c.f;
+#else
+    const float4 raw = *reinterpret_cast<const float4*>(p);
+    out[0] = raw.x; out[1] = raw.y; out[2] = raw.z; out[3] = raw.w;
+#endif
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = i < valid ? to_float(p[i]) : 0.0f;
+  }
+}
+
+// BM rows x 64 columns per block of 256 threads; thread (ty, tx) owns RM = BM / 16 rows and
+// 4 columns.  K is walked in steps of 16 through LDS; inside a step k ascends.
+template <int BM>
+__global__ void __launch_bounds__(FMA_THREADS)
+gemm_fma_kernel(const elem_t* __restrict__ x, int x_stride, const elem_t* __restrict__ w, const void* __restrict__ bias,
+                int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode, bool vec_x,
+                bool vec_w) {
+  constexpr int RM = BM / 16;
+  __shared__ float xs[FMA_BK][BM + 4];
+  __shared__ float ws[FMA_BK][FMA_BN + 4];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * FMA_BN;
+
+  float acc[RM][4];
+#pragma unroll
+  for (int i = 0; i < RM; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+
+  // loader: each thread brings 4 consecutive k of one row
+  const int lrow = tid >> 2, lk = (tid & 3) * 4;
+  for (int k0 = 0; k0 < K; k0 += FMA_BK) {
+    {
+      float v[4];
+      const int n = n0 + lrow;
+      const int valid = n < N ? min(4, K - (k0 + lk)) : 0;
+      load4_guarded(w + (size_t)n * K + k0 + lk, valid > 0 ? valid : 0, vec_w, v);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ws[lk + i][lrow] = v[i];
+    }
+    if (lrow < BM) {
+      float v[4];
+      const int m = m0 + lrow;
+      const int valid = m < M ? min(4, K - (k0 + lk)) : 0;
+      load4_guarded(x + (size_t)m * x_stride + k0 + lk, valid > 0 ? valid : 0, vec_x, v);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) xs[lk + i][lrow] = v[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < FMA_BK; ++kk) {
+      float a[RM], b[4];
+#pragma unroll
+      for (int i = 0; i < RM; ++i) a[i] = xs[kk][ty * RM + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < RM; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < RM; ++i) {
+    const int m = m0 + ty * RM + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= N) continue;
+      float v = acc[i][j];
+      if (bias) v += load_vec(bias, bias_is_f32, n);
+      const size_t at = (size_t)m * out_stride + n;
+      if (mode == MODE_STORE) ((elem_t*)out)[at] = from_float(v);
+      else if (mode == MODE_ADD_F32) ((float*)out)[at] += v;
+      else ((float*)out)[at] = v;
+    }
+  }
+}
+
+static int launch_fma(const elem_t* x, int x_stride, const elem_t* w, const void* bias, int bias_is_f32, void* out,
+                      int out_stride, int m, int n, int k, int mode, hipStream_t stream) {
+  const size_t vbytes = 4 * sizeof(elem_t);
+  const bool vec_w = (k % 4 == 0) && ((uintptr_t)w % vbytes == 0);
+  const bool vec_x = (k % 4 == 0) && (x_stride % 4 == 0) && ((uintptr_t)x % vbytes == 0);
+  if (m <= 16) {
+    dim3 grid(ceil_div(n, FMA_BN), ceil_div(m, 16));
+    gemm_fma_kernel<16><<<grid, FMA_THREADS, 0, stream>>>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n,
+                                                          k, mode, vec_x, vec_w);
+  } else {
+    dim3 grid(ceil_div(n, FMA_BN), ceil_div(m, 64));
+    gemm_fma_kernel<64><<<grid, FMA_THREADS, 0, stream>>>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n,
+                                                          k, mode, vec_x, vec_w);
+  }
+  AXK_LAUNCH_CHECK("gemm_fma");
+  return 0;
+}
+
+#if AXON_BF16
+int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, bool* handled);
+#endif
+
+extern "C" int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
+                        int out_stride, int m, int n, int k, int mode, void* stream) {
+  AXK_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
+  AXK_REQUIRE(x_stride >= k && out_stride >= n, "gemm: strides x=%d (K=%d) out=%d (N=%d) too small", x_stride, k,
+              out_stride, n);
+  AXK_REQUIRE(mode >= 0 && mode <= 2, "gemm: unknown mode %d", mode);
+  AXK_REQUIRE(ceil_div(m, 16) <= 65535, "gemm: M=%d is more rows than one launch takes", m);
+  if (m == 0) return 0;
+#if AXON_BF16
+  bool handled = false;
+  int rc = launch_gemm_mfma((const bf16_t*)x, x_stride, (const bf16_t*)w, bias, bias_is_f32, out, out_stride, m, n, k,
+                            mode, (hipStream_t)stream, &handled);
+  if (rc != 0 || handled) return rc;
+#endif
+  return launch_fma((const elem_t*)x, x_stride, (const elem_t*)w, bias, bias_is_f32, out, out_stride, m, n, k, mode,
+                    (hipStream_t)stream);
+}

@@ -1,0 +1,148 @@
+// Picking on the device: greedy argmax and the candidates of a sampled row.
+//
+// Both order logits by one 64-bit key, (order key of the logit) << 32 | id, as the
+// reference's sampler does (src/sample.rs:280-305; src/cuda/sample.cu:124-220): a larger
+// logit has a larger key, -0.0 ties +0.0, NaN is below everything, and of equal logits the
+// larger id wins.  The largest key is the greedy pick: of equal maxima the last index, NaN
+// never, all NaN gives n - 1 (src/generate.rs:222-264).  Keys are distinct, so selection is
+// exact and has no order-dependent step: integer histograms only.
+#include "api.h"
+#include "common.h"
+
+#define PICK_THREADS 1024
+
+__device__ inline uint32_t order_key(float v) {
+  if (v != v) return 0u;
+  uint32_t b = v == 0.0f ? 0u : __float_as_uint(v);
+  return (b >> 31) ? ~b : (b | 0x80000000u);
+}
+
+__device__ inline uint64_t key64(float v, int id) { return ((uint64_t)order_key(v) << 32) | (uint32_t)id; }
+
+__device__ inline uint64_t wave_max_u64(uint64_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint32_t lo = __shfl_xor((uint32_t)v, off, AXON_WAVE);
+    const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off, AXON_WAVE);
+    const uint64_t o = ((uint64_t)hi << 32) | lo;
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+__global__ void __launch_bounds__(PICK_THREADS)
+argmax_kernel(const float* __restrict__ logits, int stride, int32_t* __restrict__ picks, int n) {
+  __shared__ uint64_t partial[PICK_THREADS / AXON_WAVE];
+  const float* row = logits + (size_t)blockIdx.x * stride;
+  uint64_t best = 0;
+  for (int i = threadIdx.x; i < n; i += PICK_THREADS) {
+    const uint64_t k = key64(row[i], i);
+    best = k > best ? k : best;
+  }
+  best = wave_max_u64(best);
+  if ((threadIdx.x & (AXON_WAVE - 1)) == 0) partial[threadIdx.x / AXON_WAVE] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint64_t b = partial[0];
+    for (int w = 1; w < PICK_THREADS / AXON_WAVE; ++w) b = partial[w] > b ? partial[w] : b;
+    // every key of an all-NaN row is (0 << 32 | id): the largest id, n - 1, wins
+    picks[blockIdx.x] = (int32_t)(uint32_t)b;
+  }
+}
+
+extern "C" int axk_argmax(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n, void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && n > 0 && logits_stride >= n, "argmax: bad sizes rows=%d n=%d stride=%d", n_rows, n,
+              logits_stride);
+  if (n_rows == 0) return 0;
+  argmax_kernel<<<n_rows, PICK_THREADS, 0, (hipStream_t)stream>>>(logits, logits_stride, picks, n);
+  AXK_LAUNCH_CHECK("argmax");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------- candidates
+// One block per row.  (1) llama.cpp's repeat penalty on the distinct ids of the row's recent
+// window, in place: a positive logit is divided by p, any other multiplied
+// (src/sample.rs:307-326).  (2) An 8-pass radix select on the 64-bit keys finds the k-th
+// largest key exactly.  (3) Every key at or above it is appended to the row's candidates:
+// exactly k of them, in no particular order (the host sorts k pairs).
+__global__ void __launch_bounds__(PICK_THREADS)
+topk_kernel(float* __restrict__ logits, int stride, const int32_t* __restrict__ recent, int recent_stride,
+            const int32_t* __restrict__ n_recent, const float* __restrict__ penalty,
+            const int32_t* __restrict__ k_of_row, uint64_t* __restrict__ cands, int cands_stride, int n) {
+  __shared__ int hist[256];
+  __shared__ int s_digit, s_remaining, s_count;
+  const int r = blockIdx.x;
+  float* row = logits + (size_t)r * stride;
+  int k = k_of_row[r];
+  if (k <= 0) return;
+  if (k > n) k = n;
+
+  const float p = penalty[r];
+  const int nr = n_recent[r];
+  if (p != 1.0f && nr > 0) {
+    const int32_t* rec = recent + (size_t)r * recent_stride;
+    for (int j = threadIdx.x; j < nr; j += PICK_THREADS) {
+      const int id = rec[j];
+      bool first = id >= 0 && id < n;
+      for (int e = 0; e < j && first; ++e) first = rec[e] != id;
+      if (first) {
+        const float v = row[id];
+        row[id] = v > 0.0f ? v / p : v * p;
+      }
+    }
+    __syncthreads();
+  }
+
+  uint64_t prefix = 0, mask = 0;
+  if (threadIdx.x == 0) s_remaining = k;
+  for (int pass = 7; pass >= 0; --pass) {
+    const int shift = pass * 8;
+    if (threadIdx.x < 256) hist[threadIdx.x] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += PICK_THREADS) {
+      const uint64_t key = key64(row[i], i);
+      if ((key & mask) == prefix) atomicAdd(&hist[(int)((key >> shift) & 255u)], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int acc = 0, digit = 0;
+      const int remaining = s_remaining;
+      for (int b = 255; b >= 0; --b) {
+        if (acc + hist[b] >= remaining) {
+          digit = b;
+          break;
+        }
+        acc += hist[b];
+      }
+      s_digit = digit;
+      s_remaining = remaining - acc;
+    }
+    __syncthreads();
+    prefix |= (uint64_t)s_digit << shift;
+    mask |= (uint64_t)255u << shift;
+  }
+
+  if (threadIdx.x == 0) s_count = 0;
+  __syncthreads();
+  uint64_t* dst = cands + (size_t)r * cands_stride;
+  for (int i = threadIdx.x; i < n; i += PICK_THREADS) {
+    const uint64_t key = key64(row[i], i);
+    if (key >= prefix) {
+      const int at = atomicAdd(&s_count, 1);
+      if (at < k) dst[at] = key;
+    }
+  }
+}
+
+extern "C" int axk_topk(float* logits, int logits_stride, const int32_t* recent, int recent_stride,
+                        const int32_t* n_recent, const float* penalty, const int32_t* k_of_row, uint64_t* cands,
+                        int cands_stride, int n_rows, int n, void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && n > 0 && logits_stride >= n, "topk: bad sizes rows=%d n=%d stride=%d", n_rows, n,
+              logits_stride);
+  AXK_REQUIRE(cands_stride >= 1, "topk: candidate stride %d", cands_stride);
+  if (n_rows == 0) return 0;
+  topk_kernel<<<n_rows, PICK_THREADS, 0, (hipStream_t)stream>>>(logits, logits_stride, recent, recent_stride,
+                                                               n_recent, penalty, k_of_row, cands, cands_stride, n);
+  AXK_LAUNCH_CHECK("topk");
+  return 0;
+}

@@ -1,0 +1,186 @@
+"""The step function: one batch of (request, its next tokens) through the model, from the cache.
+
+`Engine.step(entries, end)` takes, for each request in the step, the tokens that follow what
+the cache already holds for it (a portion of a prompt, or one decoded token; cut anywhere)
+and the places among them whose logits are wanted.  All entries run as ONE batch: the tokens
+are laid side by side, every part sees them once, and attention reads each request's earlier
+positions from its pages.  It returns float32 logits [wanted, vocab] in the order of the
+entries and of their `want` lists.  Requests named in `end` give back what they hold after
+the step.
+
+Everything is validated before any work starts, and pages are reserved for all entries or
+for none (the reference refuses a bad step before it runs anything: src/cuda/qwen2/slots.rs:393-438).
+The reference runs prompt portions and decode rows as two passes of one scheduler step
+(src/serve/engine.rs:2413-2417); here they are one pass.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, Iterable, List, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheManager, OutOfPages
+from ..config.engine import EngineConfig
+from ..models.decoder import DecoderModel
+from .runtime import Runtime, Workspace
+
+
+class StepError(ValueError):
+    """A step that was refused before anything ran."""
+
+
+@dataclass
+class StepEntry:
+    id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class Span:
+    """One entry as the parts see it: its slot, where its tokens lie in the batch, and the
+    position of its first token."""
+    slot: int
+    q_start: int
+    q_len: int
+    start_pos: int
+
+
+@dataclass
+class LiveRequest:
+    slot: int
+    n_cached: int = 0
+
+
+class StepContext:
+    """What the parts are given for one step."""
+
+    def __init__(self, rt: Runtime, cache: CacheManager, ws: Workspace, meta: torch.Tensor, n_tokens: int,
+                 spans: List[Span]):
+        self.rt = rt
+        self.cache = cache
+        self.ws = ws
+        self.n_tokens = n_tokens
+        self.tokens = meta[0, :n_tokens]
+        self.positions = meta[1, :n_tokens]
+        self.seq_rows = meta[2, :n_tokens]
+        self.spans = spans
+        self.shared: Dict = {}       # per-step values shared by parts with equal parameters
+
+    def no_rotation(self) -> torch.Tensor:
+        return torch.empty((self.n_tokens, 0, 2), dtype=torch.float32, device=self.rt.device)
+
+
+class Engine:
+    def __init__(self, model: DecoderModel, rt: Runtime, cfg: EngineConfig):
+        self.model = model
+        self.rt = rt
+        self.cfg = cfg
+        self.max_seq_len = cfg.max_seq_len or model.max_positions
+        self.ws = Workspace(rt.device)
+        plans = model.group_plans(cfg.page_size, self._pool_size)
+        self.cache = CacheManager(plans, model.cache_plan.state_elems, cfg.max_seqs, self.max_seq_len, rt.device,
+                                  rt.dtype, cfg.shuffle_pages_seed)
+        self.live: Dict[Hashable, LiveRequest] = {}
+        self.has_window = any(p.spec.window > 0 for p in plans)
+        self.steps = 0
+
+    # ------------------------------------------------------------------ sizing
+    def _pool_size(self, spec, n_layers: int, page_size: int) -> int:
+        cfg = self.cfg
+        if cfg.num_pages > 0:
+            return cfg.num_pages
+        if cfg.max_cache_tokens > 0:
+            return max(1, -(-cfg.max_cache_tokens // page_size))
+        # from the memory that is free now: every group gets an equal share of the fraction
+        free, _ = torch.cuda.mem_get_info(self.rt.device)
+        n_groups = max(1, len(self.model.cache_plan.group_specs))
+        per_page = n_layers * spec.entries * spec.heads * page_size * spec.head_dim * self.rt.elem_size
+        pages = int(free * cfg.memory_fraction / n_groups) // max(per_page, 1)
+        cap = cfg.max_seqs * -(-self.max_seq_len // page_size)
+        return max(1, min(pages, cap))
+
+    # ------------------------------------------------------------------ requests
+    def n_cached(self, rid: Hashable) -> int:
+        return self.live[rid].n_cached if rid in self.live else 0
+
+    def release(self, rid: Hashable) -> None:
+        """Give back the pages, the slot and the state of a request."""
+        req = self.live.pop(rid, None)
+        if req is not None:
+            self.cache.close(req.slot)
+
+    def release_all(self) -> None:
+        for rid in list(self.live):
+            self.release(rid)
+
+    # ------------------------------------------------------------------ the step
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        seen = set()
+        vocab = self.model.vocab_size
+        for e in entries:
+            if e.id in seen:
+                raise StepError(f"request {e.id!r} appears twice in one step")
+            seen.add(e.id)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.id!r} brings no tokens")
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise StepError(f"request {e.id!r}: token {t} is outside the vocabulary of {vocab}")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"request {e.id!r}: wanted place {w} is outside its {n} tokens")
+            after = self.n_cached(e.id) + n
+            if after > self.max_seq_len:
+                raise StepError(f"request {e.id!r} would reach {after} positions, at most {self.max_seq_len}")
+        new = sum(1 for e in entries if e.id not in self.live)
+        if new > self.cache.free_slots():
+            raise StepError(f"{len(self.live) + new} live requests, at most {self.cfg.max_seqs}")
+
+    def step(self, entries: Sequence[StepEntry], end: Iterable[Hashable] = ()) -> Optional[torch.Tensor]:
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        self._validate(entries)
+        opened = []
+        try:
+            for e in entries:
+                if e.id not in self.live:
+                    self.live[e.id] = LiveRequest(self.cache.open())
+                    opened.append(e.id)
+                req = self.live[e.id]
+                self.cache.reserve(req.slot, req.n_cached + len(e.tokens))
+        except Exception:
+            for rid in opened:
+                self.release(rid)
+            raise
+
+        logits = None
+        if entries:
+            tokens, positions, rows, want_rows, spans = [], [], [], [], []
+            for e in entries:
+                req = self.live[e.id]
+                at = len(tokens)
+                n = len(e.tokens)
+                spans.append(Span(req.slot, at, n, req.n_cached))
+                tokens.extend(int(t) for t in e.tokens)
+                positions.extend(range(req.n_cached, req.n_cached + n))
+                rows.extend([req.slot] * n)
+                want_rows.extend(at + int(w) for w in e.want)
+            T = len(tokens)
+            meta = torch.tensor([tokens, positions, rows], dtype=torch.int32).to(self.rt.device)
+            self.cache.sync_tables()
+            ctx = StepContext(self.rt, self.cache, self.ws, meta, T, spans)
+            x = self.model.forward(ctx)
+            if want_rows:
+                sel = torch.tensor(want_rows, dtype=torch.int32).to(self.rt.device)
+                logits = self.model.logits(ctx, x, sel)
+            for e in entries:
+                req = self.live[e.id]
+                req.n_cached += len(e.tokens)
+                if self.has_window:
+                    self.cache.trim(req.slot, req.n_cached)
+            self.steps += 1
+        for rid in end:
+            self.release(rid)
+        return logits

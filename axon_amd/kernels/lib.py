@@ -1,0 +1,230 @@
+"""The kernel library as Python calls: tensors in, launches on the current HIP stream.
+
+`kernels(dtype)` loads (compiling at first use) the library of one compute dtype and wraps
+each C entry point.  Wrappers check what the C side cannot see (dtypes, devices, contiguity)
+and raise `KernelError` with the library's own message when a call is refused.  There is no
+other implementation behind these calls: without the library they fail.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_double, c_float, c_int, c_void_p
+from typing import Dict, Optional
+
+import torch
+
+from . import build
+
+MODE_STORE, MODE_ADD_F32, MODE_STORE_F32 = 0, 1, 2
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t: Optional[torch.Tensor]) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+_SIGNATURES = {
+    "axk_embed": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "axk_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p],
+    "axk_rope_table": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "axk_rope_kv_write": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
+                          c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "axk_attention": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                      c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "axk_gemm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "axk_swiglu": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "axk_argmax": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "axk_topk": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                 c_void_p],
+    "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
+    "axk_fill_f32": [c_void_p, c_float, c_int, c_void_p],
+}
+
+
+class Kernels:
+    """One loaded kernel library.  `dtype` is the torch dtype of `elem` tensors."""
+
+    def __init__(self, dtype_name: str):
+        self.dtype_name = dtype_name
+        self.dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype_name]
+        self.path = build.build_kernels(dtype_name)
+        self.lib = ctypes.CDLL(self.path, mode=ctypes.RTLD_LOCAL)
+        self.lib.axk_last_error.restype = c_char_p
+        for name, args in _SIGNATURES.items():
+            fn = getattr(self.lib, name)
+            fn.argtypes = args
+            fn.restype = c_int
+        if bool(self.lib.axk_is_bf16()) != (dtype_name == "bfloat16"):
+            raise KernelError(f"{self.path} was not built for {dtype_name}")
+
+    # ------------------------------------------------------------------ helpers
+    def _check(self, rc: int) -> None:
+        if rc != 0:
+            raise KernelError(self.lib.axk_last_error().decode())
+
+    def _elem(self, t: torch.Tensor, what: str) -> None:
+        if t.dtype != self.dtype or not t.is_cuda:
+            raise KernelError(f"{what}: expected a {self.dtype_name} device tensor, got {t.dtype} on {t.device}")
+
+    @staticmethod
+    def _f32(t: torch.Tensor, what: str) -> None:
+        if t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous():
+            raise KernelError(f"{what}: expected a contiguous float32 device tensor, got {t.dtype} on {t.device}")
+
+    @staticmethod
+    def _i32(t: torch.Tensor, what: str) -> None:
+        if t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous():
+            raise KernelError(f"{what}: expected a contiguous int32 device tensor, got {t.dtype} on {t.device}")
+
+    @staticmethod
+    def _vec_flag(v: Optional[torch.Tensor], what: str) -> int:
+        if v is None:
+            return 1
+        if v.dtype not in (torch.float32, torch.bfloat16) or not v.is_cuda or not v.is_contiguous():
+            raise KernelError(f"{what}: a vector must be float32 or bfloat16 on the device, got {v.dtype}")
+        return 1 if v.dtype == torch.float32 else 0
+
+    # ------------------------------------------------------------------ ops
+    def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        self._i32(tokens, "embed tokens"); self._elem(table, "embed table"); self._f32(out, "embed out")
+        vocab, dim = table.shape
+        if out.shape != (tokens.numel(), dim) or not table.is_contiguous():
+            raise KernelError(f"embed: out {tuple(out.shape)} does not fit {tokens.numel()} tokens of width {dim}")
+        self._check(self.lib.axk_embed(_ptr(tokens), _ptr(table), _ptr(out), tokens.numel(), dim, vocab, _stream()))
+        return out
+
+    def rmsnorm(self, x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        self._f32(x, "rmsnorm x"); self._elem(out, "rmsnorm out")
+        dim = x.shape[-1]
+        n = out.shape[0]
+        if rows is not None:
+            self._i32(rows, "rmsnorm rows")
+            if rows.numel() != n:
+                raise KernelError(f"rmsnorm: {rows.numel()} row indices for {n} output rows")
+        elif x.shape[0] != n:
+            raise KernelError(f"rmsnorm: {x.shape[0]} rows in, {n} rows out")
+        if gain.numel() != dim or out.shape[-1] != dim or not out.is_contiguous():
+            raise KernelError(f"rmsnorm: width {dim}, gain {gain.numel()}, out {tuple(out.shape)}")
+        self._check(self.lib.axk_rmsnorm(_ptr(x), _ptr(rows), _ptr(gain), self._vec_flag(gain, "rmsnorm gain"),
+                                         _ptr(out), n, dim, float(eps), _stream()))
+        return out
+
+    def rope_table(self, positions: torch.Tensor, freqs: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        self._i32(positions, "rope positions"); self._f32(out, "rope table")
+        if freqs.dtype != torch.float64 or not freqs.is_cuda:
+            raise KernelError("rope_table: frequencies must be float64 on the device")
+        if out.shape != (positions.numel(), freqs.numel(), 2):
+            raise KernelError(f"rope_table: table {tuple(out.shape)} for {positions.numel()} x {freqs.numel()} pairs")
+        self._check(self.lib.axk_rope_table(_ptr(positions), _ptr(freqs), _ptr(out), positions.numel(), freqs.numel(),
+                                            _stream()))
+        return out
+
+    def rope_kv_write(self, qkv, table, positions, seq_rows, block_table, k_cache, v_cache, n_heads, n_kv_heads,
+                      head_dim, rotary_dim, page_size, write_kv=True) -> None:
+        self._elem(qkv, "rope qkv"); self._f32(table, "rope table")
+        self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
+        T = positions.numel()
+        width = (n_heads + 2 * n_kv_heads) * head_dim
+        if qkv.shape != (T, width) or not qkv.is_contiguous():
+            raise KernelError(f"rope_kv_write: qkv {tuple(qkv.shape)} is not [{T}, {width}] contiguous")
+        if table.shape != (T, rotary_dim // 2, 2):
+            raise KernelError(f"rope_kv_write: table {tuple(table.shape)} for rotary_dim {rotary_dim}")
+        if write_kv:
+            self._elem(k_cache, "k cache"); self._elem(v_cache, "v cache")
+            for c in (k_cache, v_cache):
+                if c.dim() != 4 or tuple(c.shape[1:]) != (n_kv_heads, page_size, head_dim) or not c.is_contiguous():
+                    raise KernelError(f"rope_kv_write: cache {tuple(c.shape)} is not [pages, {n_kv_heads}, {page_size}, {head_dim}]")
+        self._check(self.lib.axk_rope_kv_write(
+            _ptr(qkv), _ptr(table), _ptr(positions), _ptr(seq_rows), _ptr(block_table), block_table.shape[-1],
+            _ptr(k_cache if write_kv else None), _ptr(v_cache if write_kv else None), T, n_heads, n_kv_heads, head_dim,
+            rotary_dim, page_size, 1 if write_kv else 0, _stream()))
+
+    def attention(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, n_heads, n_kv_heads,
+                  head_dim, page_size, window, scale) -> torch.Tensor:
+        self._elem(q, "attention q"); self._elem(k_cache, "k cache"); self._elem(v_cache, "v cache")
+        self._elem(out, "attention out")
+        self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
+        T = positions.numel()
+        if out.shape != (T, n_heads * head_dim) or not out.is_contiguous():
+            raise KernelError(f"attention: out {tuple(out.shape)} is not [{T}, {n_heads * head_dim}]")
+        for c in (k_cache, v_cache):
+            if c.dim() != 4 or tuple(c.shape[1:]) != (n_kv_heads, page_size, head_dim) or not c.is_contiguous():
+                raise KernelError(f"attention: cache {tuple(c.shape)} is not [pages, {n_kv_heads}, {page_size}, {head_dim}]")
+        self._check(self.lib.axk_attention(
+            _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[-1], _ptr(positions),
+            _ptr(seq_rows), _ptr(out), T, n_heads, n_kv_heads, head_dim, page_size, window, float(scale), _stream()))
+        return out
+
+    def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
+             mode: int = MODE_STORE) -> torch.Tensor:
+        """out = epilogue(x . w^T + bias); x [M, K] (rows may be strided), w [N, K] contiguous."""
+        self._elem(x, "gemm x"); self._elem(w, "gemm w")
+        M, K = x.shape
+        N = w.shape[0]
+        if w.shape[1] != K or not w.is_contiguous() or x.stride(1) != 1 or out.stride(1) != 1:
+            raise KernelError(f"gemm: x {tuple(x.shape)} w {tuple(w.shape)} do not multiply, or are not row-major")
+        if out.shape != (M, N) or not out.is_cuda:
+            raise KernelError(f"gemm: out {tuple(out.shape)} is not [{M}, {N}]")
+        want = self.dtype if mode == MODE_STORE else torch.float32
+        if out.dtype != want:
+            raise KernelError(f"gemm: mode {mode} writes {want}, out is {out.dtype}")
+        if bias is not None and bias.numel() != N:
+            raise KernelError(f"gemm: bias of {bias.numel()} for {N} columns")
+        self._check(self.lib.axk_gemm(_ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"),
+                                      _ptr(out), out.stride(0), M, N, K, mode, _stream()))
+        return out
+
+    def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        self._elem(gate_up, "swiglu in"); self._elem(out, "swiglu out")
+        T, F = out.shape
+        if gate_up.shape != (T, 2 * F) or not gate_up.is_contiguous() or not out.is_contiguous():
+            raise KernelError(f"swiglu: in {tuple(gate_up.shape)} out {tuple(out.shape)}")
+        self._check(self.lib.axk_swiglu(_ptr(gate_up), _ptr(out), T, F, _stream()))
+        return out
+
+    def argmax(self, logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        self._i32(out, "argmax out")
+        if logits.dtype != torch.float32 or not logits.is_cuda or logits.stride(1) != 1 or out.numel() != logits.shape[0]:
+            raise KernelError(f"argmax: logits {tuple(logits.shape)} {logits.dtype}, picks {out.numel()}")
+        self._check(self.lib.axk_argmax(_ptr(logits), logits.stride(0), _ptr(out), logits.shape[0], logits.shape[1],
+                                        _stream()))
+        return out
+
+    def topk(self, logits, recent, n_recent, penalty, k_of_row, cands) -> torch.Tensor:
+        self._i32(recent, "topk recent"); self._i32(n_recent, "topk n_recent"); self._i32(k_of_row, "topk k")
+        self._f32(penalty, "topk penalty")
+        rows, n = logits.shape
+        if (logits.dtype != torch.float32 or not logits.is_cuda or logits.stride(1) != 1 or cands.dtype != torch.int64
+                or cands.shape[0] != rows or not cands.is_contiguous() or recent.shape[0] != rows):
+            raise KernelError(f"topk: logits {tuple(logits.shape)} cands {tuple(cands.shape)} {cands.dtype}")
+        if int(k_of_row.max()) > cands.shape[1]:
+            raise KernelError(f"topk: k up to {int(k_of_row.max())} for {cands.shape[1]} candidate places")
+        self._check(self.lib.axk_topk(_ptr(logits), logits.stride(0), _ptr(recent), recent.shape[1], _ptr(n_recent),
+                                      _ptr(penalty), _ptr(k_of_row), _ptr(cands), cands.shape[1], rows, n, _stream()))
+        return cands
+
+    def fill_i32(self, dst: torch.Tensor, value: int) -> None:
+        self._i32(dst, "fill")
+        self._check(self.lib.axk_fill_i32(_ptr(dst), int(value), dst.numel(), _stream()))
+
+    def fill_f32(self, dst: torch.Tensor, value: float) -> None:
+        self._f32(dst, "fill")
+        self._check(self.lib.axk_fill_f32(_ptr(dst), float(value), dst.numel(), _stream()))
+
+
+_LOADED: Dict[str, Kernels] = {}
+
+
+def kernels(dtype_name: str) -> Kernels:
+    """The kernel library for "bfloat16" or "float32" (loaded once per process)."""
+    if dtype_name not in _LOADED:
+        _LOADED[dtype_name] = Kernels(dtype_name)
+    return _LOADED[dtype_name]

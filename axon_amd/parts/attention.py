@@ -1,0 +1,110 @@
+"""Grouped-query attention over the paged cache: the mixer of this architecture.
+
+q = Wq h + bq, k = Wk h + bk, v = Wv h + bv (bias after the product, before the rotation;
+used iff the tensor exists: src/model.rs:2982-2991), rotate-half on q and k, k and v stored in
+the request's pages, causal attention in which query head qh reads kv head qh // group with
+scale 1/sqrt(head_dim) (src/model.rs:3373-3463), then the output projection, whose result is
+added to the residual stream (src/model.rs:3031-3038).
+
+The three projections run as one product over a fused [q_dim + 2 kv_dim, hidden] matrix
+(fused when the weights are loaded; the reference fuses at launch: src/model.rs:2199-2238).
+
+Parameters: `hidden_size`, `num_heads`, `num_kv_heads`, `head_dim`, `qkv_bias` (True, False
+or "optional"), `out_bias`, `window` (0: all earlier positions), `position` (a PartSpec).
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional
+
+import torch
+
+from ..config.base import ConfigError
+from ..kernels import MODE_ADD_F32, MODE_STORE
+from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, build_part, register_mixer
+
+
+class GQAttention(Mixer):
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        p = params
+        self.hidden = int(p["hidden_size"])
+        self.nh = int(p["num_heads"])
+        self.nkv = int(p["num_kv_heads"])
+        self.hd = int(p["head_dim"])
+        self.window = int(p.get("window", 0))
+        self.qkv_bias = p.get("qkv_bias", False)
+        self.out_bias = bool(p.get("out_bias", False))
+        if self.nh % self.nkv:
+            raise ConfigError(f"{self.nh} query heads are not a multiple of {self.nkv} kv heads")
+        if self.hd % 16 or not 16 <= self.hd <= 256:
+            raise ConfigError(f"head_dim {self.hd} is not a multiple of 16 between 16 and 256: no kernel takes it")
+        self.q_dim, self.kv_dim = self.nh * self.hd, self.nkv * self.hd
+        self.scale = 1.0 / math.sqrt(self.hd)
+        self.position = build_part("position", p["position"]) if p.get("position") is not None else None
+        names = p.get("names", {})
+        base = prefix + names.get("scope", "self_attn.")
+        self.n = {k: base + names.get(k, k + "_proj") for k in ("q", "k", "v", "o")}
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+
+    # ------------------------------------------------------------------ declarations
+    def tensors(self) -> List[TensorDecl]:
+        t = [TensorDecl(self.n["q"] + ".weight", (self.q_dim, self.hidden)),
+             TensorDecl(self.n["k"] + ".weight", (self.kv_dim, self.hidden)),
+             TensorDecl(self.n["v"] + ".weight", (self.kv_dim, self.hidden)),
+             TensorDecl(self.n["o"] + ".weight", (self.hidden, self.q_dim))]
+        if self.qkv_bias:
+            opt = self.qkv_bias == "optional"
+            t += [TensorDecl(self.n["q"] + ".bias", (self.q_dim,), "bias", opt),
+                  TensorDecl(self.n["k"] + ".bias", (self.kv_dim,), "bias", opt),
+                  TensorDecl(self.n["v"] + ".bias", (self.kv_dim,), "bias", opt)]
+        if self.out_bias:
+            t.append(TensorDecl(self.n["o"] + ".bias", (self.hidden,), "bias"))
+        return t
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return CacheSpec(entries=2, heads=self.nkv, head_dim=self.hd, window=self.window)
+
+    def load(self, store, rt) -> None:
+        self.w_qkv = store.fused_matrix([self.n[k] + ".weight" for k in ("q", "k", "v")])
+        biases = [store.vector(self.n[k] + ".bias", optional=True) for k in ("q", "k", "v")] if self.qkv_bias else []
+        present = [b is not None for b in biases]
+        if any(present):
+            if not all(present):
+                raise ConfigError(f"{self.prefix}: q, k and v biases must all be present or all absent")
+            dt = torch.float32 if any(b.dtype == torch.float32 for b in biases) else biases[0].dtype
+            self.b_qkv = torch.cat([b.to(dt) for b in biases]).contiguous()
+        self.w_o = store.matrix(self.n["o"] + ".weight")
+        self.b_o = store.vector(self.n["o"] + ".bias") if self.out_bias else None
+        if self.position is not None:
+            self.position.load(store, rt)
+
+    # ------------------------------------------------------------------ the step
+    def forward(self, ctx, binding: CacheBinding, h, residual) -> None:
+        k = ctx.rt.k
+        T = h.shape[0]
+        group = ctx.cache.group(binding.group)
+        k_cache, v_cache = group.layer(binding.index)
+        mark = ctx.ws.mark()
+        if binding.writes:
+            qkv = ctx.ws.take((T, self.q_dim + 2 * self.kv_dim), ctx.rt.dtype)
+            k.gemm(h, self.w_qkv, qkv, self.b_qkv, MODE_STORE)
+        else:
+            # reading another run's cache: only the queries are needed
+            qkv = ctx.ws.take((T, self.q_dim + 2 * self.kv_dim), ctx.rt.dtype)
+            bias = None if self.b_qkv is None else self.b_qkv[:self.q_dim]
+            k.gemm(h, self.w_qkv[:self.q_dim], qkv[:, :self.q_dim], bias, MODE_STORE)
+        if self.position is not None:
+            table, rotary = self.position.tables(ctx), self.position.rotary_dim
+        else:
+            table, rotary = ctx.no_rotation(), 0
+        k.rope_kv_write(qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache, self.nh, self.nkv,
+                        self.hd, rotary, group.page_size, binding.writes)
+        att = ctx.ws.take((T, self.q_dim), ctx.rt.dtype)
+        k.attention(qkv, qkv.stride(0), k_cache, v_cache, group.block_table, ctx.positions, ctx.seq_rows, att, self.nh,
+                    self.nkv, self.hd, group.page_size, self.window, self.scale)
+        k.gemm(att, self.w_o, residual, self.b_o, MODE_ADD_F32)
+        ctx.ws.release(mark)
+
+
+register_mixer("gqa_attention", GQAttention)

@@ -1,0 +1,157 @@
+"""The interfaces of a layer's parts, and the registries they are found in.
+
+A model is put together from parts that know nothing of the model they are in: each takes its
+sizes and constants as parameters (a `PartSpec`'s `params`), declares the checkpoint tensors
+it needs, says what cache or per-request state it wants, and runs on the tokens of a step.
+
+* `Norm.forward(ctx, x, out)`: normalise rows of the 32-bit residual stream into the compute
+  dtype.
+* `PositionEncoding.tables(ctx)`: whatever the mixer's kernels need for the positions of
+  this step, computed once per step and shared by all layers with equal parameters.
+* `Mixer.forward(ctx, binding, h, residual)`: mix the tokens of each request (attention here),
+  reading and writing the cache `binding` names, and ADD the result to `residual` (32-bit).
+* `FeedForward.forward(ctx, h, residual)`: the same shape of call, without a cache.
+* `Block.forward(ctx, binding, x)`: the arrangement of norm, mixer and feed-forward around
+  the residual stream `x`.
+
+Another part is a subclass registered under a new name (`register_mixer`, ...); a
+configuration then names it in a `PartSpec`.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+from ..config.base import ConfigError, PartSpec
+
+
+@dataclass(frozen=True)
+class TensorDecl:
+    """A checkpoint tensor a part needs.  `role` decides storage and random initialisation:
+    "matrix" (compute dtype; normal), "bias" (vector; normal), "gain" (vector; 1 + normal),
+    "table" (integers, kept as int32).  An `optional` tensor may be absent."""
+    name: str
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+    optional: bool = False
+
+
+@dataclass(frozen=True)
+class CacheSpec:
+    """Paged per-token storage a mixer wants for one run: `entries` arrays (keys and values:
+    2) of `heads` x `head_dim` elements per position.  `window` > 0: only the last `window`
+    positions are ever read, so earlier pages can be given back."""
+    entries: int
+    heads: int
+    head_dim: int
+    window: int = 0
+
+    def group_key(self):
+        return (self.entries, self.heads, self.head_dim, self.window)
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size per-request state a mixer wants for one run: `elems` 32-bit floats, zeroed
+    when a request starts."""
+    elems: int
+
+
+@dataclass
+class CacheBinding:
+    """What a run of a layer is given by the cache manager: its cache group and its index in
+    that group's storage, whether it stores what it computes, and its state arena."""
+    group: int = -1
+    index: int = -1
+    writes: bool = True
+    state_index: int = -1
+
+
+class Part:
+    """Common to all parts: tensors in, then bound to device memory."""
+
+    def __init__(self, params: Dict[str, Any], prefix: str = ""):
+        self.params = dict(params)
+        self.prefix = prefix
+
+    def tensors(self) -> List[TensorDecl]:
+        return []
+
+    def load(self, store, rt) -> None:
+        """Take the declared tensors from `store` (a `WeightStore`); `rt` is the runtime
+        (device, dtype, kernels)."""
+
+
+class Norm(Part):
+    def forward(self, ctx, x, out=None):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def tables(self, ctx):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, ctx, binding: CacheBinding, h, residual) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx, h, residual) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement: built from the layer's parts, not from a spec of its own."""
+
+    def __init__(self, norm_factory: Callable[[str], Norm], mixer: Mixer, feed_forward: FeedForward, prefix: str):
+        super().__init__({}, prefix)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+
+    def forward(self, ctx, binding: CacheBinding, x) -> None:
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------- registries
+
+_REGISTRIES: Dict[str, Dict[str, Any]] = {k: {} for k in
+                                          ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")}
+
+
+def _register(kind: str, name: str, cls) -> None:
+    _REGISTRIES[kind][name] = cls
+
+
+def _lookup(kind: str, name: str):
+    try:
+        return _REGISTRIES[kind][name]
+    except KeyError:
+        known = ", ".join(sorted(_REGISTRIES[kind])) or "none"
+        raise ConfigError(f"no {kind.replace('_', '-')} part is registered as '{name}' (known: {known})") from None
+
+
+def register_norm(name, cls): _register("norm", name, cls)
+def register_position(name, cls): _register("position", name, cls)
+def register_mixer(name, cls): _register("mixer", name, cls)
+def register_feed_forward(name, cls): _register("feed_forward", name, cls)
+def register_block(name, cls): _register("block", name, cls)
+def register_embedding(name, cls): _register("embedding", name, cls)
+def register_head(name, cls): _register("head", name, cls)
+
+
+def build_part(kind: str, spec: PartSpec, prefix: str = "") -> Part:
+    return _lookup(kind, spec.kind)(spec.params, prefix)
+
+
+def build_block(name: str, norm_spec: PartSpec, mixer: Mixer, feed_forward: FeedForward, prefix: str) -> Block:
+    def norm_factory(tensor_name: str) -> Norm:
+        return build_part("norm", PartSpec(norm_spec.kind, {**norm_spec.params, "tensor": tensor_name}), prefix)
+    return _lookup("block", name)(norm_factory, mixer, feed_forward, prefix)

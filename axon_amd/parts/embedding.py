@@ -1,0 +1,65 @@
+"""Token embedding and the language-model head.
+
+The embedding row is the token's starting vector as it is (src/model.rs:2657-2675).  The head
+is `lm_head.weight` if the tensor exists, else the embedding matrix; a model that is not tied
+must have it (src/model.rs:1800-1803, src/safetensors.rs:1608-1614).  Logits are float32 and
+are computed only at the rows asked for (src/model.rs:2647-2654).
+"""
+from __future__ import annotations
+
+from typing import List
+
+import torch
+
+from ..kernels import MODE_STORE_F32
+from .base import Part, TensorDecl, register_embedding, register_head
+
+
+class TokenEmbedding(Part):
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        self.vocab = int(params["vocab_size"])
+        self.hidden = int(params["hidden_size"])
+        self.name = prefix + params["tensor"]
+        self.table = None
+
+    def tensors(self) -> List[TensorDecl]:
+        return [TensorDecl(self.name, (self.vocab, self.hidden), "matrix")]
+
+    def load(self, store, rt) -> None:
+        self.table = store.matrix(self.name)
+
+    def forward(self, ctx, out=None):
+        if out is None:
+            out = ctx.ws.take_persistent((ctx.n_tokens, self.hidden), torch.float32)
+        return ctx.rt.k.embed(ctx.tokens, self.table, out)
+
+
+class LMHead(Part):
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        self.vocab = int(params["vocab_size"])
+        self.hidden = int(params["hidden_size"])
+        self.name = prefix + params["tensor"]
+        self.tied_to = params.get("tied_to")
+        self.tied = bool(params.get("tied", False))
+        self.weight = None
+
+    def tensors(self) -> List[TensorDecl]:
+        # tied: the head's own tensor is used if the checkpoint has one
+        return [TensorDecl(self.name, (self.vocab, self.hidden), "matrix", optional=self.tied)]
+
+    def load(self, store, rt) -> None:
+        self.weight = store.matrix(self.name, optional=self.tied)
+        if self.weight is None:
+            self.weight = store.matrix(self.tied_to)
+
+    def forward(self, ctx, h, out=None):
+        """h: [rows, hidden] in the compute dtype -> float32 logits [rows, vocab]."""
+        if out is None:
+            out = torch.empty((h.shape[0], self.vocab), dtype=torch.float32, device=h.device)
+        return ctx.rt.k.gemm(h, self.weight, out, None, MODE_STORE_F32)
+
+
+register_embedding("token_embedding", TokenEmbedding)
+register_head("lm_head", LMHead)

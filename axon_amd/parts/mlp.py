@@ -1,0 +1,45 @@
+"""The dense SwiGLU feed-forward: down(silu(gate h) * up h), added to the residual stream.
+
+act = (g / (1 + exp(-g))) * u (src/vmath.rs:128-132), no biases (src/model.rs:3043-3055).
+gate and up run as one product over a fused [2 ffn, hidden] matrix.  Parameters:
+`hidden_size`, `intermediate_size`.
+"""
+from __future__ import annotations
+
+from typing import List
+
+from ..kernels import MODE_ADD_F32, MODE_STORE
+from .base import FeedForward, TensorDecl, register_feed_forward
+
+
+class SwiGLUMLP(FeedForward):
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        self.hidden = int(params["hidden_size"])
+        self.ffn = int(params["intermediate_size"])
+        names = params.get("names", {})
+        base = prefix + names.get("scope", "mlp.")
+        self.n = {k: base + names.get(k, k + "_proj") + ".weight" for k in ("gate", "up", "down")}
+        self.w_gate_up = self.w_down = None
+
+    def tensors(self) -> List[TensorDecl]:
+        return [TensorDecl(self.n["gate"], (self.ffn, self.hidden)), TensorDecl(self.n["up"], (self.ffn, self.hidden)),
+                TensorDecl(self.n["down"], (self.hidden, self.ffn))]
+
+    def load(self, store, rt) -> None:
+        self.w_gate_up = store.fused_matrix([self.n["gate"], self.n["up"]])
+        self.w_down = store.matrix(self.n["down"])
+
+    def forward(self, ctx, h, residual) -> None:
+        k = ctx.rt.k
+        T = h.shape[0]
+        mark = ctx.ws.mark()
+        gate_up = ctx.ws.take((T, 2 * self.ffn), ctx.rt.dtype)
+        k.gemm(h, self.w_gate_up, gate_up, None, MODE_STORE)
+        act = ctx.ws.take((T, self.ffn), ctx.rt.dtype)
+        k.swiglu(gate_up, act)
+        k.gemm(act, self.w_down, residual, None, MODE_ADD_F32)
+        ctx.ws.release(mark)
+
+
+register_feed_forward("swiglu_mlp", SwiGLUMLP)
