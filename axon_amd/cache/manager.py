@@ -71,6 +71,14 @@ def host_lib():
             "axh_sched_remove": (c_int, [c_void_p, ctypes.c_int64]),
             "axh_sched_counts": (None, [c_void_p, LP, LP, LP]),
             "axh_sched_progress": (c_int, [c_void_p, ctypes.c_int64, LP, LP, IP]),
+            "axh_rng_seed": (None, [ctypes.c_uint64, c_void_p]),
+            "axh_rng_next_u64": (ctypes.c_uint64, [c_void_p]),
+            "axh_rng_next_f64": (ctypes.c_double, [c_void_p]),
+            "axh_sample_pick_keys": (c_int, [c_void_p, c_int, ctypes.c_float, ctypes.c_float, ctypes.c_float,
+                                             ctypes.c_double]),
+            "axh_sample_pick_row": (c_int, [c_void_p, c_int, c_void_p, c_int, ctypes.c_float, c_int, ctypes.c_float,
+                                            ctypes.c_float, ctypes.c_float, ctypes.c_double]),
+            "axh_argmax_row": (c_int, [c_void_p, c_int]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(lib, name)

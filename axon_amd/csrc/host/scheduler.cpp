@@ -55,12 +55,6 @@ Request* find(Scheduler& s, int64_t id) {
   return nullptr;
 }
 
-bool fits(const Scheduler& s, const std::vector<long>& free, long from, long to) {
-  for (size_t g = 0; g < s.groups.size(); ++g)
-    if (pages_to_grow(s.groups[g], from, to) > free[g]) return false;
-  return true;
-}
-
 void take(const Scheduler& s, std::vector<long>& free, long from, long to) {
   for (size_t g = 0; g < s.groups.size(); ++g) free[g] -= pages_to_grow(s.groups[g], from, to);
 }

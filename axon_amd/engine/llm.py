@@ -1,0 +1,170 @@
+"""The Python entry point: `axon_amd.load(model).generate(token_ids, ...)`.
+
+In the manner of the reference's library root (src/lib.rs:19-35, 112-127: `load`, then a
+backend, then `generate` with greedy or sampled options, src/generate.rs:29-114), with token
+ids in and token ids out: there is no tokenizer here.  Any number of prompts may be given;
+they are batched continuously by the scheduler.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Union
+
+import torch
+
+from ..config import EngineConfig, ModelConfig, config_from_dict
+from ..sampling import Sampler, SamplingParams, pick_rows
+from .loading import load_model, random_model
+from .runtime import Runtime
+from .scheduler import Scheduler
+from .step import Engine, StepEntry
+
+
+@dataclass
+class GenStats:
+    """What a `generate` call did (the reference's GenStats, src/generate.rs:29-45, reduced to
+    what this engine has): steps run, tokens fed as prompt, tokens decided, time."""
+    steps: int = 0
+    prompt_tokens: int = 0
+    decided: int = 0
+    preemptions: int = 0
+    seconds: float = 0.0
+
+
+@dataclass
+class _Request:
+    tokens: List[int]
+    prompt_len: int
+    max_new: int
+    sampler: Optional[Sampler]
+    out: List[int] = field(default_factory=list)
+    done: bool = False
+
+
+class LLM:
+    def __init__(self, model, rt: Runtime, cfg: EngineConfig):
+        self.model = model
+        self.rt = rt
+        self.cfg = cfg
+        self.engine = Engine(model, rt, cfg)
+        self.last_stats = GenStats()
+        self._next_id = 0
+
+    @property
+    def config(self) -> ModelConfig:
+        return self.model.config
+
+    # ------------------------------------------------------------------ generation
+    def generate(self, prompts: Union[Sequence[int], Sequence[Sequence[int]]], max_new_tokens: int = 32,
+                 temperature: float = 0.0, top_k: int = 40, top_p: float = 0.9, min_p: float = 0.0,
+                 repeat_penalty: float = 1.1, repeat_last_n: int = 64, seed: Optional[int] = None,
+                 stop: Sequence[int] = (), sampling: Optional[SamplingParams] = None) -> List[List[int]]:
+        """New tokens for every prompt (lists of token ids).  `temperature` 0 is greedy: the
+        highest logit, and no other sampling setting applies.  With a temperature, request i
+        draws from the stream seeded `seed + i`.  A token in `stop` ends its request and is not
+        returned (src/generate.rs:169-171)."""
+        single = len(prompts) > 0 and isinstance(prompts[0], int)
+        batch = [list(prompts)] if single else [list(p) for p in prompts]
+        params = sampling or SamplingParams(temperature, top_k, top_p, min_p, repeat_penalty, repeat_last_n, seed)
+        sched = Scheduler.for_cache(self.engine.cache, self.cfg.max_batch_tokens)
+        reqs: Dict[int, _Request] = {}
+        order = []
+        for i, p in enumerate(batch):
+            if not p:
+                raise ValueError("a prompt needs at least one token")
+            rid = self._next_id
+            self._next_id += 1
+            sampler = None
+            if not params.greedy:
+                base = params.seed if params.seed is not None else None
+                sampler = Sampler(SamplingParams(params.temperature, params.top_k, params.top_p, params.min_p,
+                                                 params.repeat_penalty, params.repeat_last_n,
+                                                 None if base is None else base + i))
+            reqs[rid] = _Request(p, len(p), max_new_tokens, sampler)
+            order.append(rid)
+            if max_new_tokens <= 0:
+                reqs[rid].done = True
+            else:
+                sched.add(rid, len(p), max_new_tokens)
+        stats = GenStats()
+        t0 = time.time()
+        stop = set(int(s) for s in stop)
+        cache = self.engine.cache
+        n_groups = len(cache.groups)
+        try:
+            while any(not r.done for r in reqs.values()):
+                plan, preempted = sched.plan([cache.free_pages(g) for g in range(n_groups)])
+                for rid in preempted:
+                    self.engine.release(rid)
+                    stats.preemptions += 1
+                if not plan:
+                    raise RuntimeError("the scheduler has requests but planned nothing: the cache pool is too small")
+                entries = [StepEntry(p.id, reqs[p.id].tokens[p.start:p.start + p.count],
+                                     [p.count - 1] if p.wants_logits else []) for p in plan]
+                logits = self.engine.step(entries)
+                stats.steps += 1
+                wanted = [p for p in plan if p.wants_logits]
+                picks = []
+                if wanted:
+                    picks = pick_rows(self.rt, logits, [reqs[p.id].sampler for p in wanted],
+                                      [reqs[p.id].tokens for p in wanted])
+                at = 0
+                for p in plan:
+                    r = reqs[p.id]
+                    appended = finished = False
+                    if p.wants_logits:
+                        tok = int(picks[at])
+                        at += 1
+                        stats.decided += 1
+                        if tok in stop:
+                            finished = True
+                        else:
+                            r.tokens.append(tok)
+                            r.out.append(tok)
+                            appended = True
+                            finished = len(r.out) >= r.max_new
+                    else:
+                        stats.prompt_tokens += p.count
+                    sched.commit(p.id, p.count, appended, finished)
+                    if finished:
+                        r.done = True
+                        self.engine.release(p.id)
+        finally:
+            for rid in order:
+                self.engine.release(rid)
+        stats.seconds = time.time() - t0
+        self.last_stats = stats
+        outs = [reqs[rid].out for rid in order]
+        return outs
+
+    # ------------------------------------------------------------------ logits
+    def logits(self, token_ids: Sequence[int], all_positions: bool = False) -> torch.Tensor:
+        """float32 logits after `token_ids`: at the last position [vocab], or at every position
+        [len, vocab].  The cache is left as it was."""
+        ids = list(token_ids)
+        rid = ("logits", self._next_id)
+        self._next_id += 1
+        want = list(range(len(ids))) if all_positions else [len(ids) - 1]
+        out = self.engine.step([StepEntry(rid, ids, want)], end=[rid])
+        return out if all_positions else out[0]
+
+
+def load(model: Union[str, dict, ModelConfig], dtype: str = "bfloat16", *, random_seed: Optional[int] = None,
+         init_std: float = 0.02, device: str = "cuda:0", page_size: int = 16, num_pages: int = 0,
+         max_cache_tokens: int = 0, memory_fraction: float = 0.85, max_seqs: int = 64, max_batch_tokens: int = 2048,
+         max_seq_len: int = 0, use_graphs: bool = True) -> LLM:
+    """A model folder (config.json + safetensors), or a configuration (a dict of config.json
+    keys or a ModelConfig) with `random_seed` for random weights, to a ready `LLM`."""
+    rt = Runtime(dtype, device)
+    if isinstance(model, str):
+        m = load_model(model, rt)
+    else:
+        config = config_from_dict(model) if isinstance(model, dict) else model
+        if random_seed is None:
+            raise ValueError("a configuration without a model folder needs random_seed")
+        m = random_model(config, rt, random_seed, init_std)
+    cfg = EngineConfig(dtype=dtype, page_size=page_size, num_pages=num_pages, max_cache_tokens=max_cache_tokens,
+                       memory_fraction=memory_fraction, max_seqs=max_seqs, max_batch_tokens=max_batch_tokens,
+                       max_seq_len=max_seq_len, use_graphs=use_graphs)
+    return LLM(m, rt, cfg)

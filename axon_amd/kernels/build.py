@@ -29,7 +29,7 @@ ARCH = "gfx950"
 
 KERNEL_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "attention.hip", "attention_mfma.hip",
                   "sampling.hip"]
-HOST_SOURCES = ["host/cache.cpp", "host/scheduler.cpp"]
+HOST_SOURCES = ["host/cache.cpp", "host/scheduler.cpp", "host/sampler.cpp"]
 
 # Packed 32-bit float instructions are switched off for all device code.
 HIP_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
