@@ -30,6 +30,10 @@ class GenStats:
     decided: int = 0
     preemptions: int = 0
     seconds: float = 0.0
+    prompt_seconds: float = 0.0     # steps that fed prompt tokens
+    decode_seconds: float = 0.0     # steps that only decoded
+    decode_steps: int = 0
+    decode_tokens: int = 0
 
 
 @dataclass
@@ -102,6 +106,7 @@ class LLM:
                     raise RuntimeError("the scheduler has requests but planned nothing: the cache pool is too small")
                 entries = [StepEntry(p.id, reqs[p.id].tokens[p.start:p.start + p.count],
                                      [p.count - 1] if p.wants_logits else []) for p in plan]
+                t_step = time.time()
                 logits = self.engine.step(entries)
                 stats.steps += 1
                 wanted = [p for p in plan if p.wants_logits]
@@ -130,6 +135,14 @@ class LLM:
                     if finished:
                         r.done = True
                         self.engine.release(p.id)
+                dt = time.time() - t_step
+                if all(p.count == 1 and p.start > 0 for p in plan):
+                    stats.decode_seconds += dt
+                    stats.decode_steps += 1
+                    stats.decode_tokens += len(plan)
+                else:
+                    stats.prompt_seconds += dt
+                    stats.prompt_tokens += sum(p.count for p in plan if p.wants_logits and p.count > 1)
         finally:
             for rid in order:
                 self.engine.release(rid)
