@@ -1,0 +1,277 @@
+"""Each kernel alone against its plain reference, at other sizes than the engine's tests use,
+in float32 and in bfloat16.  Where random inputs would hide a fault (a far key among hundreds,
+a window's edge, a page's edge) the inputs are made so that it shows."""
+import math
+
+import pytest
+import torch
+
+from axon_amd.kernels import MODE_ADD_F32, MODE_STORE, MODE_STORE_F32, KernelError, kernels
+from gpu_helpers import DTYPES, TORCH, paged_cache, tol
+from plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+def as_dtype(x, dtype):
+    """Round to the compute dtype and return (device tensor, float64 copy of the rounded values)."""
+    d = x.to(TORCH[dtype])
+    return d.cuda(), d.double()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(dtype):
+    k = kernels(dtype)
+    table, ref = as_dtype(rnd(37, 100), dtype)
+    tokens = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32).cuda()
+    out = torch.empty(5, 100, dtype=torch.float32, device="cuda")
+    k.embed(tokens, table, out)
+    assert torch.equal(out.cpu().double(), ref[tokens.cpu().long()])          # exact: a widening copy
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dim,eps", [(100, 1e-6), (777, 0.5), (3584, 1e-5), (8, 1e-3)])
+def test_rmsnorm(dtype, dim, eps):
+    k = kernels(dtype)
+    x = rnd(6, dim, seed=1, scale=3.0)
+    for gdt in (torch.float32, torch.bfloat16):                                # a gain keeps its stored precision
+        gain = (1 + 0.3 * rnd(dim, seed=2)).to(gdt)
+        out = torch.empty(6, dim, dtype=TORCH[dtype], device="cuda")
+        k.rmsnorm(x.cuda(), gain.cuda(), eps, out)
+        ref = P.rms_norm(x.double(), gain.double(), eps)
+        assert (out.cpu().double() - ref).abs().max() <= tol(dtype, ref, 1e-6, 8e-3)
+    rows = torch.tensor([4, 0, 4], dtype=torch.int32).cuda()                   # gathered rows (the wanted places)
+    out = torch.empty(3, dim, dtype=TORCH[dtype], device="cuda")
+    k.rmsnorm(x.cuda(), gain.cuda(), eps, out, rows)
+    ref = P.rms_norm(x[[4, 0, 4]].double(), gain.double(), eps)
+    assert (out.cpu().double() - ref).abs().max() <= tol(dtype, ref, 1e-6, 8e-3)
+
+
+def test_rope_table_is_float64_accurate():
+    k = kernels("float32")
+    pos = torch.tensor([0, 1, 2, 77, 4095, 32767, 131071], dtype=torch.int32)
+    for hd, theta in [(16, 1e4), (128, 1e6), (80, 5e4)]:
+        freqs = P.rope_freqs(hd, theta)
+        out = torch.empty(len(pos), hd // 2, 2, dtype=torch.float32, device="cuda")
+        k.rope_table(pos.cuda(), freqs.cuda(), out)
+        sin, cos = P.rope_table(pos, freqs)
+        assert (out[..., 0].cpu().double() - sin).abs().max() < 1e-7           # float32 rounding of a float64 value
+        assert (out[..., 1].cpu().double() - cos).abs().max() < 1e-7
+        assert torch.equal(out[0, :, 0].cpu(), torch.zeros(hd // 2)) and torch.equal(out[0, :, 1].cpu(), torch.ones(hd // 2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,page", [(4, 2, 16, 8), (3, 1, 32, 16), (6, 3, 80, 4), (7, 7, 48, 5), (28, 4, 128, 16)])
+def test_rope_and_cache_store(dtype, nh, nkv, hd, page):
+    k = kernels(dtype)
+    T = 11
+    qkv, ref = as_dtype(rnd(T, (nh + 2 * nkv) * hd, seed=3), dtype)
+    pos = torch.tensor([5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15], dtype=torch.int32)
+    rows = torch.zeros(T, dtype=torch.int32)
+    n_pages = 9
+    table = torch.tensor([[7, 2, 5, 0, 3, 1, 8, 4]], dtype=torch.int32)       # scattered pages
+    kc = torch.zeros(n_pages, nkv, page, hd, dtype=TORCH[dtype], device="cuda")
+    vc = torch.zeros_like(kc)
+    freqs = P.rope_freqs(hd, 1e4)
+    tab = torch.empty(T, hd // 2, 2, dtype=torch.float32, device="cuda")
+    k.rope_table(pos.cuda(), freqs.cuda(), tab)
+    k.rope_kv_write(qkv, tab, pos.cuda(), rows.cuda(), table.cuda(), kc, vc, nh, nkv, hd, hd, page)
+    sin, cos = P.rope_table(pos, freqs)
+    q_ref = P.apply_rope(ref[:, :nh * hd].view(T, nh, hd), sin, cos)
+    k_ref = P.apply_rope(ref[:, nh * hd:(nh + nkv) * hd].view(T, nkv, hd), sin, cos)
+    v_ref = ref[:, (nh + nkv) * hd:].view(T, nkv, hd)
+    t = tol(dtype, q_ref, 1e-6, 8e-3)
+    assert (qkv[:, :nh * hd].cpu().double().view(T, nh, hd) - q_ref).abs().max() <= t
+    for i, p in enumerate(pos.tolist()):
+        pg, o = int(table[0, p // page]), p % page
+        assert (kc[pg, :, o].cpu().double() - k_ref[i]).abs().max() <= t
+        assert torch.equal(vc[pg, :, o].cpu().double(), v_ref[i])              # values are stored as they are
+    written = sum(1 for _ in pos)
+    assert int((vc.abs().sum(dim=(1, 3)) > 0).sum()) == written                # nothing else was touched
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,page,T,window", [
+    (4, 2, 16, 8, 70, 0), (3, 1, 32, 16, 133, 0), (6, 3, 80, 4, 65, 0), (8, 2, 128, 16, 200, 0), (4, 4, 64, 64, 130, 0),
+    (4, 2, 16, 8, 150, 37), (2, 1, 48, 5, 129, 64), (5, 5, 256, 16, 40, 0)])
+def test_attention_over_the_paged_cache(dtype, nh, nkv, hd, page, T, window):
+    k = kernels(dtype)
+    q, qr = as_dtype(rnd(T, nh, hd, seed=4), dtype)
+    kk, kr = as_dtype(rnd(T, nkv, hd, seed=5), dtype)
+    vv, vr = as_dtype(rnd(T, nkv, hd, seed=6), dtype)
+    kc, vc, table = paged_cache(kr, vr, page, dtype)
+    pos = torch.arange(T, dtype=torch.int32).cuda()
+    rows = torch.zeros(T, dtype=torch.int32).cuda()
+    out = torch.empty(T, nh * hd, dtype=TORCH[dtype], device="cuda")
+    k.attention(q.view(T, nh * hd), nh * hd, kc, vc, table, pos, rows, out, nh, nkv, hd, page, window,
+                1.0 / math.sqrt(hd))
+    ref = P.causal_attention(qr, kr, vr, window).view(T, nh * hd)
+    assert not torch.isnan(out).any()                                          # rows past a token's position hold NaN
+    assert (out.cpu().double() - ref).abs().max() <= tol(dtype, ref, 2e-6, 1e-2)
+    # a decode row alone (one token at the last position, queried out of order) is the same row
+    last = torch.tensor([T - 1], dtype=torch.int32).cuda()
+    one = torch.empty(1, nh * hd, dtype=TORCH[dtype], device="cuda")
+    k.attention(q[T - 1:].view(1, nh * hd), nh * hd, kc, vc, table, last, rows[:1], one, nh, nkv, hd, page, window,
+                1.0 / math.sqrt(hd))
+    assert torch.equal(one[0], out[T - 1])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_a_far_key_and_respects_the_windows_edge(dtype):
+    k = kernels(dtype)
+    nh, nkv, hd, page, T = 4, 2, 32, 16, 700
+    q = rnd(T, nh, hd, seed=7) * 0.1
+    kk = rnd(T, nkv, hd, seed=8) * 0.1
+    vv = rnd(T, nkv, hd, seed=9)
+    far = 15                                              # the last slot of the first page, hundreds of keys away
+    kk[far, 1] = 0
+    kk[far, 1, 3] = 40.0
+    q[T - 1, 2] = 0
+    q[T - 1, 2, 3] = 40.0                                 # head 2 reads kv head 1: score 1600 / sqrt(32) stands out
+    qd, qr = as_dtype(q, dtype)
+    _, kr = as_dtype(kk, dtype)
+    _, vr = as_dtype(vv, dtype)
+    kc, vc, table = paged_cache(kr, vr, page, dtype)
+    pos = torch.tensor([T - 1], dtype=torch.int32).cuda()
+    rows = torch.zeros(1, dtype=torch.int32).cuda()
+    out = torch.empty(1, nh * hd, dtype=TORCH[dtype], device="cuda")
+    scale = 1.0 / math.sqrt(hd)
+    k.attention(qd[T - 1:].view(1, -1), nh * hd, kc, vc, table, pos, rows, out, nh, nkv, hd, page, 0, scale)
+    got = out.cpu().double().view(nh, hd)
+    assert (got[2] - vr[far, 1]).abs().max() < 1e-2       # all the weight is on the far key
+    ref = P.causal_attention(qr, kr, vr)[T - 1]
+    assert (got - ref).abs().max() <= tol(dtype, ref, 2e-6, 1e-2)
+    # the window's edge: with window w the token at T-1 sees T-w .. T-1.  Put the loud key just
+    # outside, then just inside.
+    for w, seen in ((T - 1 - far, False), (T - far, True)):
+        k.attention(qd[T - 1:].view(1, -1), nh * hd, kc, vc, table, pos, rows, out, nh, nkv, hd, page, w, scale)
+        got = out.cpu().double().view(nh, hd)
+        ref = P.causal_attention(qr, kr, vr, w)[T - 1]
+        assert (got - ref).abs().max() <= tol(dtype, ref, 2e-6, 1e-2)
+        assert ((got[2] - vr[far, 1]).abs().max() < 1e-2) == seen
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (3, 100, 70), (17, 259, 130), (70, 96, 33), (130, 48, 257),
+                                   (5, 1000, 512), (64, 256, 256), (200, 384, 1024), (33, 152, 3584)])
+def test_gemm_every_epilogue(dtype, M, N, K):
+    k = kernels(dtype)
+    x, xr = as_dtype(rnd(M, K, seed=10), dtype)
+    w, wr = as_dtype(rnd(N, K, seed=11, scale=0.2), dtype)
+    ref = xr @ wr.T
+    for bias_dt in (None, torch.float32, torch.bfloat16):
+        bias = None if bias_dt is None else rnd(N, seed=12).to(bias_dt)
+        want = ref if bias is None else ref + bias.double()
+        b = None if bias is None else bias.cuda()
+        out = torch.empty(M, N, dtype=TORCH[dtype], device="cuda")
+        k.gemm(x, w, out, b, MODE_STORE)
+        assert (out.cpu().double() - want).abs().max() <= tol(dtype, want, 2e-6 * math.sqrt(K), 1e-2)
+        f32 = torch.empty(M, N, dtype=torch.float32, device="cuda")
+        k.gemm(x, w, f32, b, MODE_STORE_F32)
+        assert (f32.cpu().double() - want).abs().max() <= tol(dtype, want, 2e-6 * math.sqrt(K), 2e-5 * math.sqrt(K))
+        res = rnd(M, N, seed=13).cuda()
+        acc = res.clone()
+        k.gemm(x, w, acc, b, MODE_ADD_F32)
+        assert (acc.cpu().double() - (want + res.cpu().double())).abs().max() <= tol(dtype, want, 2e-6 * math.sqrt(K),
+                                                                                      2e-5 * math.sqrt(K))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_rows_do_not_depend_on_the_batch(dtype):
+    """The same row of x gives the same bits whatever rows ride along (1, 3, 16, 17, 64, 200)."""
+    k = kernels(dtype)
+    for N, K in [(96, 80), (256, 512), (130, 1000)]:
+        x, _ = as_dtype(rnd(200, K, seed=14), dtype)
+        w, _ = as_dtype(rnd(N, K, seed=15, scale=0.2), dtype)
+        full = torch.empty(200, N, dtype=torch.float32, device="cuda")
+        k.gemm(x, w, full, None, MODE_STORE_F32)
+        for m in (1, 3, 16, 17, 64, 130):
+            part = torch.empty(m, N, dtype=torch.float32, device="cuda")
+            k.gemm(x[:m], w, part, None, MODE_STORE_F32)
+            assert torch.equal(part, full[:m]), (N, K, m)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_strided_rows(dtype):
+    k = kernels(dtype)
+    big, br = as_dtype(rnd(9, 300, seed=16), dtype)
+    w, wr = as_dtype(rnd(50, 100, seed=17, scale=0.3), dtype)
+    out = torch.zeros(9, 80, dtype=TORCH[dtype], device="cuda")
+    k.gemm(big[:, 100:200], w, out[:, 10:60], None, MODE_STORE)              # a slice in, a slice out
+    want = br[:, 100:200] @ wr.T
+    assert (out[:, 10:60].cpu().double() - want).abs().max() <= tol(dtype, want, 1e-5, 1e-2)
+    assert out[:, :10].abs().sum() == 0 and out[:, 60:].abs().sum() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(dtype):
+    k = kernels(dtype)
+    T, Fn = 7, 203
+    gu, gr = as_dtype(rnd(T, 2 * Fn, seed=18, scale=4.0), dtype)
+    gu[0, 0], gu[0, Fn] = -200.0, 1.0
+    gu[0, 1], gu[0, Fn + 1] = 200.0, 1.0
+    gr = gu.cpu().double()
+    out = torch.empty(T, Fn, dtype=TORCH[dtype], device="cuda")
+    k.swiglu(gu, out)
+    ref = P.swiglu(gr[:, :Fn], gr[:, Fn:])
+    assert (out.cpu().double() - ref).abs().max() <= tol(dtype, ref, 1e-6, 8e-3)
+    assert out[0, 0].item() == 0.0 and out[0, 1].item() == 200.0               # src/vmath.rs:495-497
+
+
+def test_argmax_rules_on_the_device():
+    k = kernels("float32")
+    inf, nan = float("inf"), float("nan")
+    rows = [[-inf] * 5, [1.0, 3.0, 3.0, 2.0, 0.0], [nan, 1.0, nan, 0.5, 1.0], [nan] * 5, [-1.0, 0.0, -0.0, -2.0, -3.0]]
+    logits = torch.tensor(rows, dtype=torch.float32).cuda()
+    out = torch.empty(5, dtype=torch.int32, device="cuda")
+    k.argmax(logits, out)
+    assert out.tolist() == [P.argmax_last(r) for r in rows] == [4, 2, 4, 4, 2]
+    big = rnd(3, 152064, seed=19).cuda()
+    big[1, 777] = big[1, 150000] = 9.0                                         # a tie far apart: the last wins
+    out = torch.empty(3, dtype=torch.int32, device="cuda")
+    k.argmax(big, out)
+    assert out.tolist() == [int(big[0].argmax()), 150000, int(big[2].argmax())]
+
+
+def test_topk_with_penalty_on_the_device():
+    k = kernels("float32")
+    V = 5003
+    logits = rnd(4, V, seed=20, scale=2.0)
+    logits[1, 10] = logits[1, 4000] = logits[1].max() + 1                      # ties at the top
+    logits[2, 5] = float("nan")
+    recent = torch.tensor([[3, 5, 1, 1, 2, 1, 0, 0], [10, 10, 4000, 7, 0, 0, 0, 0], [0] * 8, [9] * 8], dtype=torch.int32)
+    n_recent = torch.tensor([6, 4, 0, 8], dtype=torch.int32)
+    penalty = torch.tensor([2.0, 1.3, 1.0, 1.1])
+    ks = torch.tensor([40, 7, 256, 1], dtype=torch.int32)
+    dev = logits.clone().cuda()
+    cands = torch.zeros(4, 256, dtype=torch.int64, device="cuda")
+    k.topk(dev, recent.cuda(), n_recent.cuda(), penalty.cuda(), ks.cuda(), cands)
+    for r in range(4):
+        pen = P.penalize(logits[r].tolist(), recent[r, :n_recent[r]].tolist(), 10 ** 6, float(penalty[r]))
+        pen = torch.tensor(pen, dtype=torch.float32)
+        assert torch.equal(dev[r].cpu().nan_to_num(7.0), pen.nan_to_num(7.0))   # penalised in place, each id once
+        want = [i for _, i in P.candidates(pen.tolist(), int(ks[r]))]
+        got = sorted(cands[r, :int(ks[r])].tolist(), reverse=True)
+        assert [g & 0xFFFFFFFF for g in got] == want, r
+
+
+def test_kernels_refuse_what_they_cannot_run():
+    k = kernels("float32")
+    x = torch.zeros(2, 8, device="cuda")
+    with pytest.raises(KernelError):
+        k.gemm(x, torch.zeros(4, 9, device="cuda"), torch.zeros(2, 4, device="cuda"))       # K differs
+    with pytest.raises(KernelError):
+        k.gemm(x.bfloat16(), torch.zeros(4, 8, device="cuda"), torch.zeros(2, 4, device="cuda"))   # wrong dtype
+    with pytest.raises(KernelError):
+        k.gemm(x.cpu(), torch.zeros(4, 8), torch.zeros(2, 4))                               # not on the device
+    q = torch.zeros(1, 24, device="cuda")
+    cache = torch.zeros(2, 1, 8, 24, device="cuda")
+    i32 = torch.zeros(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(KernelError) as e:
+        k.attention(q, 24, cache, cache, i32.view(1, 1), i32, i32, torch.zeros(1, 24, device="cuda"), 1, 1, 24, 8, 0,
+                    1.0)
+    assert "head_dim 24" in str(e.value)

@@ -1,0 +1,138 @@
+"""Trace replay through bin/trace_run, as a user drives it: the same requests whole, with the
+last 32 tokens decoded one by one, in portions of changing size down to two tokens, and mixed
+with other requests in a pool so small that pages are used again; float32 and bfloat16; all
+compared with the plain implementation."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import TINY, TraceBuilder, prompts_for, run_trace, tolerance
+from plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [1, 5, 17, 33, 70, 100], "B": [2, 9, 70, 41, 130, 64], "C": [3, 66, 129]}
+
+
+def oracle(model_dir, prompts):
+    cfg, w = P.load_plain(model_dir)
+    return [P.forward_logits(cfg, w, p).float().numpy() for p in prompts]
+
+
+def check(rows, refs, ids, dtype):
+    worst = 0.0
+    for (rid, pos), got in rows.items():
+        ref = refs[ids.index(rid)][pos]
+        tol = tolerance(dtype, torch.from_numpy(refs[ids.index(rid)]))
+        err = float(np.abs(got - ref).max())
+        assert err <= tol, f"request {rid} position {pos}: |diff| {err} > {tol}"
+        worst = max(worst, err)
+    return worst
+
+
+def whole(prompts):
+    tb = TraceBuilder()
+    for i, p in enumerate(prompts):
+        tb.step([(f"r{i}", p, list(range(len(p))))], end=[f"r{i}"])
+    return tb
+
+
+def last_32_one_by_one(prompts):
+    tb = TraceBuilder()
+    for i, p in enumerate(prompts):
+        head = max(len(p) - 32, 1)
+        tb.step([(f"r{i}", p[:head], [head - 1])])
+        for t in range(head, len(p)):
+            tb.step([(f"r{i}", [p[t]], [0])], end=[f"r{i}"] if t == len(p) - 1 else [])
+        if head == len(p):
+            tb.step([], end=[f"r{i}"])
+    return tb
+
+
+def changing_portions(prompts, sizes=(7, 2, 16, 3, 2, 33, 1, 5, 64, 2)):
+    tb = TraceBuilder()
+    for i, p in enumerate(prompts):
+        at, k = 0, i
+        while at < len(p):
+            n = min(sizes[k % len(sizes)], len(p) - at)
+            tb.step([(f"r{i}", p[at:at + n], list(range(n)))], end=[f"r{i}"] if at + n == len(p) else [])
+            at, k = at + n, k + 1
+    return tb
+
+
+def mixed(prompts, seed=0, live_at_most=4):
+    """Up to four live requests: portions of some beside single tokens of others; a request
+    may sit out a step; finished requests give their pages to the ones that start later."""
+    rng = np.random.default_rng(seed)
+    tb = TraceBuilder()
+    waiting = list(range(len(prompts)))
+    live = {}
+    while waiting or live:
+        while waiting and len(live) < live_at_most:
+            live[waiting.pop(0)] = 0
+        entries, end = [], []
+        for i in list(live):
+            if len(live) > 1 and rng.random() < 0.2:
+                continue                                         # left out of this step
+            p, at = prompts[i], live[i]
+            decode = at >= max(len(p) - 32, 1) or rng.random() < 0.3
+            n = 1 if decode else int(min(rng.choice([2, 3, 7, 16, 29]), len(p) - at))
+            entries.append((f"r{i}", p[at:at + n], list(range(n)) if rng.random() < 0.8 else [n - 1]))
+            live[i] = at + n
+            if live[i] == len(p):
+                end.append(f"r{i}")
+                del live[i]
+        if entries:
+            tb.step(entries, end)
+    return tb
+
+
+def max_tokens_for(tb, prompts_by_id):
+    """The most tokens live requests hold at any time, each rounded up to 64."""
+    live, most = {}, 0
+    for s in tb.steps:
+        for e in s["entries"]:
+            live[e["id"]] = live.get(e["id"], 0) + len(e["tokens"])
+        most = max(most, sum(-(-n // 64) * 64 for n in live.values()))
+        for rid in s["end"]:
+            live.pop(rid, None)
+    return most
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_every_schedule_matches_the_plain_implementation(name, dtype, model_dirs, tmp_path):
+    model_dir = model_dirs(name, "float32" if dtype == "float32" else "bfloat16")
+    prompts = prompts_for(name, LENGTHS[name], seed=3)
+    ids = [f"r{i}" for i in range(len(prompts))]
+    refs = oracle(model_dir, prompts)
+    page = ["--page-size", str(TINY[name]["page_size"])]
+    results = {}
+    for label, tb in (("whole", whole(prompts)), ("last32", last_32_one_by_one(prompts)),
+                      ("portions", changing_portions(prompts)), ("mixed", mixed(prompts, seed=len(name)))):
+        budget = max_tokens_for(tb, None)
+        out = run_trace(model_dir, dtype, tb.steps, str(tmp_path / label), budget, extra=page)
+        rows = tb.collect(out)
+        check(rows, refs, ids, dtype)
+        results[label] = rows
+    # every position was asked for in the whole and portions schedules
+    assert len(results["whole"]) == sum(len(p) for p in prompts) == len(results["portions"])
+    if dtype == "float32":
+        # beyond the tolerance: however the tokens were cut, the float32 logits are the same bits
+        for label in ("last32", "portions", "mixed"):
+            for key, row in results[label].items():
+                assert np.array_equal(row, results["whole"][key]), (label, key)
+
+
+def test_a_step_that_wants_nothing_writes_nothing_and_requests_can_pause(model_dirs, tmp_path):
+    model_dir = model_dirs("A")
+    p, q = prompts_for("A", [20, 12], seed=9)
+    tb = TraceBuilder()
+    tb.step([("a", p[:10], [])])                                  # nothing wanted: no file
+    tb.step([("b", q[:12], [11])])                                # "a" is left out of this step
+    tb.step([("a", p[10:], [9])], end=["a", "b"])
+    out = run_trace(model_dir, "float32", tb.steps, str(tmp_path / "o"), 128, extra=["--page-size", "8"])
+    assert sorted(out) == [1, 2]
+    rows = tb.collect(out)
+    refs = oracle(model_dir, [p, q])
+    check(rows, refs, ["a", "b"], "float32")
