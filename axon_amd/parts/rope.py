@@ -22,7 +22,7 @@ class RotaryEncoding(PositionEncoding):
         self.theta = float(params["theta"])
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
             raise ConfigError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {self.head_dim}")
-        self.key = ("rope", self.rotary_dim, self.theta)
+        self.key = None
         self._freqs = None
 
     def frequencies(self) -> torch.Tensor:
@@ -30,7 +30,11 @@ class RotaryEncoding(PositionEncoding):
         return torch.tensor([self.theta ** (-2.0 * i / self.rotary_dim) for i in range(n)], dtype=torch.float64)
 
     def load(self, store, rt) -> None:
-        self._freqs = self.frequencies().to(rt.device)
+        f = self.frequencies()
+        # encodings with the same frequencies share one table per step; a subclass that
+        # changes the frequencies gets a table of its own
+        self.key = ("rotary", tuple(f.tolist()))
+        self._freqs = f.to(rt.device)
 
     def tables(self, ctx) -> torch.Tensor:
         """float32 [T, rotary_dim / 2, 2] for the positions of this step (made once per step)."""

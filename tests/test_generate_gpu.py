@@ -1,0 +1,161 @@
+"""Generation through the Python entry point and the command line against the plain
+implementation: greedy, sampled with a seed, under page pressure (requests give way and come
+back), long decoding, and the first tokens of a sequence."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import axon_amd
+from helpers import ROOT, TINY, prompts_for, tolerance
+from plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_matches_the_plain_loop(name, dtype, model_dirs):
+    d = model_dirs(name, "float32" if dtype == "float32" else "bfloat16")
+    cfg, w = P.load_plain(d)
+    prompts = prompts_for(name, [1, 5, 17, 33] if name == "A" else [2, 9, 70, 41, 3, 25], seed=1)
+    n_new = 16 if name == "A" else 24
+    llm = axon_amd.load(d, dtype=dtype, page_size=TINY[name]["page_size"], num_pages=64, max_seqs=4, max_batch_tokens=48)
+    outs = llm.generate(prompts, max_new_tokens=n_new)
+    for p, o in zip(prompts, outs):
+        assert len(o) == n_new
+        if dtype == "float32":
+            assert o == P.greedy_generate(cfg, w, p, n_new)
+        else:
+            # bfloat16 may take another branch at a near tie: follow the engine's own tokens and
+            # require each pick to be within tolerance of the oracle's best logit
+            logits = P.forward_logits(cfg, w, p + o)
+            for i, tok in enumerate(o):
+                row = logits[len(p) - 1 + i]
+                assert row.max() - row[tok] <= 2 * tolerance(dtype, row), (i, tok)
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_pages() == 64 and not llm.engine.live
+
+
+def test_sampled_generation_matches_the_plain_sampler(model_dirs):
+    d = model_dirs("B")
+    cfg, w = P.load_plain(d)
+    prompts = prompts_for("B", [2, 30, 11], seed=2)
+    llm = axon_amd.load(d, dtype="float32", page_size=16, num_pages=32, max_seqs=4)
+    kw = dict(temperature=0.8, top_k=40, top_p=0.9, min_p=0.0, repeat_penalty=1.1, repeat_last_n=64)
+    outs = llm.generate(prompts, max_new_tokens=24, seed=5, **kw)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        assert o == P.sample_generate(cfg, w, p, 24, temp=0.8, top_k=40, top_p=0.9, min_p=0.0, repeat_penalty=1.1,
+                                      repeat_last_n=64, seed=5 + i)
+    # the same seed gives the same tokens whatever else is in the batch
+    alone = llm.generate([prompts[1]], max_new_tokens=24, seed=6, **kw)[0]
+    assert alone == llm.generate(prompts, max_new_tokens=24, seed=5, **kw)[1]
+    # top-k off (every token a candidate) and top-k above the device's limit run on the host
+    for k in (0, 300):
+        o = llm.generate([prompts[0]], max_new_tokens=8, seed=9, temperature=1.2, top_k=k, top_p=1.0, repeat_penalty=1.0)[0]
+        assert o == P.sample_generate(cfg, w, prompts[0], 8, temp=1.2, top_k=k, top_p=1.0, min_p=0.0,
+                                      repeat_penalty=1.0, repeat_last_n=64, seed=9)
+
+
+def test_stop_tokens_end_a_request_and_are_not_returned(model_dirs):
+    d = model_dirs("A")
+    cfg, w = P.load_plain(d)
+    p = prompts_for("A", [9], seed=4)[0]
+    full = P.greedy_generate(cfg, w, p, 12)
+    stop = full[5]
+    want = P.greedy_generate(cfg, w, p, 12, stop=[stop])
+    assert len(want) < 12
+    llm = axon_amd.load(d, dtype="float32", page_size=8, num_pages=16, max_seqs=2)
+    assert llm.generate(p, max_new_tokens=12, stop=[stop]) == [want]
+    assert llm.generate(p, max_new_tokens=0) == [[]]
+
+
+def test_under_page_pressure_requests_give_way_and_continue_with_the_same_tokens(model_dirs):
+    d = model_dirs("B")
+    cfg, w = P.load_plain(d)
+    prompts = prompts_for("B", [20, 25, 18, 30, 22], seed=6)
+    roomy = axon_amd.load(d, dtype="float32", page_size=16, num_pages=64, max_seqs=4, max_batch_tokens=32)
+    want = roomy.generate(prompts, max_new_tokens=40)
+    assert roomy.last_stats.preemptions == 0
+    # 9 pages of 16: one request needs up to 70 tokens = 5 pages, so two cannot both finish
+    tight = axon_amd.load(d, dtype="float32", page_size=16, num_pages=9, max_seqs=4, max_batch_tokens=32)
+    got = tight.generate(prompts, max_new_tokens=40)
+    assert tight.last_stats.preemptions > 0
+    assert got == want == [P.greedy_generate(cfg, w, p, 40) for p in prompts]
+    tight.engine.cache.check()
+    assert tight.engine.cache.free_pages() == 9
+    # sampled requests keep their random stream across a preemption
+    s_want = roomy.generate(prompts, max_new_tokens=30, temperature=0.9, seed=3)
+    s_got = tight.generate(prompts, max_new_tokens=30, temperature=0.9, seed=3)
+    assert s_got == s_want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_stays_on_the_oracle(dtype, model_dirs):
+    """300 tokens decoded one by one after a short prompt (pages 8: dozens of page edges, five
+    attention blocks), then every decode step's logits against the whole sequence at once."""
+    d = model_dirs("A", "float32" if dtype == "float32" else "bfloat16")
+    cfg, w = P.load_plain(d)
+    p = prompts_for("A", [3], seed=8)[0]
+    c = dict(TINY["A"]["config"], max_position_embeddings=512)
+    import json, shutil, tempfile
+    tmp = tempfile.mkdtemp()
+    try:
+        shutil.copy(os.path.join(d, "model.safetensors"), tmp)
+        json.dump(c, open(os.path.join(tmp, "config.json"), "w"))
+        llm = axon_amd.load(tmp, dtype=dtype, page_size=8, num_pages=48, max_seqs=2)
+        out = llm.generate(p, max_new_tokens=300)[0]
+        seq = p + out
+        ref = P.forward_logits(cfg, w, seq).float()
+        from axon_amd.engine import StepEntry
+        eng = llm.engine
+        eng.step([StepEntry("x", seq[:3], [])])
+        worst = 0.0
+        for t in range(3, len(seq)):
+            row = eng.step([StepEntry("x", [seq[t]], [0])])[0].cpu()
+            worst = max(worst, float((row - ref[t]).abs().max()))
+        eng.release("x")
+        assert worst <= tolerance(dtype, ref), worst
+    finally:
+        shutil.rmtree(tmp)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_first_tokens_of_a_sequence(dtype, model_dirs):
+    """Position 0 alone, then 1, 2, 3: no earlier key, the rotation is the identity at 0."""
+    d = model_dirs("B", "float32" if dtype == "float32" else "bfloat16")
+    cfg, w = P.load_plain(d)
+    llm = axon_amd.load(d, dtype=dtype, page_size=16, num_pages=8, max_seqs=2)
+    for p in prompts_for("B", [1, 1, 2, 4], seed=10):
+        ref = P.forward_logits(cfg, w, p).float()
+        got = llm.logits(p, all_positions=True).cpu()
+        assert (got - ref).abs().max() <= tolerance(dtype, ref)
+        one = llm.logits(p).cpu()
+        assert torch.equal(one, got[-1])
+
+
+def test_command_line_gen_and_logits(model_dirs):
+    d = model_dirs("A")
+    cfg, w = P.load_plain(d)
+    p = prompts_for("A", [7], seed=11)[0]
+    ids = " ".join(map(str, p))
+    axon = [sys.executable, os.path.join(ROOT, "bin", "axon")]
+    r = subprocess.run(axon + ["gen", d, ids, "-n", "10", "--dtype", "float32", "--page-size", "8"], capture_output=True,
+                       text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert [int(t) for t in r.stdout.split()] == P.greedy_generate(cfg, w, p, 10)
+    assert "prompt eval: 7 tok" in r.stderr and "decode: " in r.stderr and "tok/s" in r.stderr
+    r = subprocess.run(axon + ["gen", d, ids, "-n", "6", "--dtype", "float32", "--temp", "0.7", "--seed", "4"],
+                       capture_output=True, text=True, timeout=300)
+    assert [int(t) for t in r.stdout.split()] == P.sample_generate(
+        cfg, w, p, 6, temp=0.7, top_k=40, top_p=0.9, min_p=0.0, repeat_penalty=1.1, repeat_last_n=64, seed=4)
+    r = subprocess.run(axon + ["logits", d, ids, "-k", "3", "--dtype", "float32"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr
+    ref = P.forward_logits(cfg, w, p)[-1]
+    top = torch.topk(ref, 3)
+    lines = [l.split() for l in r.stdout.splitlines() if "logit" in l]
+    assert [int(l[0]) for l in lines] == top.indices.tolist()
+    assert all(abs(float(l[2]) - v) < 1e-3 for l, v in zip(lines, top.values.tolist()))
