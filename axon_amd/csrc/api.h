@@ -34,7 +34,8 @@ int axk_rope_table(const int32_t* positions, const double* freqs, float* table, 
 
 // Rotate-half on the first `rotary_dim` dims of each q and k head of qkv [T, (nh + 2 nkv) hd]
 // (q in place), and store k and v rows into the paged cache at each token's position.
-// write_kv = 0 rotates q only.  Cache layout per array: [page][kv head][slot in page][hd].
+// write_kv = 0 rotates q only.  Cache layout: keys [page][kv head][slot in page][hd], values
+// [page][kv head][hd][slot in page] (the positions of one dim are contiguous).
 int axk_rope_kv_write(void* qkv, const float* table, const int32_t* positions, const int32_t* seq_rows,
                       const int32_t* block_table, int table_stride, void* k_cache, void* v_cache,
                       int n_tokens, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
@@ -47,6 +48,26 @@ int axk_attention(const void* q, int q_stride, const void* k_cache, const void* 
                   const int32_t* block_table, int table_stride, const int32_t* positions,
                   const int32_t* seq_rows, void* out, int n_tokens, int n_heads, int n_kv_heads,
                   int head_dim, int page_size, int window, float scale, void* stream);
+
+// The matrix-core attention kernels (bfloat16 build; the float32 build refuses them).
+// axk_attention_fast_ok: 1 if they take this head size, page size and group of heads.
+// axk_attention_prefill: tiles [n_tiles][2] = (first token, count <= 128): consecutive tokens of
+// one request; every token of the step in some tile gets its row of `out`.
+// axk_attention_decode: token_index [n_tokens] names single tokens; a context longer than 256
+// positions is cut into chunks whose partial results go through `partial`
+// (axk_attention_decode_workspace floats) and are folded in ascending order.
+int axk_attention_fast_ok(int head_dim, int page_size, int n_heads, int n_kv_heads);
+int axk_attention_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                          const int32_t* block_table, int table_stride, const int32_t* positions,
+                          const int32_t* seq_rows, void* out, const int32_t* tiles, int n_tiles,
+                          int n_heads, int n_kv_heads, int head_dim, int page_size, int window,
+                          float scale, void* stream);
+long axk_attention_decode_workspace(int n_tokens, int n_heads, int head_dim, int max_chunks);
+int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                         const int32_t* block_table, int table_stride, const int32_t* positions,
+                         const int32_t* seq_rows, void* out, const int32_t* token_index, int n_tokens,
+                         float* partial, int max_chunks, int n_heads, int n_kv_heads, int head_dim,
+                         int page_size, int window, float scale, void* stream);
 
 // out = epilogue(X [M, K] . W [N, K]^T + bias).  mode 0: store elem [M, N]; 1: add into
 // float32 [M, N] (the residual stream); 2: store float32 [M, N] (logits).

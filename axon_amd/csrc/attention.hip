@@ -59,7 +59,7 @@ attention_rows_kernel(const elem_t* __restrict__ q, int q_stride, const elem_t* 
       float dot = 0.0f;
       for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
       s = dot * scale;
-      vrow[lane] = cache_row(v_cache, table_row, p, page_size, n_kv_heads, kvh, head_dim);
+      vrow[lane] = v_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * head_dim * page_size + (p % page_size);
     }
     const float mb = wave_max(s);
     const float e = live ? expf(s - mb) : 0.0f;
@@ -76,7 +76,7 @@ attention_rows_kernel(const elem_t* __restrict__ q, int q_stride, const elem_t* 
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
         const int d = lane + i * AXON_WAVE;
-        if (d < head_dim) ob[i] = fmaf(ej, to_float(vr[d]), ob[i]);
+        if (d < head_dim) ob[i] = fmaf(ej, to_float(vr[(size_t)d * page_size]), ob[i]);
       }
     }
     __syncthreads();

@@ -1,0 +1,526 @@
+// Paged causal attention on the matrix cores (bfloat16 build only): one kernel for prompt
+// portions, one for decoding tokens.  Both keep the order of attention.hip: positions in
+// blocks of 64 aligned to absolute position, folded in ascending order with running
+// (max, sum, output); the decoding kernel splits a long context into chunks of 256
+// positions (4 blocks, a size that depends on nothing) and a second kernel folds the chunks
+// in ascending order.  No atomics.  Scores, softmax and all sums are 32-bit; q, k, v and the
+// softmax weights enter the MFMAs as bfloat16.
+//
+// Both compute the TRANSPOSED products, S^T = K Q^T and O^T = V^T P^T, so that what one MFMA
+// leaves in a lane's registers is what the next one wants there, without a trip through LDS:
+// after S^T a lane holds, for ONE query, several key positions; the softmax over positions is
+// then a loop over the lane's registers plus one or two exchanges between lane groups, and the
+// rounded weights are already laid out as the B operand of O^T.  The MFMA's k slots are
+// matched to the positions a lane holds by reading V^T accordingly (values are cached
+// position-contiguous: [page][kv head][dim][slot]).
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+#if AXON_BF16
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+#define LOG2E 1.4426950408889634f
+
+__device__ inline bf16x8 frag_of(uint4 v) {
+  union { uint4 u; bf16x8 f; } c;
+  c.u = v;
+  return c.f;
+}
+
+__device__ inline bf16x8 frag_of2(uint2 lo, uint2 hi) {
+  union { uint2 u[2]; bf16x8 f; } c;
+  c.u[0] = lo;
+  c.u[1] = hi;
+  return c.f;
+}
+
+__device__ inline uint32_t pack_bf16(float a, float b) {
+  return (uint32_t)float_to_bf16(a).bits | ((uint32_t)float_to_bf16(b).bits << 16);
+}
+
+// ============================================================================ prompt portions
+// grid (tiles, query heads); a tile is up to 128 consecutive tokens of one request.  4 waves,
+// each owning 32 query rows.  Per block of 64 key positions the waves bring K [64][HD] and
+// V^T [HD][64] into LDS with direct global -> LDS loads (two stages: the next block's loads are
+// in flight while this one is multiplied).  16-byte slots of an LDS row are permuted
+// (slot ^ row & 7) so that fragment reads of neighbouring rows fall into different banks.
+#define PF_TOKENS 128
+#define PF_BLOCK 64
+
+template <int HD>
+__global__ void __launch_bounds__(256)
+attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
+                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
+                         const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
+                         bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int n_heads, int n_kv_heads,
+                         int page_size, int window, float scale) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int K_BYTES = PF_BLOCK * HD * 2;      // K tile: 64 rows of HD
+  constexpr int V_BYTES = HD * PF_BLOCK * 2;      // V^T tile: HD rows of 64 positions
+  constexpr int STAGE = K_BYTES + V_BYTES;
+  constexpr int KROW = HD * 2;                    // bytes per K row
+  constexpr int KCH = HD / 8;                     // 16-byte slots per K row
+  constexpr int K_ROWS_PER_INSTR = 1024 / KROW;
+  constexpr int K_INSTR = PF_BLOCK / K_ROWS_PER_INSTR / 4;  // per wave
+  constexpr int V_INSTR = HD / 8 / 4;                       // V^T: 8 rows per instruction
+  constexpr int DT = HD / 32;                     // output tiles (32 dims each)
+  constexpr int KS = HD / 16;                     // k steps of S^T
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int t0 = tiles[2 * blockIdx.x], count = tiles[2 * blockIdx.x + 1];
+  const int head = blockIdx.y, kvh = head / (n_heads / n_kv_heads);
+  const int pos0 = positions[t0];
+  const int32_t* table_row = block_table + (size_t)seq_rows[t0] * table_stride;
+  const int hi = pos0 + count - 1;                               // last position any row of the tile sees
+  const int lo = window > 0 ? max(0, pos0 + 1 - window) : 0;     // first position any row sees
+  const int first_block = (lo / PF_BLOCK) * PF_BLOCK;
+  const int n_blocks = (hi - first_block) / PF_BLOCK + 1;
+
+  const int l32 = lane & 31, half = lane >> 5;
+  const int my_row = wave * 32 + l32;                            // this lane's query row in the tile
+  const int my_pos = pos0 + min(my_row, count - 1);
+  const int my_lo = window > 0 ? max(0, my_pos + 1 - window) : 0;
+  const int wave_hi = pos0 + min(wave * 32 + 31, count - 1);     // last position this wave's rows see
+  const bool wave_live = wave * 32 < count;
+
+  // Q^T fragments (B operand): column = query row, 8 consecutive dims from 16 ks + 8 half
+  bf16x8 qf[KS];
+  {
+    const bf16_t* qrow = q + (size_t)(t0 + min(my_row, count - 1)) * q_stride + (size_t)head * HD + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = frag_of(*reinterpret_cast<const uint4*>(qrow + ks * 16));
+  }
+
+  const size_t kv_head_stride = (size_t)HD * page_size;           // elements of one (page, kv head)
+  auto issue = [&](int b) {
+    unsigned char* stage = smem + (b & 1) * STAGE;
+    const int p0 = first_block + b * PF_BLOCK;
+    // K: lane i of an instruction brings row i / KCH, slot i % KCH holding chunk slot ^ (row & 7)
+#pragma unroll
+    for (int n = 0; n < K_INSTR; ++n) {
+      const int instr = n * 4 + wave;
+      const int row = instr * K_ROWS_PER_INSTR + lane / KCH;
+      const int chunk = (lane % KCH) ^ (row & 7);
+      const int p = min(p0 + row, hi);                            // rows past the tile's last position: any valid row
+      const bf16_t* src = k_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * kv_head_stride +
+                          (size_t)(p % page_size) * HD + chunk * 8;
+      __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + instr * 1024), 16, 0, 0);
+    }
+    // V^T: lane i brings row (dim) i / 8, slot i % 8 holding the 8 positions of chunk slot ^ (row & 7)
+#pragma unroll
+    for (int n = 0; n < V_INSTR; ++n) {
+      const int instr = n * 4 + wave;
+      const int d = instr * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ (d & 7);
+      const int p = min(p0 + chunk * 8, hi);
+      const bf16_t* src = v_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * kv_head_stride +
+                          (size_t)d * page_size + ((p % page_size) & ~7);
+      __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + K_BYTES + instr * 1024), 16, 0, 0);
+    }
+  };
+
+  f32x16 o_acc[DT];
+#pragma unroll
+  for (int i = 0; i < DT; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o_acc[i][e] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+  const float c = scale * LOG2E;
+
+  issue(0);
+  for (int b = 0; b < n_blocks; ++b) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (b + 1 < n_blocks) issue(b + 1);
+    unsigned char* stage = smem + (b & 1) * STAGE;
+    const int p0 = first_block + b * PF_BLOCK;
+    if (p0 + PF_BLOCK - 1 > hi) {
+      // the last block: positions past `hi` were never written for this request.  Their
+      // weights are zero, but zero times whatever the page holds must stay zero: clear them.
+      const int first_bad = hi - p0 + 1;
+      for (int idx = tid; idx < HD * PF_BLOCK; idx += 256) {
+        const int d = idx / PF_BLOCK, col = idx % PF_BLOCK;
+        if (col >= first_bad) {
+          const int slot = (col >> 3) ^ (d & 7);
+          *reinterpret_cast<uint16_t*>(stage + K_BYTES + d * 128 + slot * 16 + (col & 7) * 2) = 0;
+        }
+      }
+      __syncthreads();
+    }
+    if (!wave_live || p0 > wave_hi) continue;  // nothing for this wave's rows in this block (all waves reach the barriers)
+
+    // S^T [64 positions][32 queries] = K Q^T: two tiles of 32 positions
+    f32x16 s_acc[2];
+#pragma unroll
+    for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s_acc[pt][e] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+      for (int pt = 0; pt < 2; ++pt) {
+        const int row = pt * 32 + l32;
+        const int slot = (ks * 2 + half) ^ (row & 7);
+        const bf16x8 kf = frag_of(*reinterpret_cast<const uint4*>(stage + row * KROW + slot * 16));
+        s_acc[pt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s_acc[pt], 0, 0, 0);
+      }
+    }
+    // this lane: query my_row; positions p0 + pt*32 + (e/4)*8 + half*4 + e%4
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int p = p0 + pt * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+        const bool seen = p <= my_pos && p >= my_lo;
+        const float v = seen ? s_acc[pt][e] * c : -INFINITY;
+        s_acc[pt][e] = v;
+        mloc = fmaxf(mloc, v);
+      }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, AXON_WAVE));
+    const float mn = fmaxf(m_run, mloc);
+    const float mref = mn == -INFINITY ? 0.0f : mn;     // a row that has seen nothing yet
+    const float alpha = __builtin_amdgcn_exp2f(m_run - mref);
+    float lsum = 0.0f;
+#pragma unroll
+    for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const float pv = __builtin_amdgcn_exp2f(s_acc[pt][e] - mref);
+        s_acc[pt][e] = pv;
+        lsum += pv;
+      }
+    lsum += __shfl_xor(lsum, 32, AXON_WAVE);
+    l_run = l_run * alpha + lsum;
+    m_run = mn;
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+
+    // O^T [HD][32 queries] += V^T P^T.  k step s2 (16 positions) takes registers e = 8 (s2 % 2) ..
+    // + 7 of tile s2 / 2: positions (s2/2)*32 + (s2%2)*16 + half*4 + {0..3} and the same + 8.
+#pragma unroll
+    for (int s2 = 0; s2 < 4; ++s2) {
+      const int pt = s2 >> 1, e0 = (s2 & 1) * 8;
+      union { uint32_t u[4]; bf16x8 f; } pf;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) pf.u[j] = pack_bf16(s_acc[pt][e0 + 2 * j], s_acc[pt][e0 + 2 * j + 1]);
+      const int col = pt * 32 + (s2 & 1) * 16 + half * 4;   // first of the lane's 4 + 4 positions
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const int d = dt * 32 + l32;
+        const unsigned char* vrow = stage + K_BYTES + d * 128 + (col & 7) * 2;
+        const int ch = col >> 3;
+        const uint2 v0 = *reinterpret_cast<const uint2*>(vrow + ((ch ^ (d & 7)) << 4));
+        const uint2 v1 = *reinterpret_cast<const uint2*>(vrow + (((ch + 1) ^ (d & 7)) << 4));
+        o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_of2(v0, v1), pf.f, o_acc[dt], 0, 0, 0);
+      }
+    }
+  }
+
+  if (!wave_live || my_row >= count) return;
+  const float inv = 1.0f / l_run;
+  bf16_t* orow = out + (size_t)(t0 + my_row) * n_heads * HD + (size_t)head * HD;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int d = dt * 32 + g * 8 + half * 4;
+      uint2 pk;
+      pk.x = pack_bf16(o_acc[dt][g * 4 + 0] * inv, o_acc[dt][g * 4 + 1] * inv);
+      pk.y = pack_bf16(o_acc[dt][g * 4 + 2] * inv, o_acc[dt][g * 4 + 3] * inv);
+      *reinterpret_cast<uint2*>(orow + d) = pk;
+    }
+}
+
+// ============================================================================ decoding tokens
+// grid (tokens, kv heads, chunks): one wave per (token, kv head, chunk of 256 positions).  The
+// wave streams K rows and V^T rows of its chunk straight from the pages into 16x16x32 MFMA
+// operands; the query heads of the group are the 16 columns (a group of up to 16 heads).
+// Output: if the token's whole range is one chunk, the normalised result; else the chunk's
+// (max, sum, unnormalised output) into `partial`, folded by attention_combine_kernel.
+#define DC_CHUNK 256
+#define DC_BLOCK 64
+
+template <int HD>
+__global__ void __launch_bounds__(64)
+attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
+                        const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
+                        const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
+                        bf16_t* __restrict__ out, const int32_t* __restrict__ token_index, float* __restrict__ partial,
+                        int max_chunks, int n_heads, int n_kv_heads, int page_size, int window, float scale) {
+  constexpr int KS = HD / 32;   // k steps of S^T (32 dims each)
+  constexpr int DT = HD / 16;   // output tiles (16 dims each)
+  const int lane = threadIdx.x;
+  const int t = token_index[blockIdx.x];
+  const int kvh = blockIdx.y, chunk = blockIdx.z;
+  const int group = n_heads / n_kv_heads;
+  const int pos = positions[t];
+  const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int first = (lo / DC_BLOCK) * DC_BLOCK;
+  const int n_chunks = (pos - first) / DC_CHUNK + 1;
+  if (chunk >= n_chunks) return;
+  const int c0 = first + chunk * DC_CHUNK;
+  const int c1 = min(c0 + DC_CHUNK - 1, pos);        // last position of this chunk
+  const int32_t* table_row = block_table + (size_t)seq_rows[t] * table_stride;
+  const int r16 = lane & 15, q4 = lane >> 4;
+  const size_t kv_head_stride = (size_t)HD * page_size;
+
+  // Q^T (B operand): column = head of the group (zero beyond it), 8 consecutive dims
+  bf16x8 qf[KS];
+  {
+    const bf16_t* qrow = q + (size_t)t * q_stride + (size_t)(kvh * group + min(r16, group - 1)) * HD + q4 * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      uint4 v = *reinterpret_cast<const uint4*>(qrow + ks * 32);
+      if (r16 >= group) v = uint4{0, 0, 0, 0};
+      qf[ks] = frag_of(v);
+    }
+  }
+
+  f32x4 o_acc[DT];
+#pragma unroll
+  for (int i = 0; i < DT; ++i) o_acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  float m_run = -INFINITY, l_run = 0.0f;
+  const float c = scale * LOG2E;
+
+  for (int p0 = c0; p0 <= c1; p0 += DC_BLOCK) {
+    // S^T [64 positions][16 heads]: 4 tiles of 16 positions; A = K rows straight from the pages
+    f32x4 s_acc[4];
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt) {
+      s_acc[pt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      const int p = min(p0 + pt * 16 + r16, c1);   // rows past the chunk: any valid row, masked below
+      const bf16_t* krow = k_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * kv_head_stride +
+                           (size_t)(p % page_size) * HD + q4 * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        s_acc[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag_of(*reinterpret_cast<const uint4*>(krow + ks * 32)),
+                                                            qf[ks], s_acc[pt], 0, 0, 0);
+    }
+    // this lane: head r16; positions p0 + pt*16 + q4*4 + e
+    float mloc = -INFINITY;
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int p = p0 + pt * 16 + q4 * 4 + e;
+        const float v = (p <= c1 && p >= lo) ? s_acc[pt][e] * c : -INFINITY;
+        s_acc[pt][e] = v;
+        mloc = fmaxf(mloc, v);
+      }
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, AXON_WAVE));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, AXON_WAVE));
+    const float mn = fmaxf(m_run, mloc);
+    const float mref = mn == -INFINITY ? 0.0f : mn;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - mref);
+    float lsum = 0.0f;
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float pv = __builtin_amdgcn_exp2f(s_acc[pt][e] - mref);
+        s_acc[pt][e] = pv;
+        lsum += pv;
+      }
+    lsum += __shfl_xor(lsum, 16, AXON_WAVE);
+    lsum += __shfl_xor(lsum, 32, AXON_WAVE);
+    l_run = l_run * alpha + lsum;
+    m_run = mn;
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o_acc[i][e] *= alpha;
+
+    // O^T [HD][16 heads] += V^T P^T: k step u takes tiles 2u and 2u + 1: the lane's positions are
+    // p0 + 32u + 4 q4 + {0..3} and the same + 16: two 8-byte reads of V^T per output tile
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      union { uint32_t w[4]; bf16x8 f; } pf;
+      pf.w[0] = pack_bf16(s_acc[2 * u][0], s_acc[2 * u][1]);
+      pf.w[1] = pack_bf16(s_acc[2 * u][2], s_acc[2 * u][3]);
+      pf.w[2] = pack_bf16(s_acc[2 * u + 1][0], s_acc[2 * u + 1][1]);
+      pf.w[3] = pack_bf16(s_acc[2 * u + 1][2], s_acc[2 * u + 1][3]);
+      const int pa = p0 + 32 * u + 4 * q4, pb = pa + 16;
+      // positions past the chunk's end were never written: their weights are zero, and the
+      // values read for them are replaced by zero so that zero times anything stays zero
+      const bool ok_a = pa <= c1, ok_b = pb <= c1;
+      const int pa_c = min(pa, c1), pb_c = min(pb, c1);
+      const bf16_t* va = v_cache + ((size_t)table_row[pa_c / page_size] * n_kv_heads + kvh) * kv_head_stride +
+                         ((pa_c % page_size) & ~3);
+      const bf16_t* vb = v_cache + ((size_t)table_row[pb_c / page_size] * n_kv_heads + kvh) * kv_head_stride +
+                         ((pb_c % page_size) & ~3);
+      // within a group of 4 positions, those beyond c1 are cleared one by one
+      const int keep_a = ok_a ? min(c1 - pa + 1, 4) : 0, keep_b = ok_b ? min(c1 - pb + 1, 4) : 0;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const size_t doff = (size_t)(dt * 16 + r16) * page_size;
+        uint2 v0 = *reinterpret_cast<const uint2*>(va + doff);
+        uint2 v1 = *reinterpret_cast<const uint2*>(vb + doff);
+        if (keep_a < 4) {
+          if (keep_a < 1) v0.x = 0; else if (keep_a < 2) v0.x &= 0xffffu;
+          if (keep_a < 3) v0.y = 0; else v0.y &= 0xffffu;
+        }
+        if (keep_b < 4) {
+          if (keep_b < 1) v1.x = 0; else if (keep_b < 2) v1.x &= 0xffffu;
+          if (keep_b < 3) v1.y = 0; else v1.y &= 0xffffu;
+        }
+        o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag_of2(v0, v1), pf.f, o_acc[dt], 0, 0, 0);
+      }
+    }
+  }
+
+  if (r16 >= group) return;
+  const int head = kvh * group + r16;
+  if (n_chunks == 1) {
+    const float inv = 1.0f / l_run;
+    bf16_t* orow = out + (size_t)t * n_heads * HD + (size_t)head * HD;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint2 pk;
+      pk.x = pack_bf16(o_acc[dt][0] * inv, o_acc[dt][1] * inv);
+      pk.y = pack_bf16(o_acc[dt][2] * inv, o_acc[dt][3] * inv);
+      *reinterpret_cast<uint2*>(orow + dt * 16 + q4 * 4) = pk;
+    }
+  } else {
+    // partial [token slot][head][chunk][HD + 2]: output, then max (log2 domain) and sum
+    float* dst = partial + (((size_t)blockIdx.x * n_heads + head) * max_chunks + chunk) * (HD + 2);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      *reinterpret_cast<f32x4*>(dst + dt * 16 + q4 * 4) = o_acc[dt];
+    if (q4 == 0) {
+      dst[HD] = m_run;
+      dst[HD + 1] = l_run;
+    }
+  }
+}
+
+// Fold a token's chunks in ascending order: mn = max(M, m); O = O 2^(M - mn) + o 2^(m - mn);
+// L alike; out = O / L.  grid (tokens, heads), HD threads.
+template <int HD>
+__global__ void __launch_bounds__(HD)
+attention_combine_kernel(const float* __restrict__ partial, const int32_t* __restrict__ positions,
+                         const int32_t* __restrict__ token_index, bf16_t* __restrict__ out, int max_chunks, int n_heads,
+                         int window) {
+  const int t = token_index[blockIdx.x], head = blockIdx.y, d = threadIdx.x;
+  const int pos = positions[t];
+  const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int n_chunks = (pos - (lo / DC_BLOCK) * DC_BLOCK) / DC_CHUNK + 1;
+  if (n_chunks == 1) return;  // the decoding kernel wrote the result itself
+  const float* src = partial + ((size_t)blockIdx.x * n_heads + head) * max_chunks * (HD + 2);
+  float M = -INFINITY, L = 0.0f, O = 0.0f;
+  for (int cidx = 0; cidx < n_chunks; ++cidx) {
+    const float* p = src + (size_t)cidx * (HD + 2);
+    const float m = p[HD], l = p[HD + 1], o = p[d];
+    const float mn = fmaxf(M, m);
+    const float mref = mn == -INFINITY ? 0.0f : mn;
+    const float a = __builtin_amdgcn_exp2f(M - mref), w = __builtin_amdgcn_exp2f(m - mref);
+    L = fmaf(l, w, L * a);
+    O = fmaf(o, w, O * a);
+    M = mn;
+  }
+  out[(size_t)t * n_heads * HD + (size_t)head * HD + d] = float_to_bf16(O / L);
+}
+
+#endif  // AXON_BF16
+
+// ============================================================================ entry points
+// 1 if the MFMA attention kernels take this head size, page size and group of heads.
+extern "C" int axk_attention_fast_ok(int head_dim, int page_size, int n_heads, int n_kv_heads) {
+#if AXON_BF16
+  const bool hd_ok = head_dim == 64 || head_dim == 128;
+  const bool page_ok = page_size >= 8 && page_size <= 64 && (page_size & (page_size - 1)) == 0;
+  return hd_ok && page_ok && n_kv_heads > 0 && n_heads % n_kv_heads == 0 && n_heads / n_kv_heads <= 16;
+#else
+  return 0;
+#endif
+}
+
+extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                     const int32_t* block_table, int table_stride, const int32_t* positions,
+                                     const int32_t* seq_rows, void* out, const int32_t* tiles, int n_tiles, int n_heads,
+                                     int n_kv_heads, int head_dim, int page_size, int window, float scale, void* stream) {
+#if AXON_BF16
+  AXK_REQUIRE(axk_attention_fast_ok(head_dim, page_size, n_heads, n_kv_heads),
+              "attention_prefill: head_dim %d, page size %d, %d/%d heads are not taken by this kernel", head_dim,
+              page_size, n_heads, n_kv_heads);
+  AXK_REQUIRE(n_tiles >= 0 && n_heads <= 65535 && window >= 0 && q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0,
+              "attention_prefill: bad arguments (tiles %d, heads %d, window %d, q stride %d)", n_tiles, n_heads, window,
+              q_stride);
+  if (n_tiles == 0) return 0;
+  dim3 grid(n_tiles, n_heads);
+#define LAUNCH(HD)                                                                                                  \
+  {                                                                                                                 \
+    static bool configured = false;                                                                                 \
+    constexpr int lds = 2 * (PF_BLOCK * HD * 2 + HD * PF_BLOCK * 2);                                                \
+    if (!configured) {                                                                                              \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<HD>),              \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);                          \
+      if (e != hipSuccess) {                                                                                        \
+        axk_set_error("attention_prefill: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));          \
+        return -2;                                                                                                  \
+      }                                                                                                             \
+      configured = true;                                                                                            \
+    }                                                                                                               \
+    attention_prefill_kernel<HD><<<grid, 256, lds, (hipStream_t)stream>>>(                                          \
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,      \
+        positions, seq_rows, (bf16_t*)out, tiles, n_heads, n_kv_heads, page_size, window, scale);                   \
+  }
+  if (head_dim == 64) LAUNCH(64) else LAUNCH(128)
+#undef LAUNCH
+  AXK_LAUNCH_CHECK("attention_prefill");
+  return 0;
+#else
+  axk_set_error("attention_prefill: only in the bfloat16 build");
+  return -1;
+#endif
+}
+
+// Floats of `partial` that n_tokens decoding tokens with up to max_chunks chunks need.
+extern "C" long axk_attention_decode_workspace(int n_tokens, int n_heads, int head_dim, int max_chunks) {
+  return (long)n_tokens * n_heads * max_chunks * (head_dim + 2);
+}
+
+extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                    const int32_t* block_table, int table_stride, const int32_t* positions,
+                                    const int32_t* seq_rows, void* out, const int32_t* token_index, int n_tokens,
+                                    float* partial, int max_chunks, int n_heads, int n_kv_heads, int head_dim,
+                                    int page_size, int window, float scale, void* stream) {
+#if AXON_BF16
+  AXK_REQUIRE(axk_attention_fast_ok(head_dim, page_size, n_heads, n_kv_heads),
+              "attention_decode: head_dim %d, page size %d, %d/%d heads are not taken by this kernel", head_dim,
+              page_size, n_heads, n_kv_heads);
+  AXK_REQUIRE(n_tokens >= 0 && max_chunks >= 1 && max_chunks <= 65535 && n_kv_heads <= 65535 && window >= 0 &&
+                  q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0,
+              "attention_decode: bad arguments (tokens %d, chunks %d, window %d, q stride %d)", n_tokens, max_chunks,
+              window, q_stride);
+  AXK_REQUIRE(max_chunks == 1 || partial != nullptr, "attention_decode: %d chunks need a workspace", max_chunks);
+  if (n_tokens == 0) return 0;
+  dim3 grid(n_tokens, n_kv_heads, max_chunks), cgrid(n_tokens, n_heads);
+#define LAUNCH(HD)                                                                                                   \
+  {                                                                                                                  \
+    attention_decode_kernel<HD><<<grid, 64, 0, (hipStream_t)stream>>>(                                               \
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,       \
+        positions, seq_rows, (bf16_t*)out, token_index, partial, max_chunks, n_heads, n_kv_heads, page_size, window, \
+        scale);                                                                                                      \
+    if (max_chunks > 1)                                                                                              \
+      attention_combine_kernel<HD><<<cgrid, HD, 0, (hipStream_t)stream>>>(partial, positions, token_index,          \
+                                                                         (bf16_t*)out, max_chunks, n_heads, window); \
+  }
+  if (head_dim == 64) LAUNCH(64) else LAUNCH(128)
+#undef LAUNCH
+  AXK_LAUNCH_CHECK("attention_decode");
+  return 0;
+#else
+  axk_set_error("attention_decode: only in the bfloat16 build");
+  return -1;
+#endif
+}

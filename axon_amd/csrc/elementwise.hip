@@ -110,9 +110,10 @@ extern "C" int axk_rope_table(const int32_t* positions, const double* freqs, flo
 
 // ---------------------------------------------------------------------------- rotary + cache store
 // One block per (token, head slot): q heads are rotated in place, k heads rotated and stored
-// in the request's page for that position, v heads stored as they are.  Pair i of a head is
-// (i, i + rotary_dim / 2): out_i = a cos - b sin, out_{i+half} = a sin + b cos, each product
-// and sum rounded on its own (src/model.rs:3922-3929; src/cuda/prefill.cu:129-160).
+// in the request's page for that position, v heads stored as they are (transposed: a page of
+// values is [dim][slot], so that the positions of one dim are contiguous).  Pair i of a head
+// is (i, i + rotary_dim / 2): out_i = a cos - b sin, out_{i+half} = a sin + b cos, each
+// product and sum rounded on its own (src/model.rs:3922-3929; src/cuda/prefill.cu:129-160).
 __global__ void rope_kv_write_kernel(elem_t* __restrict__ qkv, const float* __restrict__ table,
                                      const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
                                      const int32_t* __restrict__ block_table, int table_stride,
@@ -126,7 +127,6 @@ __global__ void rope_kv_write_kernel(elem_t* __restrict__ qkv, const float* __re
   const float* tab = table + (size_t)t * half * 2;
 
   elem_t* dst = src;
-  bool rotate = true;
   if (slot >= n_heads) {
     if (!write_kv) return;
     const int pos = positions[t];
@@ -134,24 +134,24 @@ __global__ void rope_kv_write_kernel(elem_t* __restrict__ qkv, const float* __re
     const int in_page = pos % page_size;
     const bool is_v = slot >= n_heads + n_kv_heads;
     const int kvh = slot - n_heads - (is_v ? n_kv_heads : 0);
-    elem_t* base = is_v ? v_cache : k_cache;
-    dst = base + (((size_t)page * n_kv_heads + kvh) * page_size + in_page) * head_dim;
-    rotate = !is_v;
-  }
-  if (rotate) {
-    for (int i = threadIdx.x; i < half; i += blockDim.x) {
-      const float s = tab[2 * i], c = tab[2 * i + 1];
-      const float a = to_float(src[i]), b = to_float(src[i + half]);
-      const float lo = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s));
-      const float hi = __fadd_rn(__fmul_rn(a, s), __fmul_rn(b, c));
-      dst[i] = from_float(lo);
-      dst[i + half] = from_float(hi);
+    if (is_v) {
+      // values are kept position-contiguous: [page][kv head][dim][slot in page]
+      elem_t* vdst = v_cache + ((size_t)page * n_kv_heads + kvh) * head_dim * page_size + in_page;
+      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) vdst[(size_t)i * page_size] = src[i];
+      return;
     }
-    if (dst != src)
-      for (int i = rotary_dim + threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
-  } else {
-    for (int i = threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
+    dst = k_cache + (((size_t)page * n_kv_heads + kvh) * page_size + in_page) * head_dim;
   }
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float s = tab[2 * i], c = tab[2 * i + 1];
+    const float a = to_float(src[i]), b = to_float(src[i + half]);
+    const float lo = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s));
+    const float hi = __fadd_rn(__fmul_rn(a, s), __fmul_rn(b, c));
+    dst[i] = from_float(lo);
+    dst[i + half] = from_float(hi);
+  }
+  if (dst != src)
+    for (int i = rotary_dim + threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
 }
 
 extern "C" int axk_rope_kv_write(void* qkv, const float* table, const int32_t* positions, const int32_t* seq_rows,

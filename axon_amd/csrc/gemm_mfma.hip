@@ -1,11 +1,364 @@
-// bfloat16 matrix products on the matrix cores (MFMA).  Only in the bfloat16 build.
+// bfloat16 matrix products on the matrix cores: out = X [M, K] . W [N, K]^T, both operands
+// K-major, 32-bit accumulation.  Only in the bfloat16 build.
+//
+// Two kernels, chosen by M alone so that a given (N, K) always meets the same pair:
+//
+// * gemm_tile (M > 64): a block of 4 or 8 waves owns a BM x BN tile of the output (256 x 256,
+//   or 128 x 128 when that would leave CUs without work), walks K in steps of 64 through two
+//   LDS stages filled by direct global -> LDS loads (the next step's loads in flight while
+//   this one multiplies), and each wave keeps a tile of 32x32x16 MFMA accumulators.  The
+//   16-byte slots of an LDS row are permuted so that fragment reads of neighbouring rows fall
+//   into different banks.  Blocks are numbered so that the blocks of one XCD (every eighth
+//   block) share weight tiles in that XCD's L2.
+//
+// * gemm_skinny (M <= 64, decoding): bound by reading W once.  A wave owns 16 or 32 rows of
+//   W, streams them from memory straight into MFMA fragments (16x16x32: a lane's 8
+//   consecutive k are one 16-byte load), multiplies with up to 64 rows of X, and the waves
+//   of a block split K between them; their partial sums are added in wave order through LDS.
+//   No atomics, so the result does not depend on timing.
+//
+// The two kernels sum k in different groupings, so a row's bits differ between M <= 64 and
+// M > 64 by rounding (and only by rounding); within one kernel a row does not depend on the
+// other rows of the batch.
+#include <stdlib.h>
+
 #include "api.h"
 #include "common.h"
 
 #if AXON_BF16
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+enum { MODE_STORE = 0, MODE_ADD_F32 = 1, MODE_STORE_F32 = 2 };
+
+#define TILE_BK 64
+#define TILE_ROW_BYTES 128  // one LDS row: 64 bf16, in eight 16-byte slots
+
+__device__ inline bf16x8 as_frag(uint4 v) {
+  union { uint4 u; bf16x8 f; } c;
+  c.u = v;
+  return c.f;
+}
+
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// ---------------------------------------------------------------------------- gemm_tile
+// LDS holds, per stage, BM rows of X and BN rows of W, 64 k each, written by direct
+// global -> LDS loads of 16 bytes per lane (a wave instruction fills 8 rows).  Within a row
+// the eight 16-byte slots are permuted: slot p of row r holds k chunk p ^ (r & 7), so that the
+// fragment reads of 8 neighbouring rows at one k chunk hit 8 different slots (no bank
+// conflicts) without padding, which direct loads could not skip.
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const void* __restrict__ bias,
+                 int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode, int m_blocks,
+                 int n_blocks) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // a wave's tile
+  constexpr int TM = WM / 32, TN = WN / 32;            // in 32 x 32 MFMA tiles
+  constexpr int XQ = BM / 8 / NW, WQ = BN / 8 / NW;    // load instructions per wave and stage
+  constexpr int STAGE = (BM + BN) * TILE_ROW_BYTES;    // bytes per stage
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  // Block numbering: every eighth block runs on the same XCD; give one XCD consecutive m
+  // blocks of the same n block, so a weight tile is fetched into one L2 and reused there.
+  const int bid = blockIdx.x;
+  int mb, nb;
+  if (bid < (n_blocks / 8) * 8 * m_blocks) {
+    const int xcd = bid & 7, j = bid >> 3;
+    nb = (j / m_blocks) * 8 + xcd;
+    mb = j % m_blocks;
+  } else {  // the last, incomplete group of n blocks: plain order
+    const int r = bid - (n_blocks / 8) * 8 * m_blocks;
+    nb = (n_blocks / 8) * 8 + r / m_blocks;
+    mb = r % m_blocks;
+  }
+  const int m0 = mb * BM, n0 = nb * BN;
+
+  // what this lane fetches: row (q * NW + wave) * 8 + lane / 8 of a tile, k chunk (lane % 8) ^ (lane / 8)
+  const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
+  unsigned xoff[XQ], woff[WQ];
+#pragma unroll
+  for (int q = 0; q < XQ; ++q)
+    xoff[q] = (unsigned)min(m0 + (q * NW + wave) * 8 + lrow, M - 1) * (unsigned)x_stride + lchunk * 8;
+#pragma unroll
+  for (int q = 0; q < WQ; ++q)
+    woff[q] = (unsigned)min(n0 + (q * NW + wave) * 8 + lrow, N - 1) * (unsigned)K + lchunk * 8;
+
+  auto issue = [&](int kt) {
+    unsigned char* stage = smem + (kt & 1) * STAGE;
+    const int koff = kt * TILE_BK;
+#pragma unroll
+    for (int q = 0; q < XQ; ++q)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(x + xoff[q] + koff),
+                                       (lds_ptr_t)(stage + (q * NW + wave) * 8 * TILE_ROW_BYTES), 16, 0, 0);
+#pragma unroll
+    for (int q = 0; q < WQ; ++q)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(w + woff[q] + koff),
+                                       (lds_ptr_t)(stage + (BM + (q * NW + wave) * 8) * TILE_ROW_BYTES), 16, 0, 0);
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  // fragment addresses: row = tile row + lane % 32, k chunk = 2 ks + lane / 32, slot = chunk ^ (row & 7)
+  const int frow = lane & 31, fhalf = lane >> 5, fsw = lane & 7;
+  const int xbase = (wm * WM + frow) * TILE_ROW_BYTES;
+  const int wbase = (BM + wn * WN + frow) * TILE_ROW_BYTES;
+
+  const int nk = K / TILE_BK;
+  issue(0);
+  for (int kt = 0; kt < nk; ++kt) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // tile kt is in LDS for every wave, and every wave is done with tile kt - 1
+    if (kt + 1 < nk) issue(kt + 1);
+    const unsigned char* stage = smem + (kt & 1) * STAGE;
+    bf16x8 a[2][TM], b[2][TN];
+    {
+      const int slot = ((0 + fhalf) ^ fsw) << 4;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        a[0][i] = as_frag(*reinterpret_cast<const uint4*>(stage + xbase + i * 32 * TILE_ROW_BYTES + slot));
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        b[0][j] = as_frag(*reinterpret_cast<const uint4*>(stage + wbase + j * 32 * TILE_ROW_BYTES + slot));
+    }
+#pragma unroll
+    for (int ks = 0; ks < TILE_BK / 16; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < TILE_BK / 16) {
+        const int slot = (((ks + 1) * 2 + fhalf) ^ fsw) << 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          a[nxt][i] = as_frag(*reinterpret_cast<const uint4*>(stage + xbase + i * 32 * TILE_ROW_BYTES + slot));
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          b[nxt][j] = as_frag(*reinterpret_cast<const uint4*>(stage + wbase + j * 32 * TILE_ROW_BYTES + slot));
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
+      // ask the scheduler to spread the next step's fragment reads between this step's MFMAs
+      if (ks + 1 < TILE_BK / 16) {
+#pragma unroll
+        for (int r = 0; r < TM + TN; ++r) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                         // one LDS read
+          __builtin_amdgcn_sched_group_barrier(0x008, (TM * TN) / (TM + TN), 0);     // a share of the MFMAs
+        }
+      }
+    }
+  }
+
+  // epilogue: lane holds column n = lane % 32 of each tile and rows (e/4)*8 + (lane/32)*4 + e%4
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn * WN + j * 32 + (lane & 31);
+    if (n >= N) continue;
+    const float bv = bias ? load_vec(bias, bias_is_f32, n) : 0.0f;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int m = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        if (m >= M) continue;
+        const float v = acc[i][j][e] + bv;
+        const size_t at = (size_t)m * out_stride + n;
+        if (mode == MODE_STORE) reinterpret_cast<bf16_t*>(out)[at] = float_to_bf16(v);
+        else if (mode == MODE_ADD_F32) reinterpret_cast<float*>(out)[at] += v;
+        else reinterpret_cast<float*>(out)[at] = v;
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                       int out_stride, int m, int n, int k, int mode, hipStream_t stream) {
+  static bool configured = false;
+  constexpr int lds_bytes = 2 * (BM + BN) * TILE_ROW_BYTES;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) {
+      axk_set_error("gemm_tile: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+      return -2;
+    }
+    configured = true;
+  }
+  const int m_blocks = ceil_div(m, BM), n_blocks = ceil_div(n, BN);
+  gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N><<<m_blocks * n_blocks, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks);
+  AXK_LAUNCH_CHECK("gemm_tile");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------- gemm_skinny
+// A block of WAVES waves owns NT16 * 16 rows of W; wave v takes the k steps (of 64) v, v + WAVES,
+// ...  C[n][m] tiles of 16 x 16: the MFMA's A operand is W (lane: row n = lane % 16, 8
+// consecutive k from (lane / 16) * 8), its B operand X (lane: row m = lane % 16, the same k).
+// A lane ends with 4 consecutive n of one m: one vector store.
+template <int NT16, int MT16, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w,
+                   const void* __restrict__ bias, int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N,
+                   int K, int mode) {
+  __shared__ float partial[WAVES][NT16 * MT16][64][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * NT16 * 16;
+  const int r16 = lane & 15, kq = (lane >> 4) * 8;
+
+  const bf16_t* wrow[NT16];
+#pragma unroll
+  for (int i = 0; i < NT16; ++i) wrow[i] = w + (size_t)min(n0 + i * 16 + r16, N - 1) * K + kq;
+  const bf16_t* xrow[MT16];
+#pragma unroll
+  for (int j = 0; j < MT16; ++j) xrow[j] = x + (size_t)min(j * 16 + r16, M - 1) * x_stride + kq;
+
+  f32x4 acc[NT16][MT16];
+#pragma unroll
+  for (int i = 0; i < NT16; ++i)
+#pragma unroll
+    for (int j = 0; j < MT16; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  const int steps = K / 64;
+  constexpr int UNROLL = 4;
+  int s = wave;
+  for (; s + (UNROLL - 1) * WAVES < steps; s += UNROLL * WAVES) {
+    uint4 wf[UNROLL][NT16][2], xf[UNROLL][MT16][2];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int k0 = (s + u * WAVES) * 64;
+#pragma unroll
+      for (int i = 0; i < NT16; ++i) {
+        wf[u][i][0] = *reinterpret_cast<const uint4*>(wrow[i] + k0);
+        wf[u][i][1] = *reinterpret_cast<const uint4*>(wrow[i] + k0 + 32);
+      }
+#pragma unroll
+      for (int j = 0; j < MT16; ++j) {
+        xf[u][j][0] = *reinterpret_cast<const uint4*>(xrow[j] + k0);
+        xf[u][j][1] = *reinterpret_cast<const uint4*>(xrow[j] + k0 + 32);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int i = 0; i < NT16; ++i)
+#pragma unroll
+          for (int j = 0; j < MT16; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[u][i][h]), as_frag(xf[u][j][h]), acc[i][j], 0, 0, 0);
+  }
+  for (; s < steps; s += WAVES) {
+    const int k0 = s * 64;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint4 wf[NT16], xf[MT16];
+#pragma unroll
+      for (int i = 0; i < NT16; ++i) wf[i] = *reinterpret_cast<const uint4*>(wrow[i] + k0 + h * 32);
+#pragma unroll
+      for (int j = 0; j < MT16; ++j) xf[j] = *reinterpret_cast<const uint4*>(xrow[j] + k0 + h * 32);
+#pragma unroll
+      for (int i = 0; i < NT16; ++i)
+#pragma unroll
+        for (int j = 0; j < MT16; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[i]), as_frag(xf[j]), acc[i][j], 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < NT16; ++i)
+#pragma unroll
+    for (int j = 0; j < MT16; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) partial[wave][i * MT16 + j][lane][e] = acc[i][j][e];
+  __syncthreads();
+
+  // tiles are shared out between the waves; each sums the partials in wave order
+  for (int t = wave; t < NT16 * MT16; t += WAVES) {
+    const int i = t / MT16, j = t % MT16;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float sum = partial[0][t][lane][e];
+#pragma unroll
+      for (int q = 1; q < WAVES; ++q) sum += partial[q][t][lane][e];
+      v[e] = sum;
+    }
+    const int m = j * 16 + r16;
+    const int n = n0 + i * 16 + (lane >> 4) * 4;
+    if (m >= M) continue;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (n + e >= N) continue;
+      float r = v[e];
+      if (bias) r += load_vec(bias, bias_is_f32, n + e);
+      const size_t at = (size_t)m * out_stride + n + e;
+      if (mode == MODE_STORE) reinterpret_cast<bf16_t*>(out)[at] = float_to_bf16(r);
+      else if (mode == MODE_ADD_F32) reinterpret_cast<float*>(out)[at] += r;
+      else reinterpret_cast<float*>(out)[at] = r;
+    }
+  }
+}
+
+template <int NT16, int MT16, int WAVES>
+static int launch_skinny(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                         int out_stride, int m, int n, int k, int mode, hipStream_t stream) {
+  gemm_skinny_kernel<NT16, MT16, WAVES><<<ceil_div(n, NT16 * 16), WAVES * 64, 0, stream>>>(
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode);
+  AXK_LAUNCH_CHECK("gemm_skinny");
+  return 0;
+}
+
+// Shapes the MFMA kernels take: K a multiple of 64 and 16-byte aligned rows.  Decided by (N, K)
+// and the pointers' alignment, never by M, so a weight matrix always meets the same kernels.
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                      int out_stride, int m, int n, int k, int mode, hipStream_t stream, bool* handled) {
   *handled = false;
-  return 0;
+  if (k % 64 != 0 || x_stride % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return 0;
+  *handled = true;
+#define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream
+  if (m <= 64) {
+    // wide outputs: 32 rows of W per wave and 4 waves; narrow ones: 16 rows and 8 waves, so that
+    // enough waves stream the weights
+    const bool wide = n >= 16384;
+    if (m <= 16) return wide ? launch_skinny<2, 1, 4>(ARGS) : launch_skinny<1, 1, 8>(ARGS);
+    if (m <= 32) return wide ? launch_skinny<2, 2, 4>(ARGS) : launch_skinny<1, 2, 8>(ARGS);
+    return wide ? launch_skinny<2, 4, 4>(ARGS) : launch_skinny<1, 4, 8>(ARGS);
+  }
+  // offsets inside the kernels are 32-bit element counts
+  if ((size_t)n * k >= (1ull << 32) || (size_t)m * x_stride >= (1ull << 32)) {
+    *handled = false;
+    return 0;
+  }
+  static const int forced = getenv("AXON_GEMM_TILE") ? atoi(getenv("AXON_GEMM_TILE")) : 0;
+  switch (forced) {
+    case 1: return launch_tile<256, 256, 2, 2>(ARGS);
+    case 2: return launch_tile<256, 256, 2, 4>(ARGS);
+    case 3: return launch_tile<128, 256, 2, 2>(ARGS);
+    case 4: return launch_tile<128, 128, 2, 2>(ARGS);
+    case 5: return launch_tile<256, 256, 4, 2>(ARGS);
+    case 6: return launch_tile<256, 128, 2, 2>(ARGS);
+    case 7: return launch_tile<128, 256, 1, 4>(ARGS);
+    default: break;
+  }
+  // 256 x 256 tiles (8 waves) when they still give every CU two blocks; else 128 x 128
+  if ((long)ceil_div(m, 256) * ceil_div(n, 256) >= 512) return launch_tile<256, 256, 4, 2>(ARGS);
+  return launch_tile<128, 128, 2, 2>(ARGS);
+#undef ARGS
 }
-#endif
+
+#endif  // AXON_BF16

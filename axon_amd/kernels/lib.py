@@ -38,6 +38,11 @@ _SIGNATURES = {
                           c_int, c_int, c_int, c_int, c_int, c_void_p],
     "axk_attention": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
                       c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "axk_attention_prefill": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                              c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "axk_attention_decode": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                             c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "axk_attention_fast_ok": [c_int, c_int, c_int, c_int],
     "axk_gemm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "axk_swiglu": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_argmax": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
@@ -61,6 +66,8 @@ class Kernels:
             fn = getattr(self.lib, name)
             fn.argtypes = args
             fn.restype = c_int
+        self.lib.axk_attention_decode_workspace.argtypes = [c_int, c_int, c_int, c_int]
+        self.lib.axk_attention_decode_workspace.restype = ctypes.c_long
         if bool(self.lib.axk_is_bf16()) != (dtype_name == "bfloat16"):
             raise KernelError(f"{self.path} was not built for {dtype_name}")
 
@@ -90,6 +97,17 @@ class Kernels:
         if v.dtype not in (torch.float32, torch.bfloat16) or not v.is_cuda or not v.is_contiguous():
             raise KernelError(f"{what}: a vector must be float32 or bfloat16 on the device, got {v.dtype}")
         return 1 if v.dtype == torch.float32 else 0
+
+    def _check_caches(self, k_cache, v_cache, n_kv_heads, page_size, head_dim) -> None:
+        """Keys are [pages, kv heads, page_size, head_dim]; values are kept position-contiguous:
+        [pages, kv heads, head_dim, page_size]."""
+        self._elem(k_cache, "k cache"); self._elem(v_cache, "v cache")
+        if (k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (n_kv_heads, page_size, head_dim)
+                or not k_cache.is_contiguous()):
+            raise KernelError(f"key cache {tuple(k_cache.shape)} is not [pages, {n_kv_heads}, {page_size}, {head_dim}]")
+        if (v_cache.dim() != 4 or tuple(v_cache.shape[1:]) != (n_kv_heads, head_dim, page_size)
+                or not v_cache.is_contiguous() or v_cache.shape[0] != k_cache.shape[0]):
+            raise KernelError(f"value cache {tuple(v_cache.shape)} is not [pages, {n_kv_heads}, {head_dim}, {page_size}]")
 
     # ------------------------------------------------------------------ ops
     def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -138,10 +156,7 @@ class Kernels:
         if table.shape != (T, rotary_dim // 2, 2):
             raise KernelError(f"rope_kv_write: table {tuple(table.shape)} for rotary_dim {rotary_dim}")
         if write_kv:
-            self._elem(k_cache, "k cache"); self._elem(v_cache, "v cache")
-            for c in (k_cache, v_cache):
-                if c.dim() != 4 or tuple(c.shape[1:]) != (n_kv_heads, page_size, head_dim) or not c.is_contiguous():
-                    raise KernelError(f"rope_kv_write: cache {tuple(c.shape)} is not [pages, {n_kv_heads}, {page_size}, {head_dim}]")
+            self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
         self._check(self.lib.axk_rope_kv_write(
             _ptr(qkv), _ptr(table), _ptr(positions), _ptr(seq_rows), _ptr(block_table), block_table.shape[-1],
             _ptr(k_cache if write_kv else None), _ptr(v_cache if write_kv else None), T, n_heads, n_kv_heads, head_dim,
@@ -155,12 +170,52 @@ class Kernels:
         T = positions.numel()
         if out.shape != (T, n_heads * head_dim) or not out.is_contiguous():
             raise KernelError(f"attention: out {tuple(out.shape)} is not [{T}, {n_heads * head_dim}]")
-        for c in (k_cache, v_cache):
-            if c.dim() != 4 or tuple(c.shape[1:]) != (n_kv_heads, page_size, head_dim) or not c.is_contiguous():
-                raise KernelError(f"attention: cache {tuple(c.shape)} is not [pages, {n_kv_heads}, {page_size}, {head_dim}]")
+        self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
         self._check(self.lib.axk_attention(
             _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[-1], _ptr(positions),
             _ptr(seq_rows), _ptr(out), T, n_heads, n_kv_heads, head_dim, page_size, window, float(scale), _stream()))
+        return out
+
+    def attention_fast_ok(self, head_dim: int, page_size: int, n_heads: int, n_kv_heads: int) -> bool:
+        """Whether the matrix-core attention kernels take these sizes (never in float32)."""
+        return bool(self.lib.axk_attention_fast_ok(head_dim, page_size, n_heads, n_kv_heads))
+
+    def attention_prefill(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, tiles, n_heads,
+                          n_kv_heads, head_dim, page_size, window, scale) -> torch.Tensor:
+        """Attention of prompt portions: tiles [n, 2] int32 = (first token, count <= 128)."""
+        self._elem(q, "attention q"); self._elem(out, "attention out")
+        self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
+        self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
+        self._i32(tiles, "tiles")
+        if out.shape[1] != n_heads * head_dim or not out.is_contiguous() or tiles.dim() != 2 or tiles.shape[1] != 2:
+            raise KernelError(f"attention_prefill: out {tuple(out.shape)}, tiles {tuple(tiles.shape)}")
+        self._check(self.lib.axk_attention_prefill(
+            _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[-1], _ptr(positions),
+            _ptr(seq_rows), _ptr(out), _ptr(tiles), tiles.shape[0], n_heads, n_kv_heads, head_dim, page_size, window,
+            float(scale), _stream()))
+        return out
+
+    def attention_decode_workspace(self, n_tokens: int, n_heads: int, head_dim: int, max_chunks: int) -> int:
+        return int(self.lib.axk_attention_decode_workspace(n_tokens, n_heads, head_dim, max_chunks))
+
+    def attention_decode(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, token_index,
+                         partial, max_chunks, n_heads, n_kv_heads, head_dim, page_size, window, scale) -> torch.Tensor:
+        """Attention of single decoding tokens named by token_index (int32)."""
+        self._elem(q, "attention q"); self._elem(out, "attention out")
+        self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
+        self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
+        self._i32(token_index, "token_index")
+        n = token_index.numel()
+        if out.shape[1] != n_heads * head_dim or not out.is_contiguous():
+            raise KernelError(f"attention_decode: out {tuple(out.shape)}")
+        if max_chunks > 1:
+            self._f32(partial, "attention partial")
+            if partial.numel() < self.attention_decode_workspace(n, n_heads, head_dim, max_chunks):
+                raise KernelError(f"attention_decode: workspace of {partial.numel()} floats is too small")
+        self._check(self.lib.axk_attention_decode(
+            _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[-1], _ptr(positions),
+            _ptr(seq_rows), _ptr(out), _ptr(token_index), n, _ptr(partial if max_chunks > 1 else None), max_chunks,
+            n_heads, n_kv_heads, head_dim, page_size, window, float(scale), _stream()))
         return out
 
     def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,

@@ -24,6 +24,49 @@ from ..kernels import MODE_ADD_F32, MODE_STORE
 from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, build_part, register_mixer
 
 
+PREFILL_TILE = 128     # tokens of one request per tile of the prompt kernel
+DECODE_CHUNK = 256     # positions per chunk of the decoding kernel
+DECODE_BLOCK = 64
+
+
+class AttentionPlan:
+    """How the matrix-core kernels split a step: prompt portions (2 tokens or more) go to the
+    prompt kernel in tiles of up to 128 tokens, single tokens to the decoding kernel.  Made
+    once per step and window, shared by all layers."""
+
+    def __init__(self, ctx, window: int, n_heads: int, head_dim: int):
+        tiles, singles, chunks = [], [], 1
+        for s in ctx.spans:
+            if s.q_len == 1:
+                singles.append(s.q_start)
+                pos = s.start_pos
+                lo = max(0, pos + 1 - window) if window > 0 else 0
+                first = lo // DECODE_BLOCK * DECODE_BLOCK
+                chunks = max(chunks, (pos - first) // DECODE_CHUNK + 1)
+            else:
+                for at in range(0, s.q_len, PREFILL_TILE):
+                    tiles.append((s.q_start + at, min(PREFILL_TILE, s.q_len - at)))
+        # the kernels trust these indices: check them here, on the host
+        if any(a < 0 or n < 1 or a + n > ctx.n_tokens for a, n in tiles) or any(not 0 <= t < ctx.n_tokens for t in singles):
+            raise ValueError("attention plan: a span lies outside the tokens of the step")
+        dev = ctx.rt.device
+        self.tiles = torch.tensor(tiles, dtype=torch.int32).to(dev) if tiles else None
+        self.decode_tokens = torch.tensor(singles, dtype=torch.int32).to(dev) if singles else None
+        self.max_chunks = chunks
+        self.partial = None
+        if singles and chunks > 1:
+            n = ctx.rt.k.attention_decode_workspace(len(singles), n_heads, head_dim, chunks)
+            self.partial = torch.empty(n, dtype=torch.float32, device=dev)
+
+
+def attention_plan(ctx, window: int, n_heads: int, head_dim: int) -> AttentionPlan:
+    key = ("attention_plan", window, n_heads, head_dim)
+    plan = ctx.shared.get(key)
+    if plan is None:
+        plan = ctx.shared[key] = AttentionPlan(ctx, window, n_heads, head_dim)
+    return plan
+
+
 class GQAttention(Mixer):
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
@@ -85,6 +128,8 @@ class GQAttention(Mixer):
         T = h.shape[0]
         group = ctx.cache.group(binding.group)
         k_cache, v_cache = group.layer(binding.index)
+        # values are kept position-contiguous: a page of them is [heads, head_dim, page_size]
+        v_cache = v_cache.view(v_cache.shape[0], self.nkv, self.hd, group.page_size)
         mark = ctx.ws.mark()
         if binding.writes:
             qkv = ctx.ws.take((T, self.q_dim + 2 * self.kv_dim), ctx.rt.dtype)
@@ -101,8 +146,17 @@ class GQAttention(Mixer):
         k.rope_kv_write(qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache, self.nh, self.nkv,
                         self.hd, rotary, group.page_size, binding.writes)
         att = ctx.ws.take((T, self.q_dim), ctx.rt.dtype)
-        k.attention(qkv, qkv.stride(0), k_cache, v_cache, group.block_table, ctx.positions, ctx.seq_rows, att, self.nh,
-                    self.nkv, self.hd, group.page_size, self.window, self.scale)
+        if k.attention_fast_ok(self.hd, group.page_size, self.nh, self.nkv):
+            plan = attention_plan(ctx, self.window, self.nh, self.hd)
+            common = (k_cache, v_cache, group.block_table, ctx.positions, ctx.seq_rows, att)
+            sizes = (self.nh, self.nkv, self.hd, group.page_size, self.window, self.scale)
+            if plan.tiles is not None:
+                k.attention_prefill(qkv, qkv.stride(0), *common, plan.tiles, *sizes)
+            if plan.decode_tokens is not None:
+                k.attention_decode(qkv, qkv.stride(0), *common, plan.decode_tokens, plan.partial, plan.max_chunks, *sizes)
+        else:
+            k.attention(qkv, qkv.stride(0), k_cache, v_cache, group.block_table, ctx.positions, ctx.seq_rows, att,
+                        self.nh, self.nkv, self.hd, group.page_size, self.window, self.scale)
         k.gemm(att, self.w_o, residual, self.b_o, MODE_ADD_F32)
         ctx.ws.release(mark)
 

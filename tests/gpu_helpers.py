@@ -15,7 +15,8 @@ def tol(dtype, ref, f32=2e-5, bf16=2e-2):
 
 def paged_cache(k, v, page_size, dtype, n_extra_pages=3, seed=0, fill=None):
     """Scatter k, v [T, nkv, hd] of ONE request into shuffled pages.  Returns
-    (k_cache, v_cache, block_table [1, pages]); unused rows hold `fill` (NaN by default, so a
+    (k_cache [pages, nkv, page, hd], v_cache [pages, nkv, hd, page], block_table [1, pages]);
+    unused rows hold `fill` (NaN by default, so a
     kernel that reads past what it may is caught)."""
     T, nkv, hd = k.shape
     n_logical = -(-T // page_size)
@@ -30,6 +31,7 @@ def paged_cache(k, v, page_size, dtype, n_extra_pages=3, seed=0, fill=None):
         kc[p, :, o] = k[t].float()
         vc[p, :, o] = v[t].float()
     dt = TORCH[dtype]
+    vc = vc.permute(0, 1, 3, 2).contiguous()          # values: [pages, heads, head_dim, page_size]
     return kc.to(dt).cuda(), vc.to(dt).cuda(), perm.to(torch.int32)[None, :].contiguous().cuda()
 
 

@@ -16,12 +16,12 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "E"])
 def test_greedy_generation_matches_the_plain_loop(name, dtype, model_dirs):
     d = model_dirs(name, "float32" if dtype == "float32" else "bfloat16")
     cfg, w = P.load_plain(d)
-    prompts = prompts_for(name, [1, 5, 17, 33] if name == "A" else [2, 9, 70, 41, 3, 25], seed=1)
-    n_new = 16 if name == "A" else 24
+    prompts = prompts_for(name, {"A": [1, 5, 17, 33], "B": [2, 9, 70, 41, 3, 25], "E": [3, 140, 66]}[name], seed=1)
+    n_new = {"A": 16, "B": 24, "E": 12}[name]
     llm = axon_amd.load(d, dtype=dtype, page_size=TINY[name]["page_size"], num_pages=64, max_seqs=4, max_batch_tokens=48)
     outs = llm.generate(prompts, max_new_tokens=n_new)
     for p, o in zip(prompts, outs):

@@ -75,7 +75,7 @@ def test_rope_and_cache_store(dtype, nh, nkv, hd, page):
     n_pages = 9
     table = torch.tensor([[7, 2, 5, 0, 3, 1, 8, 4]], dtype=torch.int32)       # scattered pages
     kc = torch.zeros(n_pages, nkv, page, hd, dtype=TORCH[dtype], device="cuda")
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(n_pages, nkv, hd, page, dtype=TORCH[dtype], device="cuda")
     freqs = P.rope_freqs(hd, 1e4)
     tab = torch.empty(T, hd // 2, 2, dtype=torch.float32, device="cuda")
     k.rope_table(pos.cuda(), freqs.cuda(), tab)
@@ -89,9 +89,9 @@ def test_rope_and_cache_store(dtype, nh, nkv, hd, page):
     for i, p in enumerate(pos.tolist()):
         pg, o = int(table[0, p // page]), p % page
         assert (kc[pg, :, o].cpu().double() - k_ref[i]).abs().max() <= t
-        assert torch.equal(vc[pg, :, o].cpu().double(), v_ref[i])              # values are stored as they are
+        assert torch.equal(vc[pg, :, :, o].cpu().double(), v_ref[i])           # values are stored as they are
     written = sum(1 for _ in pos)
-    assert int((vc.abs().sum(dim=(1, 3)) > 0).sum()) == written                # nothing else was touched
+    assert int((vc.abs().sum(dim=(1, 2)) > 0).sum()) == written                # nothing else was touched
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -182,17 +182,23 @@ def test_gemm_every_epilogue(dtype, M, N, K):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_rows_do_not_depend_on_the_batch(dtype):
-    """The same row of x gives the same bits whatever rows ride along (1, 3, 16, 17, 64, 200)."""
+    """The same row of x gives the same bits whatever rows ride along.  float32: for any number
+    of rows.  bfloat16: among batches of up to 64 rows (the decoding kernel) and among larger
+    ones (the tiled kernel); between the two a row differs by the rounding of 32-bit sums."""
     k = kernels(dtype)
-    for N, K in [(96, 80), (256, 512), (130, 1000)]:
-        x, _ = as_dtype(rnd(200, K, seed=14), dtype)
+    for N, K in [(96, 80), (256, 512), (130, 1000), (512, 1024), (300, 4096)]:
+        x, _ = as_dtype(rnd(400, K, seed=14), dtype)
         w, _ = as_dtype(rnd(N, K, seed=15, scale=0.2), dtype)
-        full = torch.empty(200, N, dtype=torch.float32, device="cuda")
+        full = torch.empty(400, N, dtype=torch.float32, device="cuda")
         k.gemm(x, w, full, None, MODE_STORE_F32)
-        for m in (1, 3, 16, 17, 64, 130):
+        small = torch.empty(64, N, dtype=torch.float32, device="cuda")
+        k.gemm(x[:64], w, small, None, MODE_STORE_F32)
+        for m in (1, 3, 16, 17, 33, 64, 65, 130, 257, 300):
             part = torch.empty(m, N, dtype=torch.float32, device="cuda")
             k.gemm(x[:m], w, part, None, MODE_STORE_F32)
-            assert torch.equal(part, full[:m]), (N, K, m)
+            same_as = full if (dtype == "float32" or m > 64) else small
+            assert torch.equal(part, same_as[:m]), (N, K, m)
+        assert (small - full[:64]).abs().max() <= 1e-5 * full.abs().max()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -259,6 +265,126 @@ def test_topk_with_penalty_on_the_device():
         assert [g & 0xFFFFFFFF for g in got] == want, r
 
 
+# --------------------------------------------------------------------------- matrix-core attention
+def _mfma_case(nh, nkv, hd, page, T, window, seed=0, scale_q=1.0):
+    q = rnd(T, nh, hd, seed=seed + 1) * scale_q
+    kk = rnd(T, nkv, hd, seed=seed + 2)
+    vv = rnd(T, nkv, hd, seed=seed + 3)
+    qd, qr = as_dtype(q, "bfloat16")
+    _, kr = as_dtype(kk, "bfloat16")
+    _, vr = as_dtype(vv, "bfloat16")
+    kc, vc, table = paged_cache(kr, vr, page, "bfloat16", seed=seed)
+    ref = P.causal_attention(qr, kr, vr, window).view(T, nh * hd)
+    return qd.view(T, nh * hd), kc, vc, table, ref
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page,T,window", [
+    (4, 2, 64, 16, 300, 0), (7, 1, 128, 16, 257, 0), (6, 2, 128, 8, 130, 0), (2, 2, 64, 64, 200, 0),
+    (8, 2, 128, 32, 333, 0), (4, 1, 64, 16, 400, 100), (14, 2, 128, 16, 129, 37), (16, 1, 64, 8, 70, 0)])
+def test_prompt_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
+    k = kernels("bfloat16")
+    assert k.attention_fast_ok(hd, page, nh, nkv)
+    q, kc, vc, table, ref = _mfma_case(nh, nkv, hd, page, T, window)
+    pos = torch.arange(T, dtype=torch.int32).cuda()
+    rows = torch.zeros(T, dtype=torch.int32).cuda()
+    scale = 1.0 / math.sqrt(hd)
+    # the whole sequence in tiles of 128, then a portion that starts in the middle of a block
+    for start in (0, 77 if T > 100 else 3):
+        tiles = [(a, min(128, T - a)) for a in range(start, T, 128)]
+        out = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+        k.attention_prefill(q, nh * hd, kc, vc, table, pos, rows, out, torch.tensor(tiles, dtype=torch.int32).cuda(), nh, nkv,
+                            hd, page, window, scale)
+        assert not torch.isnan(out).any()                      # unused cache rows hold NaN: they must not leak
+        assert (out[start:].cpu().double() - ref[start:]).abs().max() <= tol("bfloat16", ref, bf16=1.5e-2)
+        assert out[:start].abs().sum() == 0                    # rows outside the tiles are not touched
+    # odd tiles: 2 tokens, 33 tokens, one token short of a block edge
+    tiles = [(5, 2), (60, min(33, T - 63)), (T - 3, 3)]          # every tile lies inside the T tokens
+    out = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+    k.attention_prefill(q, nh * hd, kc, vc, table, pos, rows, out, torch.tensor(tiles, dtype=torch.int32).cuda(), nh, nkv, hd,
+                        page, window, scale)
+    for a, n in tiles:
+        assert (out[a:a + n].cpu().double() - ref[a:a + n]).abs().max() <= tol("bfloat16", ref, bf16=1.5e-2)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,page,T,window", [
+    (4, 2, 64, 16, 300, 0), (7, 1, 128, 16, 1030, 0), (28, 4, 128, 16, 600, 0), (6, 2, 128, 8, 255, 0),
+    (2, 2, 64, 64, 257, 0), (16, 1, 64, 32, 513, 0), (4, 1, 64, 16, 900, 300), (5, 5, 128, 16, 64, 0)])
+def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
+    k = kernels("bfloat16")
+    q, kc, vc, table, ref = _mfma_case(nh, nkv, hd, page, T, window, seed=5)
+    pos = torch.arange(T, dtype=torch.int32).cuda()
+    rows = torch.zeros(T, dtype=torch.int32).cuda()
+    scale = 1.0 / math.sqrt(hd)
+    # single tokens at chosen positions: first, block and chunk edges, last
+    picks = sorted({0, 1, 15, 16, 63, 64, 65, 255, 256, 257, 511, 512, T // 2, T - 2, T - 1} & set(range(T)))
+    idx = torch.tensor(picks, dtype=torch.int32).cuda()
+    lo = max(0, max(picks) + 1 - window) if window else 0
+    chunks = (max(picks) - lo // 64 * 64) // 256 + 1 if window == 0 else max(
+        (p - (max(0, p + 1 - window) // 64 * 64)) // 256 + 1 for p in picks)
+    partial = torch.empty(k.attention_decode_workspace(len(picks), nh, hd, chunks), dtype=torch.float32, device="cuda")
+    out = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+    k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, out, idx, partial, chunks, nh, nkv, hd, page, window, scale)
+    assert not torch.isnan(out).any()
+    got, want = out[picks].cpu().double(), ref[picks]
+    assert (got - want).abs().max() <= tol("bfloat16", ref, bf16=1.5e-2)
+    untouched = sorted(set(range(T)) - set(picks))
+    assert out[untouched].abs().sum() == 0
+    # a token's row does not depend on which other tokens share the launch
+    solo = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+    one = torch.tensor([picks[-1]], dtype=torch.int32).cuda()
+    k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, solo, one, partial, chunks, nh, nkv, hd, page, window, scale)
+    assert torch.equal(solo[picks[-1]], out[picks[-1]])
+
+
+def test_matrix_core_attention_finds_a_far_key_and_respects_the_windows_edge():
+    k = kernels("bfloat16")
+    nh, nkv, hd, page, T = 4, 2, 128, 16, 700
+    q = rnd(T, nh, hd, seed=7) * 0.1
+    kk = rnd(T, nkv, hd, seed=8) * 0.1
+    vv = rnd(T, nkv, hd, seed=9)
+    far = 15
+    kk[far, 1] = 0
+    kk[far, 1, 3] = 40.0
+    q[T - 1, 2] = 0
+    q[T - 1, 2, 3] = 40.0
+    qd, qr = as_dtype(q, "bfloat16")
+    _, kr = as_dtype(kk, "bfloat16")
+    _, vr = as_dtype(vv, "bfloat16")
+    kc, vc, table = paged_cache(kr, vr, page, "bfloat16")
+    pos = torch.arange(T, dtype=torch.int32).cuda()
+    rows = torch.zeros(T, dtype=torch.int32).cuda()
+    scale = 1.0 / math.sqrt(hd)
+    one = torch.tensor([T - 1], dtype=torch.int32).cuda()
+    tile = torch.tensor([[T - 40, 40]], dtype=torch.int32).cuda()
+    partial = torch.empty(k.attention_decode_workspace(1, nh, hd, 4), dtype=torch.float32, device="cuda")
+    for w, seen in ((0, True), (T - 1 - far, False), (T - far, True)):
+        ref = P.causal_attention(qr, kr, vr, w)[T - 1]
+        for which in ("decode", "prefill"):
+            out = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+            if which == "decode":
+                k.attention_decode(qd.view(T, -1), nh * hd, kc, vc, table, pos, rows, out, one, partial, 4, nh, nkv, hd,
+                                   page, w, scale)
+            else:
+                k.attention_prefill(qd.view(T, -1), nh * hd, kc, vc, table, pos, rows, out, tile, nh, nkv, hd, page, w, scale)
+            got = out[T - 1].cpu().double().view(nh, hd)
+            assert (got - ref).abs().max() <= tol("bfloat16", ref, bf16=1.5e-2), (w, which)
+            assert ((got[2] - vr[far, 1]).abs().max() < 2e-2) == seen, (w, which)
+
+
+def test_matrix_core_attention_refuses_other_sizes():
+    k = kernels("bfloat16")
+    assert not k.attention_fast_ok(80, 16, 4, 2) and not k.attention_fast_ok(128, 5, 4, 2)
+    assert not k.attention_fast_ok(128, 16, 34, 2)             # a group of 17 heads
+    assert not kernels("float32").attention_fast_ok(128, 16, 4, 2)
+    q = torch.zeros(4, 160, dtype=torch.bfloat16, device="cuda")
+    kc = torch.zeros(2, 1, 16, 80, dtype=torch.bfloat16, device="cuda")
+    i32 = torch.zeros(4, dtype=torch.int32, device="cuda")
+    with pytest.raises(KernelError) as e:
+        k.attention_prefill(q, 160, kc, kc.view(2, 1, 80, 16), i32.view(1, 4), i32, i32, torch.zeros_like(q),
+                            torch.tensor([[0, 4]], dtype=torch.int32).cuda(), 2, 1, 80, 16, 0, 1.0)
+    assert "head_dim 80" in str(e.value)
+
+
 def test_kernels_refuse_what_they_cannot_run():
     k = kernels("float32")
     x = torch.zeros(2, 8, device="cuda")
@@ -272,6 +398,6 @@ def test_kernels_refuse_what_they_cannot_run():
     cache = torch.zeros(2, 1, 8, 24, device="cuda")
     i32 = torch.zeros(1, dtype=torch.int32, device="cuda")
     with pytest.raises(KernelError) as e:
-        k.attention(q, 24, cache, cache, i32.view(1, 1), i32, i32, torch.zeros(1, 24, device="cuda"), 1, 1, 24, 8, 0,
+        k.attention(q, 24, cache, cache.view(2, 1, 24, 8), i32.view(1, 1), i32, i32, torch.zeros(1, 24, device="cuda"), 1, 1, 24, 8, 0,
                     1.0)
     assert "head_dim 24" in str(e.value)

@@ -11,7 +11,8 @@ from plain import qwen2_plain as P
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [1, 5, 17, 33, 70, 100], "B": [2, 9, 70, 41, 130, 64], "C": [3, 66, 129]}
+LENGTHS = {"A": [1, 5, 17, 33, 70, 100], "B": [2, 9, 70, 41, 130, 64], "C": [3, 66, 129], "D": [4, 70, 300, 131],
+           "E": [2, 129, 64, 520]}
 
 
 def oracle(model_dir, prompts):
@@ -100,7 +101,7 @@ def max_tokens_for(tb, prompts_by_id):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_every_schedule_matches_the_plain_implementation(name, dtype, model_dirs, tmp_path):
     model_dir = model_dirs(name, "float32" if dtype == "float32" else "bfloat16")
     prompts = prompts_for(name, LENGTHS[name], seed=3)
