@@ -112,8 +112,11 @@ class LLM:
                 wanted = [p for p in plan if p.wants_logits]
                 picks = []
                 if wanted:
-                    picks = pick_rows(self.rt, logits, [reqs[p.id].sampler for p in wanted],
-                                      [reqs[p.id].tokens for p in wanted])
+                    if self.engine.last_picks is not None and all(reqs[p.id].sampler is None for p in wanted):
+                        picks = self.engine.last_picks.tolist()     # a decoding step picked greedily already
+                    else:
+                        picks = pick_rows(self.rt, logits, [reqs[p.id].sampler for p in wanted],
+                                          [reqs[p.id].tokens for p in wanted])
                 at = 0
                 for p in plan:
                     r = reqs[p.id]

@@ -67,6 +67,11 @@ class StepContext:
         self.seq_rows = meta[2, :n_tokens]
         self.spans = spans
         self.shared: Dict = {}       # per-step values shared by parts with equal parameters
+        # a step of single tokens that may be replayed from a graph: the index list 0..T-1 on the
+        # device, and what the mixers said about the step's shape (see Mixer.decode_shape)
+        self.decode_only = False
+        self.decode_index: Optional[torch.Tensor] = None
+        self.decode_shapes: Dict = {}
 
     def no_rotation(self) -> torch.Tensor:
         return torch.empty((self.n_tokens, 0, 2), dtype=torch.float32, device=self.rt.device)
@@ -85,6 +90,25 @@ class Engine:
         self.live: Dict[Hashable, LiveRequest] = {}
         self.has_window = any(p.spec.window > 0 for p in plans)
         self.steps = 0
+        # decoding steps replayed from HIP graphs: static inputs and outputs, one graph per shape
+        parts = [model.embedding, model.final_norm, model.head] + list(model.blocks) + [b.mixer for b in model.blocks] \
+            + [b.feed_forward for b in model.blocks]
+        self.graphs_ok = cfg.use_graphs and all(getattr(p, "graph_safe", False) for p in parts)
+        self._graphs: Dict = {}
+        self._graph_pool = None
+        self._shape_mixers = []         # one mixer for each distinct thing a decoding step's shape depends on
+        seen = set()
+        for b in model.blocks:
+            pair = b.mixer.decode_shape([0])
+            if pair is not None and pair[0] not in seen:
+                seen.add(pair[0])
+                self._shape_mixers.append(b.mixer)
+        self._meta = torch.zeros((3, cfg.max_seqs), dtype=torch.int32, device=rt.device)
+        self._meta_host = torch.zeros((3, cfg.max_seqs), dtype=torch.int32).pin_memory()
+        self._index = torch.arange(cfg.max_seqs, dtype=torch.int32, device=rt.device)
+        self._logits = None
+        self._picks = torch.zeros(cfg.max_seqs, dtype=torch.int32, device=rt.device)
+        self.last_picks: Optional[torch.Tensor] = None
 
     # ------------------------------------------------------------------ sizing
     def _pool_size(self, spec, n_layers: int, page_size: int) -> int:
@@ -156,6 +180,7 @@ class Engine:
             raise
 
         logits = None
+        self.last_picks = None
         if entries:
             tokens, positions, rows, want_rows, spans = [], [], [], [], []
             for e in entries:
@@ -168,13 +193,16 @@ class Engine:
                 rows.extend([req.slot] * n)
                 want_rows.extend(at + int(w) for w in e.want)
             T = len(tokens)
-            meta = torch.tensor([tokens, positions, rows], dtype=torch.int32).to(self.rt.device)
             self.cache.sync_tables()
-            ctx = StepContext(self.rt, self.cache, self.ws, meta, T, spans)
-            x = self.model.forward(ctx)
-            if want_rows:
-                sel = torch.tensor(want_rows, dtype=torch.int32).to(self.rt.device)
-                logits = self.model.logits(ctx, x, sel)
+            if T == len(entries) and len(want_rows) == T and T <= self.cfg.max_seqs:
+                logits = self._decode_step(tokens, positions, rows, spans)
+            else:
+                meta = torch.tensor([tokens, positions, rows], dtype=torch.int32).to(self.rt.device)
+                ctx = StepContext(self.rt, self.cache, self.ws, meta, T, spans)
+                x = self.model.forward(ctx)
+                if want_rows:
+                    sel = torch.tensor(want_rows, dtype=torch.int32).to(self.rt.device)
+                    logits = self.model.logits(ctx, x, sel)
             for e in entries:
                 req = self.live[e.id]
                 req.n_cached += len(e.tokens)
@@ -183,4 +211,54 @@ class Engine:
             self.steps += 1
         for rid in end:
             self.release(rid)
+        return logits
+
+    # ------------------------------------------------------------------ decoding steps
+    def _decode_forward(self, T: int, spans: List[Span], shapes: Dict):
+        """A step of T single tokens whose tokens, positions and slots are in `self._meta`: the
+        launches that a graph captures.  Logits go to the static buffer, greedy picks beside them."""
+        ctx = StepContext(self.rt, self.cache, self.ws, self._meta, T, spans)
+        ctx.decode_only = True
+        ctx.decode_index = self._index[:T]
+        ctx.decode_shapes = shapes
+        x = self.model.forward(ctx)
+        logits = self.model.logits(ctx, x, ctx.decode_index, out=self._logits[:T])
+        self.rt.k.argmax(logits, self._picks[:T])
+        return logits
+
+    def _decode_step(self, tokens, positions, rows, spans) -> torch.Tensor:
+        """Every entry brings one token and wants its logits.  Inputs are copied into static
+        device buffers; with graphs on, the launches of this (number of tokens, shape) are
+        captured once and replayed afterwards.  Returns a view of a static logits buffer, valid
+        until the next decoding step; `last_picks` holds the greedy pick of each row."""
+        T = len(tokens)
+        if self._logits is None:
+            self._logits = torch.empty((self.cfg.max_seqs, self.model.vocab_size), dtype=torch.float32,
+                                       device=self.rt.device)
+        host = self._meta_host
+        host[:, :T] = torch.tensor([tokens, positions, rows], dtype=torch.int32)
+        self._meta.copy_(host)          # one small copy, complete before the host buffer is written again
+        shapes = {}
+        for mixer in self._shape_mixers:
+            name, value = mixer.decode_shape(positions)
+            shapes[name] = value
+        if not self.graphs_ok:
+            logits = self._decode_forward(T, spans, shapes)
+        else:
+            key = (T, tuple(sorted(shapes.items(), key=repr)))
+            entry = self._graphs.get(key)
+            if entry is None:
+                # once without capture: kernels set themselves up at their first launch, and a
+                # decoding step writes the same cache rows however often it runs
+                self._decode_forward(T, spans, shapes)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                if self._graph_pool is None:
+                    self._graph_pool = torch.cuda.graph_pool_handle()
+                with torch.cuda.graph(graph, pool=self._graph_pool):
+                    logits = self._decode_forward(T, spans, shapes)
+                entry = self._graphs[key] = (graph, logits)
+            entry[0].replay()
+            logits = entry[1]
+        self.last_picks = self._picks[:T]
         return logits

@@ -35,28 +35,41 @@ class AttentionPlan:
     once per step and window, shared by all layers."""
 
     def __init__(self, ctx, window: int, n_heads: int, head_dim: int):
-        tiles, singles, chunks = [], [], 1
-        for s in ctx.spans:
-            if s.q_len == 1:
-                singles.append(s.q_start)
-                pos = s.start_pos
-                lo = max(0, pos + 1 - window) if window > 0 else 0
-                first = lo // DECODE_BLOCK * DECODE_BLOCK
-                chunks = max(chunks, (pos - first) // DECODE_CHUNK + 1)
-            else:
-                for at in range(0, s.q_len, PREFILL_TILE):
-                    tiles.append((s.q_start + at, min(PREFILL_TILE, s.q_len - at)))
-        # the kernels trust these indices: check them here, on the host
-        if any(a < 0 or n < 1 or a + n > ctx.n_tokens for a, n in tiles) or any(not 0 <= t < ctx.n_tokens for t in singles):
-            raise ValueError("attention plan: a span lies outside the tokens of the step")
         dev = ctx.rt.device
-        self.tiles = torch.tensor(tiles, dtype=torch.int32).to(dev) if tiles else None
-        self.decode_tokens = torch.tensor(singles, dtype=torch.int32).to(dev) if singles else None
-        self.max_chunks = chunks
+        self.tiles = None
         self.partial = None
-        if singles and chunks > 1:
-            n = ctx.rt.k.attention_decode_workspace(len(singles), n_heads, head_dim, chunks)
+        if ctx.decode_only:
+            # every span is one token: the engine keeps the index list on the device and has
+            # counted the chunks (what a captured graph replays must not come from the host)
+            self.decode_tokens = ctx.decode_index
+            self.max_chunks = ctx.decode_shapes[("attention_chunks", window)]
+            n_single = ctx.n_tokens
+        else:
+            tiles, singles, chunks = [], [], 1
+            for s in ctx.spans:
+                if s.q_len == 1:
+                    singles.append(s.q_start)
+                    chunks = max(chunks, decode_chunks_of(s.start_pos, window))
+                else:
+                    for at in range(0, s.q_len, PREFILL_TILE):
+                        tiles.append((s.q_start + at, min(PREFILL_TILE, s.q_len - at)))
+            # the kernels trust these indices: check them here, on the host
+            if (any(a < 0 or n < 1 or a + n > ctx.n_tokens for a, n in tiles)
+                    or any(not 0 <= t < ctx.n_tokens for t in singles)):
+                raise ValueError("attention plan: a span lies outside the tokens of the step")
+            self.tiles = torch.tensor(tiles, dtype=torch.int32).to(dev) if tiles else None
+            self.decode_tokens = torch.tensor(singles, dtype=torch.int32).to(dev) if singles else None
+            self.max_chunks = chunks
+            n_single = len(singles)
+        if n_single and self.max_chunks > 1:
+            n = ctx.rt.k.attention_decode_workspace(n_single, n_heads, head_dim, self.max_chunks)
             self.partial = torch.empty(n, dtype=torch.float32, device=dev)
+
+
+def decode_chunks_of(pos: int, window: int) -> int:
+    """Chunks of 256 positions the decoding kernel cuts a token's range into."""
+    lo = max(0, pos + 1 - window) if window > 0 else 0
+    return (pos - lo // DECODE_BLOCK * DECODE_BLOCK) // DECODE_CHUNK + 1
 
 
 def attention_plan(ctx, window: int, n_heads: int, head_dim: int) -> AttentionPlan:
@@ -68,6 +81,7 @@ def attention_plan(ctx, window: int, n_heads: int, head_dim: int) -> AttentionPl
 
 
 class GQAttention(Mixer):
+    graph_safe = True
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
         p = params
@@ -107,6 +121,12 @@ class GQAttention(Mixer):
 
     def cache_spec(self) -> Optional[CacheSpec]:
         return CacheSpec(entries=2, heads=self.nkv, head_dim=self.hd, window=self.window)
+
+    def decode_shape(self, positions):
+        """The decoding kernel's grid depends on the longest context, in chunks of 256 positions,
+        rounded up to a power of two so that few shapes exist."""
+        most = max(decode_chunks_of(p, self.window) for p in positions)
+        return ("attention_chunks", self.window), 1 << (most - 1).bit_length()
 
     def load(self, store, rt) -> None:
         self.w_qkv = store.fused_matrix([self.n[k] + ".weight" for k in ("q", "k", "v")])

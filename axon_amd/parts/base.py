@@ -68,7 +68,13 @@ class CacheBinding:
 
 
 class Part:
-    """Common to all parts: tensors in, then bound to device memory."""
+    """Common to all parts: tensors in, then bound to device memory.
+
+    `graph_safe`: the part's work in a step is a fixed sequence of kernel launches that read
+    everything that changes between steps (tokens, positions, block tables) from device memory,
+    so a decoding step can be captured once into a HIP graph and replayed.  A part that
+    branches on host values or keeps per-request state must leave it False."""
+    graph_safe = False
 
     def __init__(self, params: Dict[str, Any], prefix: str = ""):
         self.params = dict(params)
@@ -97,6 +103,13 @@ class Mixer(Part):
         return None
 
     def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def decode_shape(self, positions) -> Optional[Tuple[Any, Any]]:
+        """For a step of single tokens at `positions`: (name, value) if the launches of this
+        mixer depend on more than the number of tokens (say, on how long the contexts are), so
+        that a captured graph is replayed only for steps of the same shape.  The pair is handed
+        back in `ctx.decode_shapes[name]`.  None: nothing else matters."""
         return None
 
     def forward(self, ctx, binding: CacheBinding, h, residual) -> None:

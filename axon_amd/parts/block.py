@@ -12,6 +12,7 @@ from .base import Block, CacheBinding, TensorDecl, register_block
 
 
 class PreNormBlock(Block):
+    graph_safe = True
     norm1_name = "input_layernorm.weight"
     norm2_name = "post_attention_layernorm.weight"
 

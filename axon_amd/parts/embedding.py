@@ -16,6 +16,7 @@ from .base import Part, TensorDecl, register_embedding, register_head
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
         self.vocab = int(params["vocab_size"])
@@ -36,6 +37,7 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
+    graph_safe = True
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
         self.vocab = int(params["vocab_size"])

@@ -13,6 +13,7 @@ from .base import FeedForward, TensorDecl, register_feed_forward
 
 
 class SwiGLUMLP(FeedForward):
+    graph_safe = True
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
         self.hidden = int(params["hidden_size"])

@@ -11,6 +11,7 @@ from .base import Norm, TensorDecl, register_norm
 
 
 class RMSNorm(Norm):
+    graph_safe = True
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
         self.size = int(params["size"])

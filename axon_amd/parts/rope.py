@@ -15,6 +15,7 @@ from .base import PositionEncoding, register_position
 
 
 class RotaryEncoding(PositionEncoding):
+    graph_safe = True
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
         self.head_dim = int(params["head_dim"])
