@@ -53,8 +53,8 @@ int axk_attention(const void* q, int q_stride, const void* k_cache, const void* 
 // axk_attention_fast_ok: 1 if they take this head size, page size and group of heads.
 // axk_attention_prefill: tiles [n_tiles][2] = (first token, count <= 128): consecutive tokens of
 // one request; every token of the step in some tile gets its row of `out`.
-// axk_attention_decode: token_index [n_tokens] names single tokens; a context longer than 256
-// positions is cut into chunks whose partial results go through `partial`
+// axk_attention_decode: token_index [n_tokens] names single tokens; a context longer than 64
+// positions is cut into chunks of 64 whose partial results go through `partial`
 // (axk_attention_decode_workspace floats) and are folded in ascending order.
 int axk_attention_fast_ok(int head_dim, int page_size, int n_heads, int n_kv_heads);
 int axk_attention_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
@@ -70,7 +70,8 @@ int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const
                          int page_size, int window, float scale, void* stream);
 
 // out = epilogue(X [M, K] . W [N, K]^T + bias).  mode 0: store elem [M, N]; 1: add into
-// float32 [M, N] (the residual stream); 2: store float32 [M, N] (logits).
+// float32 [M, N] (the residual stream); 2: store float32 [M, N] (logits); 3: W holds 2 N rows,
+// gate rows then up rows, and out elem [M, N] = silu(X . gate^T) * (X . up^T) (no bias).
 // x_stride / out_stride: elements between rows.
 int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
              int out_stride, int m, int n, int k, int mode, void* stream);

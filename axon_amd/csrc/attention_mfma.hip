@@ -1,8 +1,8 @@
 // Paged causal attention on the matrix cores (bfloat16 build only): one kernel for prompt
 // portions, one for decoding tokens.  Both keep the order of attention.hip: positions in
 // blocks of 64 aligned to absolute position, folded in ascending order with running
-// (max, sum, output); the decoding kernel splits a long context into chunks of 256
-// positions (4 blocks, a size that depends on nothing) and a second kernel folds the chunks
+// (max, sum, output); the decoding kernel gives every block of 64 positions to a wave of its
+// own (a size that depends on nothing) and a second kernel folds the blocks' partial results
 // in ascending order.  No atomics.  Scores, softmax and all sums are 32-bit; q, k, v and the
 // softmax weights enter the MFMAs as bfloat16.
 //
@@ -242,13 +242,13 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
 }
 
 // ============================================================================ decoding tokens
-// grid (tokens, kv heads, chunks): one wave per (token, kv head, chunk of 256 positions).  The
-// wave streams K rows and V^T rows of its chunk straight from the pages into 16x16x32 MFMA
-// operands; the query heads of the group are the 16 columns (a group of up to 16 heads).
+// grid (tokens, kv heads, chunks): one wave per (token, kv head, chunk of 64 positions = one
+// block of the fold).  The wave issues every load of its chunk at once (K rows and V^T rows go
+// straight from the pages into 16x16x32 MFMA operands, 32 KB in flight per wave), then
+// multiplies; the query heads of the group are the 16 columns (a group of up to 16 heads).
 // Output: if the token's whole range is one chunk, the normalised result; else the chunk's
 // (max, sum, unnormalised output) into `partial`, folded by attention_combine_kernel.
-#define DC_CHUNK 256
-#define DC_BLOCK 64
+#define DC_CHUNK 64
 
 template <int HD>
 __global__ void __launch_bounds__(64)
@@ -265,15 +265,48 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
   const int group = n_heads / n_kv_heads;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
-  const int first = (lo / DC_BLOCK) * DC_BLOCK;
+  const int first = (lo / DC_CHUNK) * DC_CHUNK;
   const int n_chunks = (pos - first) / DC_CHUNK + 1;
   if (chunk >= n_chunks) return;
-  const int c0 = first + chunk * DC_CHUNK;
-  const int c1 = min(c0 + DC_CHUNK - 1, pos);        // last position of this chunk
+  const int p0 = first + chunk * DC_CHUNK;
+  const int c1 = min(p0 + DC_CHUNK - 1, pos);        // last position of this chunk
   const int32_t* table_row = block_table + (size_t)seq_rows[t] * table_stride;
   const int r16 = lane & 15, q4 = lane >> 4;
   const size_t kv_head_stride = (size_t)HD * page_size;
 
+  // ---- every load first.  K (A operand of S^T): 4 tiles of 16 positions; row = position
+  // p0 + 16 pt + r16, 8 consecutive dims from 32 ks + 8 q4.  Rows past the chunk's end: any valid
+  // row (masked below).
+  uint4 kf[4][KS];
+#pragma unroll
+  for (int pt = 0; pt < 4; ++pt) {
+    const int p = min(p0 + pt * 16 + r16, c1);
+    const bf16_t* krow = k_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * kv_head_stride +
+                         (size_t)(p % page_size) * HD + q4 * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kf[pt][ks] = *reinterpret_cast<const uint4*>(krow + ks * 32);
+  }
+  // V^T (A operand of O^T): k step u takes the lane's positions p0 + 32u + 4 q4 + {0..3} and the
+  // same + 16 (what S^T leaves in its registers): two 8-byte reads per output tile.
+  uint2 vf[2][DT][2];
+  int keep[2][2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int pa = p0 + 32 * u + 4 * q4, pb = pa + 16;
+    keep[u][0] = max(0, min(c1 - pa + 1, 4));
+    keep[u][1] = max(0, min(c1 - pb + 1, 4));
+    const int pa_c = min(pa, c1), pb_c = min(pb, c1);
+    const bf16_t* va = v_cache + ((size_t)table_row[pa_c / page_size] * n_kv_heads + kvh) * kv_head_stride +
+                       ((pa_c % page_size) & ~3);
+    const bf16_t* vb = v_cache + ((size_t)table_row[pb_c / page_size] * n_kv_heads + kvh) * kv_head_stride +
+                       ((pb_c % page_size) & ~3);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const size_t doff = (size_t)(dt * 16 + r16) * page_size;
+      vf[u][dt][0] = *reinterpret_cast<const uint2*>(va + doff);
+      vf[u][dt][1] = *reinterpret_cast<const uint2*>(vb + doff);
+    }
+  }
   // Q^T (B operand): column = head of the group (zero beyond it), 8 consecutive dims
   bf16x8 qf[KS];
   {
@@ -286,102 +319,73 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
     }
   }
 
+  // ---- S^T [64 positions][16 heads]
+  f32x4 s_acc[4];
+#pragma unroll
+  for (int pt = 0; pt < 4; ++pt) {
+    s_acc[pt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      s_acc[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag_of(kf[pt][ks]), qf[ks], s_acc[pt], 0, 0, 0);
+  }
+  // this lane: head r16; positions p0 + 16 pt + 4 q4 + e
+  const float c = scale * LOG2E;
+  float m = -INFINITY;
+#pragma unroll
+  for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int p = p0 + pt * 16 + q4 * 4 + e;
+      const float v = (p <= c1 && p >= lo) ? s_acc[pt][e] * c : -INFINITY;
+      s_acc[pt][e] = v;
+      m = fmaxf(m, v);
+    }
+  m = fmaxf(m, __shfl_xor(m, 16, AXON_WAVE));
+  m = fmaxf(m, __shfl_xor(m, 32, AXON_WAVE));
+  const float mref = m == -INFINITY ? 0.0f : m;
+  float l = 0.0f;
+#pragma unroll
+  for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float pv = __builtin_amdgcn_exp2f(s_acc[pt][e] - mref);
+      s_acc[pt][e] = pv;
+      l += pv;
+    }
+  l += __shfl_xor(l, 16, AXON_WAVE);
+  l += __shfl_xor(l, 32, AXON_WAVE);
+
+  // ---- O^T [HD][16 heads] = V^T P^T.  Positions past the chunk's end were never written: their
+  // weights are zero, and the values read for them are replaced by zero so that zero times
+  // anything stays zero.
   f32x4 o_acc[DT];
 #pragma unroll
-  for (int i = 0; i < DT; ++i) o_acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  float m_run = -INFINITY, l_run = 0.0f;
-  const float c = scale * LOG2E;
-
-  for (int p0 = c0; p0 <= c1; p0 += DC_BLOCK) {
-    // S^T [64 positions][16 heads]: 4 tiles of 16 positions; A = K rows straight from the pages
-    f32x4 s_acc[4];
+  for (int u = 0; u < 2; ++u) {
+    union { uint32_t w[4]; bf16x8 f; } pf;
+    pf.w[0] = pack_bf16(s_acc[2 * u][0], s_acc[2 * u][1]);
+    pf.w[1] = pack_bf16(s_acc[2 * u][2], s_acc[2 * u][3]);
+    pf.w[2] = pack_bf16(s_acc[2 * u + 1][0], s_acc[2 * u + 1][1]);
+    pf.w[3] = pack_bf16(s_acc[2 * u + 1][2], s_acc[2 * u + 1][3]);
 #pragma unroll
-    for (int pt = 0; pt < 4; ++pt) {
-      s_acc[pt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-      const int p = min(p0 + pt * 16 + r16, c1);   // rows past the chunk: any valid row, masked below
-      const bf16_t* krow = k_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * kv_head_stride +
-                           (size_t)(p % page_size) * HD + q4 * 8;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        s_acc[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag_of(*reinterpret_cast<const uint4*>(krow + ks * 32)),
-                                                            qf[ks], s_acc[pt], 0, 0, 0);
-    }
-    // this lane: head r16; positions p0 + pt*16 + q4*4 + e
-    float mloc = -INFINITY;
-#pragma unroll
-    for (int pt = 0; pt < 4; ++pt)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int p = p0 + pt * 16 + q4 * 4 + e;
-        const float v = (p <= c1 && p >= lo) ? s_acc[pt][e] * c : -INFINITY;
-        s_acc[pt][e] = v;
-        mloc = fmaxf(mloc, v);
+    for (int dt = 0; dt < DT; ++dt) {
+      uint2 v0 = vf[u][dt][0], v1 = vf[u][dt][1];
+      if (keep[u][0] < 4) {
+        if (keep[u][0] < 1) v0.x = 0; else if (keep[u][0] < 2) v0.x &= 0xffffu;
+        if (keep[u][0] < 3) v0.y = 0; else v0.y &= 0xffffu;
       }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, AXON_WAVE));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, AXON_WAVE));
-    const float mn = fmaxf(m_run, mloc);
-    const float mref = mn == -INFINITY ? 0.0f : mn;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - mref);
-    float lsum = 0.0f;
-#pragma unroll
-    for (int pt = 0; pt < 4; ++pt)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float pv = __builtin_amdgcn_exp2f(s_acc[pt][e] - mref);
-        s_acc[pt][e] = pv;
-        lsum += pv;
+      if (keep[u][1] < 4) {
+        if (keep[u][1] < 1) v1.x = 0; else if (keep[u][1] < 2) v1.x &= 0xffffu;
+        if (keep[u][1] < 3) v1.y = 0; else v1.y &= 0xffffu;
       }
-    lsum += __shfl_xor(lsum, 16, AXON_WAVE);
-    lsum += __shfl_xor(lsum, 32, AXON_WAVE);
-    l_run = l_run * alpha + lsum;
-    m_run = mn;
-#pragma unroll
-    for (int i = 0; i < DT; ++i)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o_acc[i][e] *= alpha;
-
-    // O^T [HD][16 heads] += V^T P^T: k step u takes tiles 2u and 2u + 1: the lane's positions are
-    // p0 + 32u + 4 q4 + {0..3} and the same + 16: two 8-byte reads of V^T per output tile
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      union { uint32_t w[4]; bf16x8 f; } pf;
-      pf.w[0] = pack_bf16(s_acc[2 * u][0], s_acc[2 * u][1]);
-      pf.w[1] = pack_bf16(s_acc[2 * u][2], s_acc[2 * u][3]);
-      pf.w[2] = pack_bf16(s_acc[2 * u + 1][0], s_acc[2 * u + 1][1]);
-      pf.w[3] = pack_bf16(s_acc[2 * u + 1][2], s_acc[2 * u + 1][3]);
-      const int pa = p0 + 32 * u + 4 * q4, pb = pa + 16;
-      // positions past the chunk's end were never written: their weights are zero, and the
-      // values read for them are replaced by zero so that zero times anything stays zero
-      const bool ok_a = pa <= c1, ok_b = pb <= c1;
-      const int pa_c = min(pa, c1), pb_c = min(pb, c1);
-      const bf16_t* va = v_cache + ((size_t)table_row[pa_c / page_size] * n_kv_heads + kvh) * kv_head_stride +
-                         ((pa_c % page_size) & ~3);
-      const bf16_t* vb = v_cache + ((size_t)table_row[pb_c / page_size] * n_kv_heads + kvh) * kv_head_stride +
-                         ((pb_c % page_size) & ~3);
-      // within a group of 4 positions, those beyond c1 are cleared one by one
-      const int keep_a = ok_a ? min(c1 - pa + 1, 4) : 0, keep_b = ok_b ? min(c1 - pb + 1, 4) : 0;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const size_t doff = (size_t)(dt * 16 + r16) * page_size;
-        uint2 v0 = *reinterpret_cast<const uint2*>(va + doff);
-        uint2 v1 = *reinterpret_cast<const uint2*>(vb + doff);
-        if (keep_a < 4) {
-          if (keep_a < 1) v0.x = 0; else if (keep_a < 2) v0.x &= 0xffffu;
-          if (keep_a < 3) v0.y = 0; else v0.y &= 0xffffu;
-        }
-        if (keep_b < 4) {
-          if (keep_b < 1) v1.x = 0; else if (keep_b < 2) v1.x &= 0xffffu;
-          if (keep_b < 3) v1.y = 0; else v1.y &= 0xffffu;
-        }
-        o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag_of2(v0, v1), pf.f, o_acc[dt], 0, 0, 0);
-      }
+      if (u == 0) o_acc[dt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag_of2(v0, v1), pf.f, o_acc[dt], 0, 0, 0);
     }
   }
 
   if (r16 >= group) return;
   const int head = kvh * group + r16;
   if (n_chunks == 1) {
-    const float inv = 1.0f / l_run;
+    const float inv = 1.0f / l;
     bf16_t* orow = out + (size_t)t * n_heads * HD + (size_t)head * HD;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -397,36 +401,57 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
     for (int dt = 0; dt < DT; ++dt)
       *reinterpret_cast<f32x4*>(dst + dt * 16 + q4 * 4) = o_acc[dt];
     if (q4 == 0) {
-      dst[HD] = m_run;
-      dst[HD + 1] = l_run;
+      dst[HD] = m;
+      dst[HD + 1] = l;
     }
   }
 }
 
-// Fold a token's chunks in ascending order: mn = max(M, m); O = O 2^(M - mn) + o 2^(m - mn);
-// L alike; out = O / L.  grid (tokens, heads), HD threads.
+// Fold a token's chunks: M = max of the chunks' maxima (exact in any order), then
+// L = sum l_c 2^(m_c - M) and O = sum o_c 2^(m_c - M); out = O / L.  The sums run in a fixed
+// order (the chunks' weights by a butterfly over lanes, the outputs chunk by chunk ascending).
+// grid (tokens, heads), HD threads.
+#define CMB_MAX_CHUNKS 1024
+
 template <int HD>
 __global__ void __launch_bounds__(HD)
 attention_combine_kernel(const float* __restrict__ partial, const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ token_index, bf16_t* __restrict__ out, int max_chunks, int n_heads,
                          int window) {
+  __shared__ float weight[CMB_MAX_CHUNKS];
+  __shared__ float red[2][HD / 64];
   const int t = token_index[blockIdx.x], head = blockIdx.y, d = threadIdx.x;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
-  const int n_chunks = (pos - (lo / DC_BLOCK) * DC_BLOCK) / DC_CHUNK + 1;
+  const int n_chunks = (pos - (lo / DC_CHUNK) * DC_CHUNK) / DC_CHUNK + 1;
   if (n_chunks == 1) return;  // the decoding kernel wrote the result itself
   const float* src = partial + ((size_t)blockIdx.x * n_heads + head) * max_chunks * (HD + 2);
-  float M = -INFINITY, L = 0.0f, O = 0.0f;
-  for (int cidx = 0; cidx < n_chunks; ++cidx) {
+  // the maximum: every thread takes chunks d, d + HD, ...
+  float mloc = -INFINITY;
+  for (int cidx = d; cidx < n_chunks; cidx += HD) mloc = fmaxf(mloc, src[(size_t)cidx * (HD + 2) + HD]);
+  mloc = wave_max(mloc);
+  if ((d & 63) == 0) red[0][d >> 6] = mloc;
+  __syncthreads();
+  float M = red[0][0];
+#pragma unroll
+  for (int i = 1; i < HD / 64; ++i) M = fmaxf(M, red[0][i]);
+  const float mref = M == -INFINITY ? 0.0f : M;
+  float lloc = 0.0f;
+  for (int cidx = d; cidx < n_chunks; cidx += HD) {
     const float* p = src + (size_t)cidx * (HD + 2);
-    const float m = p[HD], l = p[HD + 1], o = p[d];
-    const float mn = fmaxf(M, m);
-    const float mref = mn == -INFINITY ? 0.0f : mn;
-    const float a = __builtin_amdgcn_exp2f(M - mref), w = __builtin_amdgcn_exp2f(m - mref);
-    L = fmaf(l, w, L * a);
-    O = fmaf(o, w, O * a);
-    M = mn;
+    const float w = __builtin_amdgcn_exp2f(p[HD] - mref);
+    weight[cidx] = w;
+    lloc = fmaf(p[HD + 1], w, lloc);
   }
+  lloc = wave_sum(lloc);
+  if ((d & 63) == 0) red[1][d >> 6] = lloc;
+  __syncthreads();
+  float L = red[1][0];
+#pragma unroll
+  for (int i = 1; i < HD / 64; ++i) L += red[1][i];
+  float O = 0.0f;
+#pragma unroll 8
+  for (int cidx = 0; cidx < n_chunks; ++cidx) O = fmaf(src[(size_t)cidx * (HD + 2) + d], weight[cidx], O);
   out[(size_t)t * n_heads * HD + (size_t)head * HD + d] = float_to_bf16(O / L);
 }
 
@@ -498,6 +523,8 @@ extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_c
   AXK_REQUIRE(axk_attention_fast_ok(head_dim, page_size, n_heads, n_kv_heads),
               "attention_decode: head_dim %d, page size %d, %d/%d heads are not taken by this kernel", head_dim,
               page_size, n_heads, n_kv_heads);
+  AXK_REQUIRE(max_chunks <= CMB_MAX_CHUNKS, "attention_decode: %d chunks of 64 positions (at most %d: %d positions)",
+              max_chunks, CMB_MAX_CHUNKS, CMB_MAX_CHUNKS * 64);
   AXK_REQUIRE(n_tokens >= 0 && max_chunks >= 1 && max_chunks <= 65535 && n_kv_heads <= 65535 && window >= 0 &&
                   q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0,
               "attention_decode: bad arguments (tokens %d, chunks %d, window %d, q stride %d)", n_tokens, max_chunks,

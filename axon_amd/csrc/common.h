@@ -94,3 +94,10 @@ void axk_set_error(const char* fmt, ...);
   } while (0)
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Epilogues of a matrix product (see axk_gemm).
+enum { MODE_STORE = 0, MODE_ADD_F32 = 1, MODE_STORE_F32 = 2, MODE_SWIGLU = 3 };
+
+// act = (g / (1 + exp(-g))) * u: divide, then multiply (src/vmath.rs:128-132;
+// src/cuda/prefill.cu:109-123).
+__device__ inline float swiglu1(float g, float u) { return __fmul_rn(__fdiv_rn(g, 1.0f + expf(-g)), u); }

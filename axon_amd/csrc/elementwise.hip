@@ -47,7 +47,77 @@ extern "C" int axk_embed(const int32_t* tokens, const void* table, float* x, int
 // a butterfly per wave and the four waves in order: fixed by `dim` alone
 // (the reference's GPU twin does the same: src/cuda/decode.cu:212-249).
 #define NORM_THREADS 256
+#define NORM_CACHED 4  // float4 a thread keeps in registers: rows up to 4096 wide are read once
 
+__device__ inline float block_sum_256(float v, float* partial) {
+  v = wave_sum(v);
+  if ((threadIdx.x & (AXON_WAVE - 1)) == 0) partial[threadIdx.x / AXON_WAVE] = v;
+  __syncthreads();
+  float total = partial[0];
+#pragma unroll
+  for (int w = 1; w < NORM_THREADS / AXON_WAVE; ++w) total += partial[w];
+  return total;
+}
+
+__device__ inline void store4(elem_t* dst, float a, float b, float c, float d) {
+#if AXON_BF16
+  uint2 pk;
+  pk.x = (uint32_t)float_to_bf16(a).bits | ((uint32_t)float_to_bf16(b).bits << 16);
+  pk.y = (uint32_t)float_to_bf16(c).bits | ((uint32_t)float_to_bf16(d).bits << 16);
+  *reinterpret_cast<uint2*>(dst) = pk;
+#else
+  *reinterpret_cast<float4*>(dst) = make_float4(a, b, c, d);
+#endif
+}
+
+// Rows whose width is a multiple of 4: thread t takes the float4 t, t + 256, ...; the first
+// NORM_CACHED of them stay in registers between the sum and the scaling.  The order of the
+// sum depends on the width alone.
+__global__ void __launch_bounds__(NORM_THREADS)
+rmsnorm_vec_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows, const void* __restrict__ gain,
+                   int gain_is_f32, elem_t* __restrict__ out, int dim, float eps) {
+  __shared__ float partial[NORM_THREADS / AXON_WAVE];
+  const int r = blockIdx.x, n4 = dim >> 2;
+  const float4* src = reinterpret_cast<const float4*>(x + (size_t)(rows ? rows[r] : r) * dim);
+  float4 kept[NORM_CACHED];
+  float ss = 0.0f;
+#pragma unroll
+  for (int c = 0; c < NORM_CACHED; ++c) {
+    const int i = threadIdx.x + c * NORM_THREADS;
+    kept[c] = i < n4 ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    ss = fmaf(kept[c].x, kept[c].x, ss);
+    ss = fmaf(kept[c].y, kept[c].y, ss);
+    ss = fmaf(kept[c].z, kept[c].z, ss);
+    ss = fmaf(kept[c].w, kept[c].w, ss);
+  }
+  for (int i = threadIdx.x + NORM_CACHED * NORM_THREADS; i < n4; i += NORM_THREADS) {
+    const float4 v = src[i];
+    ss = fmaf(v.x, v.x, ss);
+    ss = fmaf(v.y, v.y, ss);
+    ss = fmaf(v.z, v.z, ss);
+    ss = fmaf(v.w, v.w, ss);
+  }
+  const float total = block_sum_256(ss, partial);
+  const float inv = 1.0f / sqrtf(total / (float)dim + eps);
+  elem_t* dst = out + (size_t)r * dim;
+#pragma unroll
+  for (int c = 0; c < NORM_CACHED; ++c) {
+    const int i = threadIdx.x + c * NORM_THREADS;
+    if (i < n4) {
+      const int e = i * 4;
+      store4(dst + e, (kept[c].x * inv) * load_vec(gain, gain_is_f32, e), (kept[c].y * inv) * load_vec(gain, gain_is_f32, e + 1),
+             (kept[c].z * inv) * load_vec(gain, gain_is_f32, e + 2), (kept[c].w * inv) * load_vec(gain, gain_is_f32, e + 3));
+    }
+  }
+  for (int i = threadIdx.x + NORM_CACHED * NORM_THREADS; i < n4; i += NORM_THREADS) {
+    const float4 v = src[i];
+    const int e = i * 4;
+    store4(dst + e, (v.x * inv) * load_vec(gain, gain_is_f32, e), (v.y * inv) * load_vec(gain, gain_is_f32, e + 1),
+           (v.z * inv) * load_vec(gain, gain_is_f32, e + 2), (v.w * inv) * load_vec(gain, gain_is_f32, e + 3));
+  }
+}
+
+// Any width.
 __global__ void __launch_bounds__(NORM_THREADS)
 rmsnorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows, const void* __restrict__ gain,
                int gain_is_f32, elem_t* __restrict__ out, int dim, float eps) {
@@ -59,12 +129,7 @@ rmsnorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows, co
     float v = src[i];
     ss = fmaf(v, v, ss);
   }
-  ss = wave_sum(ss);
-  if ((threadIdx.x & (AXON_WAVE - 1)) == 0) partial[threadIdx.x / AXON_WAVE] = ss;
-  __syncthreads();
-  float total = partial[0];
-#pragma unroll
-  for (int w = 1; w < NORM_THREADS / AXON_WAVE; ++w) total += partial[w];
+  const float total = block_sum_256(ss, partial);
   const float ms = total / (float)dim;
   const float inv = 1.0f / sqrtf(ms + eps);
   elem_t* dst = out + (size_t)r * dim;
@@ -78,8 +143,12 @@ extern "C" int axk_rmsnorm(const float* x, const int32_t* rows, const void* gain
                            int n_rows, int dim, float eps, void* stream) {
   AXK_REQUIRE(n_rows >= 0 && dim > 0, "rmsnorm: bad sizes rows=%d dim=%d", n_rows, dim);
   if (n_rows == 0) return 0;
-  rmsnorm_kernel<<<n_rows, NORM_THREADS, 0, (hipStream_t)stream>>>(x, rows, gain, gain_is_f32, (elem_t*)out, dim,
-                                                                  eps);
+  const bool vec = dim % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0;
+  if (vec)
+    rmsnorm_vec_kernel<<<n_rows, NORM_THREADS, 0, (hipStream_t)stream>>>(x, rows, gain, gain_is_f32, (elem_t*)out, dim,
+                                                                        eps);
+  else
+    rmsnorm_kernel<<<n_rows, NORM_THREADS, 0, (hipStream_t)stream>>>(x, rows, gain, gain_is_f32, (elem_t*)out, dim, eps);
   AXK_LAUNCH_CHECK("rmsnorm");
   return 0;
 }
@@ -174,10 +243,6 @@ extern "C" int axk_rope_kv_write(void* qkv, const float* table, const int32_t* p
 }
 
 // ---------------------------------------------------------------------------- SwiGLU
-// act = (g / (1 + exp(-g))) * u: divide, then multiply (src/vmath.rs:128-132;
-// src/cuda/prefill.cu:109-123).
-__device__ inline float swiglu1(float g, float u) { return __fmul_rn(__fdiv_rn(g, 1.0f + expf(-g)), u); }
-
 __global__ void swiglu_kernel(const elem_t* __restrict__ gate_up, elem_t* __restrict__ out, int n_ffn) {
   const int t = blockIdx.y;
   const int f = blockIdx.x * blockDim.x + threadIdx.x;

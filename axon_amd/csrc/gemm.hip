@@ -10,8 +10,6 @@
 #include "api.h"
 #include "common.h"
 
-enum { MODE_STORE = 0, MODE_ADD_F32 = 1, MODE_STORE_F32 = 2 };
-
 #define FMA_BN 64
 #define FMA_BK 16
 #define FMA_THREADS 256
@@ -37,7 +35,7 @@ __device__ inline void load4_guarded(const elem_t* __restrict__ p, int valid, bo
 
 // BM rows x 64 columns per block of 256 threads; thread (ty, tx) owns RM = BM / 16 rows and
 // 4 columns.  K is walked in steps of 16 through LDS; inside a step k ascends.
-template <int BM>
+template <int BM, bool GLU>
 __global__ void __launch_bounds__(FMA_THREADS)
 gemm_fma_kernel(const elem_t* __restrict__ x, int x_stride, const elem_t* __restrict__ w, const void* __restrict__ bias,
                 int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode, bool vec_x,
@@ -45,15 +43,19 @@ gemm_fma_kernel(const elem_t* __restrict__ x, int x_stride, const elem_t* __rest
   constexpr int RM = BM / 16;
   __shared__ float xs[FMA_BK][BM + 4];
   __shared__ float ws[FMA_BK][FMA_BN + 4];
+  __shared__ float us[GLU ? FMA_BK : 1][FMA_BN + 4];  // the up rows of the same columns (GLU: W holds 2 N rows)
   const int tid = threadIdx.x;
   const int tx = tid & 15, ty = tid >> 4;
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * FMA_BN;
 
-  float acc[RM][4];
+  float acc[RM][4], acc_up[GLU ? RM : 1][4];
 #pragma unroll
   for (int i = 0; i < RM; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.0f;
+    for (int j = 0; j < 4; ++j) {
+      acc[i][j] = 0.0f;
+      if (GLU) acc_up[i][j] = 0.0f;
+    }
 
   // loader: each thread brings 4 consecutive k of one row
   const int lrow = tid >> 2, lk = (tid & 3) * 4;
@@ -65,6 +67,11 @@ gemm_fma_kernel(const elem_t* __restrict__ x, int x_stride, const elem_t* __rest
       load4_guarded(w + (size_t)n * K + k0 + lk, valid > 0 ? valid : 0, vec_w, v);
 #pragma unroll
       for (int i = 0; i < 4; ++i) ws[lk + i][lrow] = v[i];
+      if (GLU) {
+        load4_guarded(w + (size_t)(N + n) * K + k0 + lk, valid > 0 ? valid : 0, vec_w, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) us[lk + i][lrow] = v[i];
+      }
     }
     if (lrow < BM) {
       float v[4];
@@ -86,6 +93,14 @@ gemm_fma_kernel(const elem_t* __restrict__ x, int x_stride, const elem_t* __rest
       for (int i = 0; i < RM; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+      if (GLU) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = us[kk][tx * 4 + j];
+#pragma unroll
+        for (int i = 0; i < RM; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc_up[i][j] = fmaf(a[i], b[j], acc_up[i][j]);
+      }
     }
     __syncthreads();
   }
@@ -101,7 +116,8 @@ gemm_fma_kernel(const elem_t* __restrict__ x, int x_stride, const elem_t* __rest
       float v = acc[i][j];
       if (bias) v += load_vec(bias, bias_is_f32, n);
       const size_t at = (size_t)m * out_stride + n;
-      if (mode == MODE_STORE) ((elem_t*)out)[at] = from_float(v);
+      if (GLU) ((elem_t*)out)[at] = from_float(swiglu1(v, acc_up[i][j]));
+      else if (mode == MODE_STORE) ((elem_t*)out)[at] = from_float(v);
       else if (mode == MODE_ADD_F32) ((float*)out)[at] += v;
       else ((float*)out)[at] = v;
     }
@@ -113,15 +129,15 @@ static int launch_fma(const elem_t* x, int x_stride, const elem_t* w, const void
   const size_t vbytes = 4 * sizeof(elem_t);
   const bool vec_w = (k % 4 == 0) && ((uintptr_t)w % vbytes == 0);
   const bool vec_x = (k % 4 == 0) && (x_stride % 4 == 0) && ((uintptr_t)x % vbytes == 0);
-  if (m <= 16) {
-    dim3 grid(ceil_div(n, FMA_BN), ceil_div(m, 16));
-    gemm_fma_kernel<16><<<grid, FMA_THREADS, 0, stream>>>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n,
-                                                          k, mode, vec_x, vec_w);
+#define FMA_LAUNCH(BM, GLU)                                                                                      \
+  gemm_fma_kernel<BM, GLU><<<dim3(ceil_div(n, FMA_BN), ceil_div(m, BM)), FMA_THREADS, 0, stream>>>(              \
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, vec_x, vec_w)
+  if (mode == MODE_SWIGLU) {
+    if (m <= 16) FMA_LAUNCH(16, true); else FMA_LAUNCH(64, true);
   } else {
-    dim3 grid(ceil_div(n, FMA_BN), ceil_div(m, 64));
-    gemm_fma_kernel<64><<<grid, FMA_THREADS, 0, stream>>>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n,
-                                                          k, mode, vec_x, vec_w);
+    if (m <= 16) FMA_LAUNCH(16, false); else FMA_LAUNCH(64, false);
   }
+#undef FMA_LAUNCH
   AXK_LAUNCH_CHECK("gemm_fma");
   return 0;
 }
@@ -136,7 +152,8 @@ extern "C" int axk_gemm(const void* x, int x_stride, const void* w, const void* 
   AXK_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
   AXK_REQUIRE(x_stride >= k && out_stride >= n, "gemm: strides x=%d (K=%d) out=%d (N=%d) too small", x_stride, k,
               out_stride, n);
-  AXK_REQUIRE(mode >= 0 && mode <= 2, "gemm: unknown mode %d", mode);
+  AXK_REQUIRE(mode >= 0 && mode <= 3, "gemm: unknown mode %d", mode);
+  AXK_REQUIRE(mode != MODE_SWIGLU || bias == nullptr, "gemm: the gated epilogue takes no bias");
   AXK_REQUIRE(ceil_div(m, 16) <= 65535, "gemm: M=%d is more rows than one launch takes", m);
   if (m == 0) return 0;
 #if AXON_BF16

@@ -11,17 +11,16 @@
 //   into different banks.  Blocks are numbered so that the blocks of one XCD (every eighth
 //   block) share weight tiles in that XCD's L2.
 //
-// * gemm_skinny (M <= 64, decoding): bound by reading W once.  A wave owns 16 or 32 rows of
-//   W, streams them from memory straight into MFMA fragments (16x16x32: a lane's 8
-//   consecutive k are one 16-byte load), multiplies with up to 64 rows of X, and the waves
-//   of a block split K between them; their partial sums are added in wave order through LDS.
-//   No atomics, so the result does not depend on timing.
+// * gemm_skinny (M <= 64, decoding): bound by reading W once.  A block owns 16 or 32 rows of
+//   W; its four waves split K between them and stream their share from memory straight into
+//   MFMA fragments (16x16x32: a lane's 8 consecutive k are one 16-byte load), keeping a ring
+//   of steps in flight so that the memory pipe never drains; each multiplies with up to 64
+//   rows of X, and the waves' partial sums are added in wave order through LDS.  No atomics,
+//   so the result does not depend on timing.
 //
 // The two kernels sum k in different groupings, so a row's bits differ between M <= 64 and
 // M > 64 by rounding (and only by rounding); within one kernel a row does not depend on the
 // other rows of the batch.
-#include <stdlib.h>
-
 #include "api.h"
 #include "common.h"
 
@@ -30,8 +29,6 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
-
-enum { MODE_STORE = 0, MODE_ADD_F32 = 1, MODE_STORE_F32 = 2 };
 
 #define TILE_BK 64
 #define TILE_ROW_BYTES 128  // one LDS row: 64 bf16, in eight 16-byte slots
@@ -51,7 +48,12 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // the eight 16-byte slots are permuted: slot p of row r holds k chunk p ^ (r & 7), so that the
 // fragment reads of 8 neighbouring rows at one k chunk hit 8 different slots (no bank
 // conflicts) without padding, which direct loads could not skip.
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+//
+// GLU: W holds 2 N rows (gate rows, then up rows) and the output is silu(gate) * up, N wide.
+// A block then owns BN / 2 output columns; each wave's share of the LDS tile holds the gate
+// rows of its columns and, after them, the up rows of the same columns, so that a lane ends
+// with both values of an output element.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const void* __restrict__ bias,
                  int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode, int m_blocks,
@@ -79,7 +81,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
     nb = (n_blocks / 8) * 8 + r / m_blocks;
     mb = r % m_blocks;
   }
-  const int m0 = mb * BM, n0 = nb * BN;
+  const int m0 = mb * BM, n0 = nb * (GLU ? BN / 2 : BN);
 
   // what this lane fetches: row (q * NW + wave) * 8 + lane / 8 of a tile, k chunk (lane % 8) ^ (lane / 8)
   const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
@@ -88,8 +90,18 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   for (int q = 0; q < XQ; ++q)
     xoff[q] = (unsigned)min(m0 + (q * NW + wave) * 8 + lrow, M - 1) * (unsigned)x_stride + lchunk * 8;
 #pragma unroll
-  for (int q = 0; q < WQ; ++q)
-    woff[q] = (unsigned)min(n0 + (q * NW + wave) * 8 + lrow, N - 1) * (unsigned)K + lchunk * 8;
+  for (int q = 0; q < WQ; ++q) {
+    const int r = (q * NW + wave) * 8 + lrow;  // row of the LDS tile
+    int grow;
+    if (GLU) {
+      const int owner = r / WN, within = r % WN;             // the wave whose columns these are
+      const int col = n0 + owner * (WN / 2) + within % (WN / 2);
+      grow = (within >= WN / 2 ? N : 0) + min(col, N - 1);   // up rows follow the N gate rows
+    } else {
+      grow = min(n0 + r, N - 1);
+    }
+    woff[q] = (unsigned)grow * (unsigned)K + lchunk * 8;
+  }
 
   auto issue = [&](int kt) {
     unsigned char* stage = smem + (kt & 1) * STAGE;
@@ -163,6 +175,24 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   }
 
   // epilogue: lane holds column n = lane % 32 of each tile and rows (e/4)*8 + (lane/32)*4 + e%4
+  if (GLU) {
+#pragma unroll
+    for (int j = 0; j < TN / 2; ++j) {
+      const int n = n0 + wn * (WN / 2) + j * 32 + (lane & 31);
+      if (n >= N) continue;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          if (m >= M) continue;
+          reinterpret_cast<bf16_t*>(out)[(size_t)m * out_stride + n] =
+              float_to_bf16(swiglu1(acc[i][j][e], acc[i][j + TN / 2][e]));
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int n = n0 + wn * WN + j * 32 + (lane & 31);
@@ -184,13 +214,13 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU>
 static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                        int out_stride, int m, int n, int k, int mode, hipStream_t stream) {
   static bool configured = false;
   constexpr int lds_bytes = 2 * (BM + BN) * TILE_ROW_BYTES;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, GLU>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) {
       axk_set_error("gemm_tile: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
@@ -198,8 +228,8 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
     }
     configured = true;
   }
-  const int m_blocks = ceil_div(m, BM), n_blocks = ceil_div(n, BN);
-  gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N><<<m_blocks * n_blocks, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
+  const int m_blocks = ceil_div(m, BM), n_blocks = ceil_div(n, GLU ? BN / 2 : BN);
+  gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, GLU><<<m_blocks * n_blocks, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks);
   AXK_LAUNCH_CHECK("gemm_tile");
   return 0;
@@ -210,19 +240,24 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
 // ...  C[n][m] tiles of 16 x 16: the MFMA's A operand is W (lane: row n = lane % 16, 8
 // consecutive k from (lane / 16) * 8), its B operand X (lane: row m = lane % 16, the same k).
 // A lane ends with 4 consecutive n of one m: one vector store.
-template <int NT16, int MT16, int WAVES>
+// GLU (NT16 = 2): the block's two tiles are the gate rows n0 .. n0 + 15 and the up rows of the
+// same columns (W holds 2 N rows), and the output is silu(gate) * up.
+template <int NT16, int MT16, int WAVES, int DEPTH, bool GLU>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w,
                    const void* __restrict__ bias, int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N,
                    int K, int mode) {
   __shared__ float partial[WAVES][NT16 * MT16][64][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * NT16 * 16;
+  const int n0 = blockIdx.x * (GLU ? 16 : NT16 * 16);
   const int r16 = lane & 15, kq = (lane >> 4) * 8;
 
   const bf16_t* wrow[NT16];
 #pragma unroll
-  for (int i = 0; i < NT16; ++i) wrow[i] = w + (size_t)min(n0 + i * 16 + r16, N - 1) * K + kq;
+  for (int i = 0; i < NT16; ++i) {
+    const int row = GLU ? i * N + min(n0 + r16, N - 1) : min(n0 + i * 16 + r16, N - 1);
+    wrow[i] = w + (size_t)row * K + kq;
+  }
   const bf16_t* xrow[MT16];
 #pragma unroll
   for (int j = 0; j < MT16; ++j) xrow[j] = x + (size_t)min(j * 16 + r16, M - 1) * x_stride + kq;
@@ -233,50 +268,56 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
 #pragma unroll
     for (int j = 0; j < MT16; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
+  // This wave's steps (64 k each): wave, wave + WAVES, ...  A ring of DEPTH steps is kept in
+  // flight: a step is multiplied as soon as ITS loads have landed (loads return in order), and
+  // its place in the ring is refilled at once, so the memory pipe never drains.
   const int steps = K / 64;
-  constexpr int UNROLL = 4;
-  int s = wave;
-  for (; s + (UNROLL - 1) * WAVES < steps; s += UNROLL * WAVES) {
-    uint4 wf[UNROLL][NT16][2], xf[UNROLL][MT16][2];
+  const int mine = steps > wave ? (steps - wave + WAVES - 1) / WAVES : 0;
+  uint4 wf[DEPTH][NT16][2], xf[DEPTH][MT16][2];
+  auto load = [&](int slot, int local) {
+    const int k0 = (wave + local * WAVES) * 64;
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int k0 = (s + u * WAVES) * 64;
-#pragma unroll
-      for (int i = 0; i < NT16; ++i) {
-        wf[u][i][0] = *reinterpret_cast<const uint4*>(wrow[i] + k0);
-        wf[u][i][1] = *reinterpret_cast<const uint4*>(wrow[i] + k0 + 32);
-      }
-#pragma unroll
-      for (int j = 0; j < MT16; ++j) {
-        xf[u][j][0] = *reinterpret_cast<const uint4*>(xrow[j] + k0);
-        xf[u][j][1] = *reinterpret_cast<const uint4*>(xrow[j] + k0 + 32);
-      }
+    for (int i = 0; i < NT16; ++i) {
+      wf[slot][i][0] = *reinterpret_cast<const uint4*>(wrow[i] + k0);
+      wf[slot][i][1] = *reinterpret_cast<const uint4*>(wrow[i] + k0 + 32);
     }
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+    for (int j = 0; j < MT16; ++j) {
+      xf[slot][j][0] = *reinterpret_cast<const uint4*>(xrow[j] + k0);
+      xf[slot][j][1] = *reinterpret_cast<const uint4*>(xrow[j] + k0 + 32);
+    }
+  };
+  auto multiply = [&](int slot) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
-#pragma unroll
-        for (int i = 0; i < NT16; ++i)
-#pragma unroll
-          for (int j = 0; j < MT16; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[u][i][h]), as_frag(xf[u][j][h]), acc[i][j], 0, 0, 0);
-  }
-  for (; s < steps; s += WAVES) {
-    const int k0 = s * 64;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      uint4 wf[NT16], xf[MT16];
-#pragma unroll
-      for (int i = 0; i < NT16; ++i) wf[i] = *reinterpret_cast<const uint4*>(wrow[i] + k0 + h * 32);
-#pragma unroll
-      for (int j = 0; j < MT16; ++j) xf[j] = *reinterpret_cast<const uint4*>(xrow[j] + k0 + h * 32);
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int i = 0; i < NT16; ++i)
 #pragma unroll
         for (int j = 0; j < MT16; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[i]), as_frag(xf[j]), acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[slot][i][h]), as_frag(xf[slot][j][h]), acc[i][j],
+                                                              0, 0, 0);
+  };
+
+  if (mine > 0) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) load(d, min(d, mine - 1));   // beyond this wave's steps: a valid step again
+    int base = 0;  // the ring holds local steps base .. base + DEPTH - 1
+    for (; base + 2 * DEPTH <= mine; base += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        multiply(d);
+        load(d, base + DEPTH + d);
+      }
     }
+    // the tail: what the ring holds, refilled only where a step is left, then those
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (base + d < mine) multiply(d);
+      if (base + DEPTH + d < mine) load(d, base + DEPTH + d);
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+      if (base + DEPTH + d < mine) multiply(d);
   }
 
 #pragma unroll
@@ -287,6 +328,26 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
       for (int e = 0; e < 4; ++e) partial[wave][i * MT16 + j][lane][e] = acc[i][j][e];
   __syncthreads();
 
+  if (GLU) {
+    // a wave takes both tiles of a column block: gate (tile j) and up (tile MT16 + j)
+    for (int j = wave; j < MT16; j += WAVES) {
+      const int m = j * 16 + r16;
+      const int n = n0 + (lane >> 4) * 4;
+      if (m >= M) continue;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (n + e >= N) continue;
+        float g = partial[0][j][lane][e], u = partial[0][MT16 + j][lane][e];
+#pragma unroll
+        for (int q = 1; q < WAVES; ++q) {
+          g += partial[q][j][lane][e];
+          u += partial[q][MT16 + j][lane][e];
+        }
+        reinterpret_cast<bf16_t*>(out)[(size_t)m * out_stride + n + e] = float_to_bf16(swiglu1(g, u));
+      }
+    }
+    return;
+  }
   // tiles are shared out between the waves; each sums the partials in wave order
   for (int t = wave; t < NT16 * MT16; t += WAVES) {
     const int i = t / MT16, j = t % MT16;
@@ -314,10 +375,10 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
   }
 }
 
-template <int NT16, int MT16, int WAVES>
+template <int NT16, int MT16, int WAVES, int DEPTH, bool GLU = false>
 static int launch_skinny(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                          int out_stride, int m, int n, int k, int mode, hipStream_t stream) {
-  gemm_skinny_kernel<NT16, MT16, WAVES><<<ceil_div(n, NT16 * 16), WAVES * 64, 0, stream>>>(
+  gemm_skinny_kernel<NT16, MT16, WAVES, DEPTH, GLU><<<ceil_div(n, GLU ? 16 : NT16 * 16), WAVES * 64, 0, stream>>>(
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode);
   AXK_LAUNCH_CHECK("gemm_skinny");
   return 0;
@@ -331,33 +392,31 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
   if (k % 64 != 0 || x_stride % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return 0;
   *handled = true;
 #define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream
+  if (m <= 64 && mode == MODE_SWIGLU) {
+    if (m <= 16) return launch_skinny<2, 1, 4, 8, true>(ARGS);
+    if (m <= 32) return launch_skinny<2, 2, 4, 4, true>(ARGS);
+    return launch_skinny<2, 4, 4, 2, true>(ARGS);
+  }
   if (m <= 64) {
-    // wide outputs: 32 rows of W per wave and 4 waves; narrow ones: 16 rows and 8 waves, so that
-    // enough waves stream the weights
-    const bool wide = n >= 16384;
-    if (m <= 16) return wide ? launch_skinny<2, 1, 4>(ARGS) : launch_skinny<1, 1, 8>(ARGS);
-    if (m <= 32) return wide ? launch_skinny<2, 2, 4>(ARGS) : launch_skinny<1, 2, 8>(ARGS);
-    return wide ? launch_skinny<2, 4, 4>(ARGS) : launch_skinny<1, 4, 8>(ARGS);
+    // 32 rows of W per block where that still leaves 128 blocks or more, else 16; four waves
+    // split K; the ring is as deep as the registers allow
+    const bool wide = n >= 32 * 128;
+    if (m <= 16) return wide ? launch_skinny<2, 1, 4, 8>(ARGS) : launch_skinny<1, 1, 4, 8>(ARGS);
+    if (m <= 32) return wide ? launch_skinny<2, 2, 4, 4>(ARGS) : launch_skinny<1, 2, 4, 8>(ARGS);
+    return wide ? launch_skinny<2, 4, 4, 2>(ARGS) : launch_skinny<1, 4, 4, 4>(ARGS);
   }
   // offsets inside the kernels are 32-bit element counts
-  if ((size_t)n * k >= (1ull << 32) || (size_t)m * x_stride >= (1ull << 32)) {
+  if ((size_t)n * k * (mode == MODE_SWIGLU ? 2 : 1) >= (1ull << 32) || (size_t)m * x_stride >= (1ull << 32)) {
     *handled = false;
     return 0;
   }
-  static const int forced = getenv("AXON_GEMM_TILE") ? atoi(getenv("AXON_GEMM_TILE")) : 0;
-  switch (forced) {
-    case 1: return launch_tile<256, 256, 2, 2>(ARGS);
-    case 2: return launch_tile<256, 256, 2, 4>(ARGS);
-    case 3: return launch_tile<128, 256, 2, 2>(ARGS);
-    case 4: return launch_tile<128, 128, 2, 2>(ARGS);
-    case 5: return launch_tile<256, 256, 4, 2>(ARGS);
-    case 6: return launch_tile<256, 128, 2, 2>(ARGS);
-    case 7: return launch_tile<128, 256, 1, 4>(ARGS);
-    default: break;
-  }
   // 256 x 256 tiles (8 waves) when they still give every CU two blocks; else 128 x 128
-  if ((long)ceil_div(m, 256) * ceil_div(n, 256) >= 512) return launch_tile<256, 256, 4, 2>(ARGS);
-  return launch_tile<128, 128, 2, 2>(ARGS);
+  if (mode == MODE_SWIGLU) {
+    if ((long)ceil_div(m, 256) * ceil_div(n, 128) >= 512) return launch_tile<256, 256, 4, 2, true>(ARGS);
+    return launch_tile<128, 128, 2, 2, true>(ARGS);
+  }
+  if ((long)ceil_div(m, 256) * ceil_div(n, 256) >= 512) return launch_tile<256, 256, 4, 2, false>(ARGS);
+  return launch_tile<128, 128, 2, 2, false>(ARGS);
 #undef ARGS
 }
 

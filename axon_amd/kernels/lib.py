@@ -15,7 +15,7 @@ import torch
 
 from . import build
 
-MODE_STORE, MODE_ADD_F32, MODE_STORE_F32 = 0, 1, 2
+MODE_STORE, MODE_ADD_F32, MODE_STORE_F32, MODE_SWIGLU = 0, 1, 2, 3
 
 
 class KernelError(RuntimeError):
@@ -220,15 +220,20 @@ class Kernels:
 
     def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
              mode: int = MODE_STORE) -> torch.Tensor:
-        """out = epilogue(x . w^T + bias); x [M, K] (rows may be strided), w [N, K] contiguous."""
+        """out = epilogue(x . w^T + bias); x [M, K] (rows may be strided), w [N, K] contiguous.
+        MODE_SWIGLU: w is [2 N, K], gate rows then up rows; out [M, N] = silu(x gate^T) * (x up^T)."""
         self._elem(x, "gemm x"); self._elem(w, "gemm w")
         M, K = x.shape
         N = w.shape[0]
+        if mode == MODE_SWIGLU:
+            if N % 2 or bias is not None:
+                raise KernelError("gemm: the gated epilogue needs gate and up rows and takes no bias")
+            N //= 2
         if w.shape[1] != K or not w.is_contiguous() or x.stride(1) != 1 or out.stride(1) != 1:
             raise KernelError(f"gemm: x {tuple(x.shape)} w {tuple(w.shape)} do not multiply, or are not row-major")
         if out.shape != (M, N) or not out.is_cuda:
             raise KernelError(f"gemm: out {tuple(out.shape)} is not [{M}, {N}]")
-        want = self.dtype if mode == MODE_STORE else torch.float32
+        want = self.dtype if mode in (MODE_STORE, MODE_SWIGLU) else torch.float32
         if out.dtype != want:
             raise KernelError(f"gemm: mode {mode} writes {want}, out is {out.dtype}")
         if bias is not None and bias.numel() != N:

@@ -25,7 +25,7 @@ from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, build_part, regist
 
 
 PREFILL_TILE = 128     # tokens of one request per tile of the prompt kernel
-DECODE_CHUNK = 256     # positions per chunk of the decoding kernel
+DECODE_CHUNK = 64      # positions per chunk of the decoding kernel
 DECODE_BLOCK = 64
 
 
@@ -67,7 +67,7 @@ class AttentionPlan:
 
 
 def decode_chunks_of(pos: int, window: int) -> int:
-    """Chunks of 256 positions the decoding kernel cuts a token's range into."""
+    """Chunks of 64 positions the decoding kernel cuts a token's range into."""
     lo = max(0, pos + 1 - window) if window > 0 else 0
     return (pos - lo // DECODE_BLOCK * DECODE_BLOCK) // DECODE_CHUNK + 1
 
@@ -123,7 +123,7 @@ class GQAttention(Mixer):
         return CacheSpec(entries=2, heads=self.nkv, head_dim=self.hd, window=self.window)
 
     def decode_shape(self, positions):
-        """The decoding kernel's grid depends on the longest context, in chunks of 256 positions,
+        """The decoding kernel's grid depends on the longest context, in chunks of 64 positions,
         rounded up to a power of two so that few shapes exist."""
         most = max(decode_chunks_of(p, self.window) for p in positions)
         return ("attention_chunks", self.window), 1 << (most - 1).bit_length()

@@ -1,14 +1,15 @@
 """The dense SwiGLU feed-forward: down(silu(gate h) * up h), added to the residual stream.
 
 act = (g / (1 + exp(-g))) * u (src/vmath.rs:128-132), no biases (src/model.rs:3043-3055).
-gate and up run as one product over a fused [2 ffn, hidden] matrix.  Parameters:
+gate and up run as one product over a fused [2 ffn, hidden] matrix whose epilogue applies the
+activation, so the two halves never travel through memory.  Parameters:
 `hidden_size`, `intermediate_size`.
 """
 from __future__ import annotations
 
 from typing import List
 
-from ..kernels import MODE_ADD_F32, MODE_STORE
+from ..kernels import MODE_ADD_F32, MODE_SWIGLU
 from .base import FeedForward, TensorDecl, register_feed_forward
 
 
@@ -35,10 +36,8 @@ class SwiGLUMLP(FeedForward):
         k = ctx.rt.k
         T = h.shape[0]
         mark = ctx.ws.mark()
-        gate_up = ctx.ws.take((T, 2 * self.ffn), ctx.rt.dtype)
-        k.gemm(h, self.w_gate_up, gate_up, None, MODE_STORE)
         act = ctx.ws.take((T, self.ffn), ctx.rt.dtype)
-        k.swiglu(gate_up, act)
+        k.gemm(h, self.w_gate_up, act, None, MODE_SWIGLU)      # silu(gate h) * up h, in the product's epilogue
         k.gemm(act, self.w_down, residual, None, MODE_ADD_F32)
         ctx.ws.release(mark)
 

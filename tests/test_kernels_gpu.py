@@ -6,7 +6,7 @@ import math
 import pytest
 import torch
 
-from axon_amd.kernels import MODE_ADD_F32, MODE_STORE, MODE_STORE_F32, KernelError, kernels
+from axon_amd.kernels import MODE_ADD_F32, MODE_STORE, MODE_STORE_F32, MODE_SWIGLU, KernelError, kernels
 from gpu_helpers import DTYPES, TORCH, paged_cache, tol
 from plain import qwen2_plain as P
 
@@ -181,6 +181,22 @@ def test_gemm_every_epilogue(dtype, M, N, K):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,F,K", [(1, 96, 64), (9, 176, 64), (40, 320, 192), (64, 130, 128), (70, 300, 128),
+                                   (300, 512, 256), (600, 1000, 128), (5, 100, 70), (33, 19, 33), (2100, 384, 64)])
+def test_gemm_with_the_gated_epilogue(dtype, M, F, K):
+    """One product over [gate; up] whose epilogue is silu(gate) * up."""
+    k = kernels(dtype)
+    x, xr = as_dtype(rnd(M, K, seed=30), dtype)
+    w, wr = as_dtype(rnd(2 * F, K, seed=31, scale=0.3), dtype)
+    out = torch.empty(M, F, dtype=TORCH[dtype], device="cuda")
+    k.gemm(x, w, out, None, MODE_SWIGLU)
+    ref = P.swiglu(xr @ wr[:F].T, xr @ wr[F:].T)
+    assert (out.cpu().double() - ref).abs().max() <= tol(dtype, ref, 2e-6 * math.sqrt(K), 1e-2)
+    with pytest.raises(KernelError):
+        k.gemm(x, w, out, rnd(F).cuda(), MODE_SWIGLU)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_rows_do_not_depend_on_the_batch(dtype):
     """The same row of x gives the same bits whatever rows ride along.  float32: for any number
     of rows.  bfloat16: among batches of up to 64 rows (the decoding kernel) and among larger
@@ -318,9 +334,7 @@ def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
     # single tokens at chosen positions: first, block and chunk edges, last
     picks = sorted({0, 1, 15, 16, 63, 64, 65, 255, 256, 257, 511, 512, T // 2, T - 2, T - 1} & set(range(T)))
     idx = torch.tensor(picks, dtype=torch.int32).cuda()
-    lo = max(0, max(picks) + 1 - window) if window else 0
-    chunks = (max(picks) - lo // 64 * 64) // 256 + 1 if window == 0 else max(
-        (p - (max(0, p + 1 - window) // 64 * 64)) // 256 + 1 for p in picks)
+    chunks = max((p - ((max(0, p + 1 - window) if window else 0) // 64 * 64)) // 64 + 1 for p in picks)
     partial = torch.empty(k.attention_decode_workspace(len(picks), nh, hd, chunks), dtype=torch.float32, device="cuda")
     out = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
     k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, out, idx, partial, chunks, nh, nkv, hd, page, window, scale)
@@ -356,13 +370,13 @@ def test_matrix_core_attention_finds_a_far_key_and_respects_the_windows_edge():
     scale = 1.0 / math.sqrt(hd)
     one = torch.tensor([T - 1], dtype=torch.int32).cuda()
     tile = torch.tensor([[T - 40, 40]], dtype=torch.int32).cuda()
-    partial = torch.empty(k.attention_decode_workspace(1, nh, hd, 4), dtype=torch.float32, device="cuda")
+    partial = torch.empty(k.attention_decode_workspace(1, nh, hd, 16), dtype=torch.float32, device="cuda")
     for w, seen in ((0, True), (T - 1 - far, False), (T - far, True)):
         ref = P.causal_attention(qr, kr, vr, w)[T - 1]
         for which in ("decode", "prefill"):
             out = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
             if which == "decode":
-                k.attention_decode(qd.view(T, -1), nh * hd, kc, vc, table, pos, rows, out, one, partial, 4, nh, nkv, hd,
+                k.attention_decode(qd.view(T, -1), nh * hd, kc, vc, table, pos, rows, out, one, partial, 16, nh, nkv, hd,
                                    page, w, scale)
             else:
                 k.attention_prefill(qd.view(T, -1), nh * hd, kc, vc, table, pos, rows, out, tile, nh, nkv, hd, page, w, scale)
