@@ -41,9 +41,7 @@ __device__ inline bf16x8 frag_of2(uint2 lo, uint2 hi) {
   return c.f;
 }
 
-__device__ inline uint32_t pack_bf16(float a, float b) {
-  return (uint32_t)float_to_bf16(a).bits | ((uint32_t)float_to_bf16(b).bits << 16);
-}
+__device__ inline uint32_t pack_bf16(float a, float b) { return pack2_bf16(a, b); }
 
 // ============================================================================ prompt portions
 // grid (tiles, query heads); a tile is up to 128 consecutive tokens of one request.  4 waves,
@@ -88,6 +86,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
   const int my_pos = pos0 + min(my_row, count - 1);
   const int my_lo = window > 0 ? max(0, my_pos + 1 - window) : 0;
   const int wave_hi = pos0 + min(wave * 32 + 31, count - 1);     // last position this wave's rows see
+  const int wave_lo = window > 0 ? max(0, wave_hi + 1 - window) : 0;  // the latest window start among them
   const bool wave_live = wave * 32 < count;
 
   // Q^T fragments (B operand): column = query row, 8 consecutive dims from 16 ks + 8 half
@@ -172,18 +171,32 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
         s_acc[pt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s_acc[pt], 0, 0, 0);
       }
     }
-    // this lane: query my_row; positions p0 + pt*32 + (e/4)*8 + half*4 + e%4
+    // this lane: query my_row; positions p0 + pt*32 + (e/4)*8 + half*4 + e%4.  A block that every
+    // row of the wave sees whole needs no mask (all but the blocks on the diagonal and at the
+    // window's edge).
+    const bool whole = p0 + PF_BLOCK - 1 <= pos0 + wave * 32 && p0 >= wave_lo;
     float mloc = -INFINITY;
+    if (whole) {
 #pragma unroll
-    for (int pt = 0; pt < 2; ++pt)
+      for (int pt = 0; pt < 2; ++pt)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int p = p0 + pt * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
-        const bool seen = p <= my_pos && p >= my_lo;
-        const float v = seen ? s_acc[pt][e] * c : -INFINITY;
-        s_acc[pt][e] = v;
-        mloc = fmaxf(mloc, v);
-      }
+        for (int e = 0; e < 16; ++e) {
+          const float v = s_acc[pt][e] * c;
+          s_acc[pt][e] = v;
+          mloc = fmaxf(mloc, v);
+        }
+    } else {
+#pragma unroll
+      for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int p = p0 + pt * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+          const bool seen = p <= my_pos && p >= my_lo;
+          const float v = seen ? s_acc[pt][e] * c : -INFINITY;
+          s_acc[pt][e] = v;
+          mloc = fmaxf(mloc, v);
+        }
+    }
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32, AXON_WAVE));
     const float mn = fmaxf(m_run, mloc);
     const float mref = mn == -INFINITY ? 0.0f : mn;     // a row that has seen nothing yet
@@ -200,10 +213,12 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
     lsum += __shfl_xor(lsum, 32, AXON_WAVE);
     l_run = l_run * alpha + lsum;
     m_run = mn;
+    if (__any(alpha != 1.0f)) {  // the running maximum moved for some row: rescale what is summed so far
 #pragma unroll
-    for (int i = 0; i < DT; ++i)
+      for (int i = 0; i < DT; ++i)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+        for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
+    }
 
     // O^T [HD][32 queries] += V^T P^T.  k step s2 (16 positions) takes registers e = 8 (s2 % 2) ..
     // + 7 of tile s2 / 2: positions (s2/2)*32 + (s2%2)*16 + half*4 + {0..3} and the same + 8.

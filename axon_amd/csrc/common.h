@@ -26,11 +26,16 @@ __host__ __device__ inline float bf16_to_float(bf16_t v) {
   return c.f;
 }
 
-// Round to nearest, ties to even; NaN stays NaN (quiet).
+// Round to nearest, ties to even; NaN stays NaN (quiet).  On the device this is the hardware's
+// conversion (one instruction on gfx950); the host version does the same in integer arithmetic.
 __host__ __device__ inline bf16_t float_to_bf16(float f) {
+  bf16_t r;
+#if defined(__HIP_DEVICE_COMPILE__)
+  const __bf16 h = (__bf16)f;
+  __builtin_memcpy(&r.bits, &h, sizeof r.bits);
+#else
   union { uint32_t u; float f; } c;
   c.f = f;
-  bf16_t r;
   if ((c.u & 0x7fffffffu) > 0x7f800000u) {
     r.bits = (uint16_t)((c.u >> 16) | 0x0040u);
     return r;
@@ -38,6 +43,18 @@ __host__ __device__ inline bf16_t float_to_bf16(float f) {
   uint32_t lsb = (c.u >> 16) & 1u;
   c.u += 0x7fffu + lsb;
   r.bits = (uint16_t)(c.u >> 16);
+#endif
+  return r;
+}
+
+// Two floats to a packed pair of bfloat16 (low half first).
+__device__ inline uint32_t pack2_bf16(float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  const f32x2_t v = {a, b};
+  const bf16x2_t h = __builtin_convertvector(v, bf16x2_t);
+  uint32_t r;
+  __builtin_memcpy(&r, &h, sizeof r);
   return r;
 }
 

@@ -403,6 +403,8 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
     const bool wide = n >= 32 * 128;
     if (m <= 16) return wide ? launch_skinny<2, 1, 4, 8>(ARGS) : launch_skinny<1, 1, 4, 8>(ARGS);
     if (m <= 32) return wide ? launch_skinny<2, 2, 4, 4>(ARGS) : launch_skinny<1, 2, 4, 8>(ARGS);
+    // a very wide output (the head) with more than 32 rows: the tiled kernel shares X through LDS
+    if (n >= 65536 && mode != MODE_SWIGLU && (size_t)n * k < (1ull << 32)) return launch_tile<128, 128, 2, 2, false>(ARGS);
     return wide ? launch_skinny<2, 4, 4, 2>(ARGS) : launch_skinny<1, 4, 4, 4>(ARGS);
   }
   // offsets inside the kernels are 32-bit element counts
