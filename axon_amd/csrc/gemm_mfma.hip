@@ -32,6 +32,10 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 #define TILE_BK 64
 #define TILE_ROW_BYTES 128  // one LDS row: 64 bf16, in eight 16-byte slots
+// The permutation of a row's slots.  LDS serves 256 bytes a cycle (64 banks): a 16-byte read of
+// 16 consecutive lanes (16 consecutive rows, the same k chunk) is conflict-free when the 16
+// (row parity, slot) pairs differ, which slot = chunk ^ ((row >> 1) & 7) gives.
+#define SWZ(row) (((row) >> 1) & 7)
 
 __device__ inline bf16x8 as_frag(uint4 v) {
   union { uint4 u; bf16x8 f; } c;
@@ -45,9 +49,9 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // ---------------------------------------------------------------------------- gemm_tile
 // LDS holds, per stage, BM rows of X and BN rows of W, 64 k each, written by direct
 // global -> LDS loads of 16 bytes per lane (a wave instruction fills 8 rows).  Within a row
-// the eight 16-byte slots are permuted: slot p of row r holds k chunk p ^ (r & 7), so that the
-// fragment reads of 8 neighbouring rows at one k chunk hit 8 different slots (no bank
-// conflicts) without padding, which direct loads could not skip.
+// the eight 16-byte slots are permuted (see SWZ) so that the fragment reads of neighbouring
+// rows at one k chunk fall into different banks without padding, which direct loads could
+// not skip.
 //
 // GLU: W holds 2 N rows (gate rows, then up rows) and the output is silu(gate) * up, N wide.
 // A block then owns BN / 2 output columns; each wave's share of the LDS tile holds the gate
@@ -83,15 +87,19 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   }
   const int m0 = mb * BM, n0 = nb * (GLU ? BN / 2 : BN);
 
-  // what this lane fetches: row (q * NW + wave) * 8 + lane / 8 of a tile, k chunk (lane % 8) ^ (lane / 8)
-  const int lrow = lane >> 3, lchunk = (lane & 7) ^ lrow;
+  // what this lane fetches: row r = (q * NW + wave) * 8 + lane / 8 of a tile; it fills slot lane % 8
+  // of that row, which holds k chunk (lane % 8) ^ SWZ(r)
+  const int lrow = lane >> 3;
   unsigned xoff[XQ], woff[WQ];
 #pragma unroll
-  for (int q = 0; q < XQ; ++q)
-    xoff[q] = (unsigned)min(m0 + (q * NW + wave) * 8 + lrow, M - 1) * (unsigned)x_stride + lchunk * 8;
+  for (int q = 0; q < XQ; ++q) {
+    const int r = (q * NW + wave) * 8 + lrow;
+    xoff[q] = (unsigned)min(m0 + r, M - 1) * (unsigned)x_stride + ((lane & 7) ^ SWZ(r)) * 8;
+  }
 #pragma unroll
   for (int q = 0; q < WQ; ++q) {
     const int r = (q * NW + wave) * 8 + lrow;  // row of the LDS tile
+    const int lchunk = (lane & 7) ^ SWZ(r);
     int grow;
     if (GLU) {
       const int owner = r / WN, within = r % WN;             // the wave whose columns these are
@@ -125,7 +133,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // fragment addresses: row = tile row + lane % 32, k chunk = 2 ks + lane / 32, slot = chunk ^ (row & 7)
-  const int frow = lane & 31, fhalf = lane >> 5, fsw = lane & 7;
+  const int frow = lane & 31, fhalf = lane >> 5, fsw = SWZ(frow);
   const int xbase = (wm * WM + frow) * TILE_ROW_BYTES;
   const int wbase = (BM + wn * WN + frow) * TILE_ROW_BYTES;
 

@@ -37,6 +37,8 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=2048, help="prompt tokens of every request")
     ap.add_argument("--dtype", default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
+                    help="for profiling: time only the prefill step (repeated --steps times) or only decoding")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py runs on one GPU: this engine has no multi-GPU path (asked for {args.gpus})")
@@ -70,10 +72,12 @@ def main() -> int:
     p = prompt()
     eng.step([StepEntry("warm", p, [len(p) - 1])], end=["warm"])
     torch.cuda.synchronize()
+    reps = args.steps if args.phase == "prefill" else 1
     t0 = time.perf_counter()
-    eng.step([StepEntry("pf", p, [len(p) - 1])], end=["pf"])
+    for _ in range(reps):
+        eng.step([StepEntry("pf", p, [len(p) - 1])], end=["pf"])
     torch.cuda.synchronize()
-    prefill_s = time.perf_counter() - t0
+    prefill_s = (time.perf_counter() - t0) / reps
     T = len(p)
     per_layer = 2 * T * dim * ((nh + 2 * nkv) * hd + nh * hd + 3 * ffn) + 4 * nh * hd * T * (T + 1) / 2
     prefill_flops = L * per_layer + 2 * dim * V
@@ -109,9 +113,12 @@ def main() -> int:
         kv_bytes = batch * mid_ctx * L * 2 * nkv * hd * elem
         return batch * steps / dt, dt / steps, weight_bytes + kv_bytes
 
+    if args.phase == "prefill":
+        print(json.dumps({"phase": "prefill", "prefill": prefill, "layers": L}))
+        return 0
     tok_s, step_s, bytes_read = decode(args.batch, args.steps, args.warmup)
     points = {}
-    if not args.no_points:
+    if not args.no_points and args.phase == "all":
         for b in (1, 64):
             if b == args.batch:
                 points[f"decode_b{b}"] = round(tok_s, 1)
@@ -119,7 +126,7 @@ def main() -> int:
                 points[f"decode_b{b}"] = round(decode(b, max(8, args.steps // 2), args.warmup)[0], 1)
     achieved = bytes_read / step_s / 1e9
     line = {
-        "metric": "decode tok/s (Qwen2.5-7B sizes, bf16, batch 8, 2048-token prompts)",
+        "metric": f"decode tok/s (Qwen2.5-7B sizes, {args.dtype}, batch {args.batch}, {args.prompt}-token prompts)",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
