@@ -30,13 +30,6 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-#define TILE_BK 64
-#define TILE_ROW_BYTES 128  // one LDS row: 64 bf16, in eight 16-byte slots
-// The permutation of a row's slots.  LDS serves 256 bytes a cycle (64 banks): a 16-byte read of
-// 16 consecutive lanes (16 consecutive rows, the same k chunk) is conflict-free when the 16
-// (row parity, slot) pairs differ, which slot = chunk ^ ((row >> 1) & 7) gives.
-#define SWZ(row) (((row) >> 1) & 7)
-
 __device__ inline bf16x8 as_frag(uint4 v) {
   union { uint4 u; bf16x8 f; } c;
   c.u = v;
@@ -46,28 +39,45 @@ __device__ inline bf16x8 as_frag(uint4 v) {
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+template <int N>
+__device__ inline void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
 // ---------------------------------------------------------------------------- gemm_tile
-// LDS holds, per stage, BM rows of X and BN rows of W, 64 k each, written by direct
-// global -> LDS loads of 16 bytes per lane (a wave instruction fills 8 rows).  Within a row
-// the eight 16-byte slots are permuted (see SWZ) so that the fragment reads of neighbouring
-// rows at one k chunk fall into different banks without padding, which direct loads could
-// not skip.
+// LDS holds STAGES stages; a stage is BM rows of X and BN rows of W, BK k each, written by
+// direct global -> LDS loads of 16 bytes per lane (a wave instruction fills 1024 bytes of
+// consecutive rows).  The loads of step kt + STAGES - 1 are issued while step kt is multiplied,
+// so the latency of L2 and of the path into LDS is covered by STAGES - 1 steps of MFMAs.
+//
+// A row of a stage is BK / 8 slots of 16 bytes, permuted so that fragment reads of neighbouring
+// rows at one k chunk fall into different banks without padding (which direct loads could
+// not skip).  LDS serves 256 bytes a cycle (64 banks): a 16-byte read of 16 consecutive lanes
+// (16 consecutive rows, the same k chunk) is conflict-free when the rows' 16-byte positions
+// modulo 256 differ.  With 128-byte rows (BK 64) that is slot = chunk ^ ((row >> 1) & 7); with
+// 64-byte rows (BK 32) slot = chunk ^ ((row >> 2) & 3).
 //
 // GLU: W holds 2 N rows (gate rows, then up rows) and the output is silu(gate) * up, N wide.
 // A block then owns BN / 2 output columns; each wave's share of the LDS tile holds the gate
 // rows of its columns and, after them, the up rows of the same columns, so that a lane ends
 // with both values of an output element.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK, int STAGES>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const void* __restrict__ bias,
                  int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode, int m_blocks,
                  int n_blocks) {
   extern __shared__ __align__(16) unsigned char smem[];
+  static_assert(BK == 32 || BK == 64, "K steps of 32 or 64");
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // a wave's tile
   constexpr int TM = WM / 32, TN = WN / 32;            // in 32 x 32 MFMA tiles
-  constexpr int XQ = BM / 8 / NW, WQ = BN / 8 / NW;    // load instructions per wave and stage
-  constexpr int STAGE = (BM + BN) * TILE_ROW_BYTES;    // bytes per stage
+  constexpr int ROW = BK * 2;                          // bytes of a row
+  constexpr int SLOTS = BK / 8;                        // 16-byte slots of a row
+  constexpr int RPI = 1024 / ROW;                      // rows one wave instruction fills
+  constexpr int XQ = BM / RPI / NW, WQ = BN / RPI / NW;  // load instructions per wave and stage
+  constexpr int STAGE = (BM + BN) * ROW;               // bytes per stage
+  static_assert(XQ >= 1 && WQ >= 1 && (STAGES - 2) * (XQ + WQ) < 64, "tile too small or too many loads in flight");
+#define SWZ(row) (BK == 64 ? (((row) >> 1) & 7) : (((row) >> 2) & 3))
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -87,19 +97,18 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   }
   const int m0 = mb * BM, n0 = nb * (GLU ? BN / 2 : BN);
 
-  // what this lane fetches: row r = (q * NW + wave) * 8 + lane / 8 of a tile; it fills slot lane % 8
-  // of that row, which holds k chunk (lane % 8) ^ SWZ(r)
-  const int lrow = lane >> 3;
+  // what this lane fetches: row r = (q * NW + wave) * RPI + lane / SLOTS of a tile; it fills slot
+  // lane % SLOTS of that row, which holds k chunk (lane % SLOTS) ^ SWZ(r)
+  const int lrow = lane / SLOTS, lslot = lane % SLOTS;
   unsigned xoff[XQ], woff[WQ];
 #pragma unroll
   for (int q = 0; q < XQ; ++q) {
-    const int r = (q * NW + wave) * 8 + lrow;
-    xoff[q] = (unsigned)min(m0 + r, M - 1) * (unsigned)x_stride + ((lane & 7) ^ SWZ(r)) * 8;
+    const int r = (q * NW + wave) * RPI + lrow;
+    xoff[q] = (unsigned)min(m0 + r, M - 1) * (unsigned)x_stride + (lslot ^ SWZ(r)) * 8;
   }
 #pragma unroll
   for (int q = 0; q < WQ; ++q) {
-    const int r = (q * NW + wave) * 8 + lrow;  // row of the LDS tile
-    const int lchunk = (lane & 7) ^ SWZ(r);
+    const int r = (q * NW + wave) * RPI + lrow;  // row of the LDS tile
     int grow;
     if (GLU) {
       const int owner = r / WN, within = r % WN;             // the wave whose columns these are
@@ -108,20 +117,20 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
     } else {
       grow = min(n0 + r, N - 1);
     }
-    woff[q] = (unsigned)grow * (unsigned)K + lchunk * 8;
+    woff[q] = (unsigned)grow * (unsigned)K + (lslot ^ SWZ(r)) * 8;
   }
 
   auto issue = [&](int kt) {
-    unsigned char* stage = smem + (kt & 1) * STAGE;
-    const int koff = kt * TILE_BK;
+    unsigned char* stage = smem + (kt % STAGES) * STAGE;
+    const int koff = kt * BK;
 #pragma unroll
     for (int q = 0; q < XQ; ++q)
-      __builtin_amdgcn_global_load_lds((global_ptr_t)(x + xoff[q] + koff),
-                                       (lds_ptr_t)(stage + (q * NW + wave) * 8 * TILE_ROW_BYTES), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(x + xoff[q] + koff), (lds_ptr_t)(stage + (q * NW + wave) * 1024), 16,
+                                       0, 0);
 #pragma unroll
     for (int q = 0; q < WQ; ++q)
       __builtin_amdgcn_global_load_lds((global_ptr_t)(w + woff[q] + koff),
-                                       (lds_ptr_t)(stage + (BM + (q * NW + wave) * 8) * TILE_ROW_BYTES), 16, 0, 0);
+                                       (lds_ptr_t)(stage + BM * ROW + (q * NW + wave) * 1024), 16, 0, 0);
   };
 
   f32x16 acc[TM][TN];
@@ -132,55 +141,53 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  // fragment addresses: row = tile row + lane % 32, k chunk = 2 ks + lane / 32, slot = chunk ^ (row & 7)
+  // fragment addresses: row = tile row + lane % 32, k chunk = 2 ks + lane / 32, slot = chunk ^ SWZ(row)
   const int frow = lane & 31, fhalf = lane >> 5, fsw = SWZ(frow);
-  const int xbase = (wm * WM + frow) * TILE_ROW_BYTES;
-  const int wbase = (BM + wn * WN + frow) * TILE_ROW_BYTES;
+  const int xbase = (wm * WM + frow) * ROW;
+  const int wbase = (BM + wn * WN + frow) * ROW;
 
-  const int nk = K / TILE_BK;
-  issue(0);
+  const int nk = K / BK;
+#pragma unroll
+  for (int d = 0; d < STAGES - 1; ++d)
+    if (d < nk) issue(d);
   for (int kt = 0; kt < nk; ++kt) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // tile kt has landed when only the loads of the STAGES - 2 younger tiles are outstanding
+    if (kt + STAGES - 2 < nk) wait_vmcnt<(STAGES - 2) * (XQ + WQ)>();
+    else wait_vmcnt<0>();
     __syncthreads();  // tile kt is in LDS for every wave, and every wave is done with tile kt - 1
-    if (kt + 1 < nk) issue(kt + 1);
-    const unsigned char* stage = smem + (kt & 1) * STAGE;
+    if (kt + STAGES - 1 < nk) issue(kt + STAGES - 1);  // into the stage that tile kt - 1 has left
+    const unsigned char* stage = smem + (kt % STAGES) * STAGE;
     bf16x8 a[2][TM], b[2][TN];
     {
       const int slot = ((0 + fhalf) ^ fsw) << 4;
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
-        a[0][i] = as_frag(*reinterpret_cast<const uint4*>(stage + xbase + i * 32 * TILE_ROW_BYTES + slot));
+      for (int i = 0; i < TM; ++i) a[0][i] = as_frag(*reinterpret_cast<const uint4*>(stage + xbase + i * 32 * ROW + slot));
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        b[0][j] = as_frag(*reinterpret_cast<const uint4*>(stage + wbase + j * 32 * TILE_ROW_BYTES + slot));
+      for (int j = 0; j < TN; ++j) b[0][j] = as_frag(*reinterpret_cast<const uint4*>(stage + wbase + j * 32 * ROW + slot));
     }
 #pragma unroll
-    for (int ks = 0; ks < TILE_BK / 16; ++ks) {
+    for (int ks = 0; ks < BK / 16; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks + 1 < TILE_BK / 16) {
+      if (ks + 1 < BK / 16) {
         const int slot = (((ks + 1) * 2 + fhalf) ^ fsw) << 4;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-          a[nxt][i] = as_frag(*reinterpret_cast<const uint4*>(stage + xbase + i * 32 * TILE_ROW_BYTES + slot));
+          a[nxt][i] = as_frag(*reinterpret_cast<const uint4*>(stage + xbase + i * 32 * ROW + slot));
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          b[nxt][j] = as_frag(*reinterpret_cast<const uint4*>(stage + wbase + j * 32 * TILE_ROW_BYTES + slot));
+          b[nxt][j] = as_frag(*reinterpret_cast<const uint4*>(stage + wbase + j * 32 * ROW + slot));
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
-      // ask the scheduler to spread the next step's fragment reads between this step's MFMAs
-      if (ks + 1 < TILE_BK / 16) {
-#pragma unroll
-        for (int r = 0; r < TM + TN; ++r) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                         // one LDS read
-          __builtin_amdgcn_sched_group_barrier(0x008, (TM * TN) / (TM + TN), 0);     // a share of the MFMAs
-        }
-      }
+      // let the scheduler interleave the next step's fragment reads with this step's MFMAs (its
+      // strategy for small matrix-multiply loops measured best here)
+      __builtin_amdgcn_iglp_opt(1);
     }
   }
+#undef SWZ
 
   // epilogue: lane holds column n = lane % 32 of each tile and rows (e/4)*8 + (lane/32)*4 + e%4
   if (GLU) {
@@ -222,14 +229,16 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK = 64, int STAGES = 2>
 static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                        int out_stride, int m, int n, int k, int mode, hipStream_t stream) {
   static bool configured = false;
-  constexpr int lds_bytes = 2 * (BM + BN) * TILE_ROW_BYTES;
+  constexpr int lds_bytes = STAGES * (BM + BN) * BK * 2;
+  static_assert(lds_bytes <= 160 * 1024, "the stages do not fit the LDS of a CU");
+  auto kernel = &gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, GLU, BK, STAGES>;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, GLU>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       lds_bytes);
     if (e != hipSuccess) {
       axk_set_error("gemm_tile: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
       return -2;
@@ -237,8 +246,8 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
     configured = true;
   }
   const int m_blocks = ceil_div(m, BM), n_blocks = ceil_div(n, GLU ? BN / 2 : BN);
-  gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, GLU><<<m_blocks * n_blocks, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
-      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks);
+  kernel<<<m_blocks * n_blocks, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(x, x_stride, w, bias, bias_is_f32, out, out_stride,
+                                                                           m, n, k, mode, m_blocks, n_blocks);
   AXK_LAUNCH_CHECK("gemm_tile");
   return 0;
 }
