@@ -76,6 +76,28 @@ int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const
 int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
              int out_stride, int m, int n, int k, int mode, void* stream);
 
+// The same product with an RMS norm folded into it on either side, so that the norm needs no
+// pass of its own (bfloat16 build, shapes for which axk_gemm_norm_fold_ok says 1):
+// * in_squares [M, K / 16] (or null): X holds x * gain without the row's scale and in_squares
+//   the sums of x^2 over the 16-column parts of each row; the product's result is multiplied
+//   by 1 / sqrt(sum(in_squares[m]) / K + in_eps) before the bias is added.
+// * norm_gain (or null; mode 1 only): beside out += result, norm_values elem [M, N] =
+//   out * norm_gain and norm_squares [M, ceil(N / 16)] = sums of out^2 over 16 columns each:
+//   what the in_squares side of the next product takes.
+typedef struct {
+  const float* in_squares;
+  float in_eps;
+  const void* norm_gain;
+  int norm_gain_is_f32;
+  void* norm_values;
+  float* norm_squares;
+} GemmNormFold;
+int axk_gemm_norm_fold_ok(int m, int n, int k, int mode);
+int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
+                       int out_stride, int m, int n, int k, int mode, const float* in_squares, float in_eps,
+                       const void* norm_gain, int norm_gain_is_f32, void* norm_values, float* norm_squares,
+                       void* stream);
+
 // out[t, f] = silu(gu[t, f]) * gu[t, F + f]: gate in the first F columns, up in the last.
 int axk_swiglu(const void* gate_up, void* out, int n_tokens, int n_ffn, void* stream);
 

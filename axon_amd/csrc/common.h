@@ -82,6 +82,23 @@ __device__ inline float wave_sum(float v) {
   return v;
 }
 
+// The sum of the 64 lanes in lane 63 alone (other lanes end with partial sums), through the
+// lane-permuting forms of the adder instead of the LDS crossbar: a few cycles a step where the
+// butterfly above takes an LDS round trip.  Pairs, quads, halves of a row of 16, the row, then
+// rows 0+1 and 2+3, then both: the order is fixed.
+__device__ inline float wave_sum_to_last(float v) {
+#define AXON_DPP(val, ctrl, rows) \
+  __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, val), ctrl, rows, 0xf, false))
+  v += AXON_DPP(v, 0xb1, 0xf);    // quad_perm [1, 0, 3, 2]
+  v += AXON_DPP(v, 0x4e, 0xf);    // quad_perm [2, 3, 0, 1]
+  v += AXON_DPP(v, 0x141, 0xf);   // row_half_mirror
+  v += AXON_DPP(v, 0x140, 0xf);   // row_mirror
+  v += AXON_DPP(v, 0x142, 0xa);   // lane 15 of rows 0 and 2 to the rows after them
+  v += AXON_DPP(v, 0x143, 0xc);   // lane 31 to rows 2 and 3
+#undef AXON_DPP
+  return v;
+}
+
 __device__ inline float wave_max(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, AXON_WAVE));

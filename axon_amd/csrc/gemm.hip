@@ -144,11 +144,13 @@ static int launch_fma(const elem_t* x, int x_stride, const elem_t* w, const void
 
 #if AXON_BF16
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, bool* handled);
+                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold,
+                     bool* handled);
+int gemm_norm_fold_ok(int m, int n, int k, int mode);
 #endif
 
-extern "C" int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
-                        int out_stride, int m, int n, int k, int mode, void* stream) {
+static int gemm_checked(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
+                        int out_stride, int m, int n, int k, int mode, const GemmNormFold* fold, void* stream) {
   AXK_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
   AXK_REQUIRE(x_stride >= k && out_stride >= n, "gemm: strides x=%d (K=%d) out=%d (N=%d) too small", x_stride, k,
               out_stride, n);
@@ -159,9 +161,37 @@ extern "C" int axk_gemm(const void* x, int x_stride, const void* w, const void* 
 #if AXON_BF16
   bool handled = false;
   int rc = launch_gemm_mfma((const bf16_t*)x, x_stride, (const bf16_t*)w, bias, bias_is_f32, out, out_stride, m, n, k,
-                            mode, (hipStream_t)stream, &handled);
+                            mode, (hipStream_t)stream, fold, &handled);
   if (rc != 0 || handled) return rc;
 #endif
+  AXK_REQUIRE(fold == nullptr, "gemm: no kernel folds a norm into M=%d N=%d K=%d of these strides and alignments", m, n,
+              k);
   return launch_fma((const elem_t*)x, x_stride, (const elem_t*)w, bias, bias_is_f32, out, out_stride, m, n, k, mode,
                     (hipStream_t)stream);
+}
+
+extern "C" int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
+                        int out_stride, int m, int n, int k, int mode, void* stream) {
+  return gemm_checked(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, nullptr, stream);
+}
+
+extern "C" int axk_gemm_norm_fold_ok(int m, int n, int k, int mode) {
+#if AXON_BF16
+  return m >= 0 && n > 0 && k > 0 && gemm_norm_fold_ok(m, n, k, mode);
+#else
+  return 0;   // the 32-bit build keeps the norm a pass of its own
+#endif
+}
+
+extern "C" int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32,
+                                  void* out, int out_stride, int m, int n, int k, int mode, const float* in_squares,
+                                  float in_eps, const void* norm_gain, int norm_gain_is_f32, void* norm_values,
+                                  float* norm_squares, void* stream) {
+  AXK_REQUIRE(axk_gemm_norm_fold_ok(m, n, k, mode), "gemm: no kernel folds a norm into M=%d N=%d K=%d mode %d", m, n, k,
+              mode);
+  AXK_REQUIRE(norm_gain == nullptr || (mode == MODE_ADD_F32 && norm_values && norm_squares),
+              "gemm: the following norm needs the add-into-residual epilogue and both of its outputs");
+  AXK_REQUIRE(((uintptr_t)in_squares & 15) == 0, "gemm: the rows' sums of squares must be 16-byte aligned");
+  const GemmNormFold fold = {in_squares, in_eps, norm_gain, norm_gain_is_f32, norm_values, norm_squares};
+  return gemm_checked(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, &fold, stream);
 }

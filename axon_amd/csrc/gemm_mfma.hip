@@ -259,12 +259,32 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
 // A lane ends with 4 consecutive n of one m: one vector store.
 // GLU (NT16 = 2): the block's two tiles are the gate rows n0 .. n0 + 15 and the up rows of the
 // same columns (W holds 2 N rows), and the output is silu(gate) * up.
+//
+// An RMS norm can be folded into the product on either side, which saves the norm's own pass
+// over the rows (a launch each, between products that take microseconds):
+// * in_squares: X holds x * gain, not yet scaled by its row's 1/rms, and in_squares [M, K / 16]
+//   the sums of x^2 over the 16-column parts of each row.  Every block adds a row's parts (in
+//   the same order, so all blocks agree) and multiplies the finished sums of products by
+//   1/sqrt(sum / K + eps): the scale is common to the row, so it commutes with the product.
+// * norm_gain (with the add-into-residual epilogue): beside out += result the block writes what
+//   the next product's in_squares side takes: norm_values = out * norm_gain in bfloat16 and
+//   norm_squares [M, ceil(N / 16)], the sums of out^2 over each tile's 16 columns.
+struct NormFold {
+  const float* in_squares;
+  float in_eps;
+  const void* norm_gain;
+  int norm_gain_is_f32;
+  bf16_t* norm_values;
+  float* norm_squares;
+};
+
 template <int NT16, int MT16, int WAVES, int DEPTH, bool GLU>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w,
                    const void* __restrict__ bias, int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N,
-                   int K, int mode) {
+                   int K, int mode, NormFold fold) {
   __shared__ float partial[WAVES][NT16 * MT16][64][4];
+  __shared__ float row_scale[MT16 * 16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n0 = blockIdx.x * (GLU ? 16 : NT16 * 16);
   const int r16 = lane & 15, kq = (lane >> 4) * 8;
@@ -315,9 +335,46 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
                                                               0, 0, 0);
   };
 
+  // The rows' scales.  Wave v takes rows v, v + WAVES, ...; a lane adds every 64th part, then the
+  // lanes' sums are added.  Up to 256 parts (K <= 4096): one 16-byte load a lane and row, issued before the ring's,
+  // so they return first (loads return in order) and are added up while the ring's first loads
+  // are under way, and nothing between here and the main loop waits for the ring.  A wider K
+  // is added up in a loop, before the ring starts.
+  constexpr bool FOLDS = MT16 == 1;     // steps of up to 16 rows (see gemm_norm_fold_ok)
+  constexpr int RW = FOLDS ? 16 / WAVES : 1;
+  float4 sq[RW];
+  const int parts = K / 16;             // a multiple of 4, as K is one of 64
+  const bool fold_in = FOLDS && fold.in_squares != nullptr;
+  const bool few_parts = parts <= 256;
+  if (fold_in) {
+    if (few_parts) {
+#pragma unroll
+      for (int i = 0; i < RW; ++i) {
+        const int m = wave + i * WAVES;
+        sq[i] = m < M && lane * 4 < parts ? *reinterpret_cast<const float4*>(fold.in_squares + (size_t)m * parts + lane * 4)
+                                          : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      }
+    } else {
+      for (int m = wave; m < M; m += WAVES) {
+        float sum = 0.0f;
+        for (int part = lane; part < parts; part += 64) sum += fold.in_squares[(size_t)m * parts + part];
+        const float total = wave_sum_to_last(sum);
+        if (lane == 63) row_scale[m] = 1.0f / sqrtf(total / (float)K + fold.in_eps);
+      }
+    }
+  }
   if (mine > 0) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) load(d, min(d, mine - 1));   // beyond this wave's steps: a valid step again
+  }
+  if (fold_in && few_parts) {
+#pragma unroll
+    for (int i = 0; i < RW; ++i) {
+      const float total = wave_sum_to_last((sq[i].x + sq[i].y) + (sq[i].z + sq[i].w));
+      if (lane == 63) row_scale[wave + i * WAVES] = 1.0f / sqrtf(total / (float)K + fold.in_eps);
+    }
+  }
+  if (mine > 0) {
     int base = 0;  // the ring holds local steps base .. base + DEPTH - 1
     for (; base + 2 * DEPTH <= mine; base += DEPTH) {
 #pragma unroll
@@ -351,6 +408,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
       const int m = j * 16 + r16;
       const int n = n0 + (lane >> 4) * 4;
       if (m >= M) continue;
+      const float scale = fold.in_squares ? row_scale[m] : 1.0f;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         if (n + e >= N) continue;
@@ -359,6 +417,10 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
         for (int q = 1; q < WAVES; ++q) {
           g += partial[q][j][lane][e];
           u += partial[q][MT16 + j][lane][e];
+        }
+        if (fold.in_squares) {
+          g *= scale;
+          u *= scale;
         }
         reinterpret_cast<bf16_t*>(out)[(size_t)m * out_stride + n + e] = float_to_bf16(swiglu1(g, u));
       }
@@ -378,52 +440,90 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
     }
     const int m = j * 16 + r16;
     const int n = n0 + i * 16 + (lane >> 4) * 4;
-    if (m >= M) continue;
+    const bool row_ok = m < M;
+    const float scale = fold.in_squares && row_ok ? row_scale[m] : 1.0f;
+    float squares = 0.0f;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      if (n + e >= N) continue;
+      if (!row_ok || n + e >= N) continue;
       float r = v[e];
+      if (fold.in_squares) r *= scale;
       if (bias) r += load_vec(bias, bias_is_f32, n + e);
       const size_t at = (size_t)m * out_stride + n + e;
       if (mode == MODE_STORE) reinterpret_cast<bf16_t*>(out)[at] = float_to_bf16(r);
-      else if (mode == MODE_ADD_F32) reinterpret_cast<float*>(out)[at] += r;
-      else reinterpret_cast<float*>(out)[at] = r;
+      else if (mode == MODE_ADD_F32) {
+        const float sum = reinterpret_cast<float*>(out)[at] + r;
+        reinterpret_cast<float*>(out)[at] = sum;
+        if (fold.norm_gain) {
+          fold.norm_values[(size_t)m * N + n + e] = float_to_bf16(sum * load_vec(fold.norm_gain, fold.norm_gain_is_f32, n + e));
+          squares = fmaf(sum, sum, squares);
+        }
+      } else reinterpret_cast<float*>(out)[at] = r;
+    }
+    if (fold.norm_gain) {
+      // the four lanes that hold a row's 16 columns of this tile: lane, lane ^ 16, lane ^ 32, lane ^ 48
+      squares += __shfl_xor(squares, 16, AXON_WAVE);
+      squares += __shfl_xor(squares, 32, AXON_WAVE);
+      if (row_ok && lane < 16 && n0 + i * 16 < N) fold.norm_squares[(size_t)m * ((N + 15) >> 4) + (n0 >> 4) + i] = squares;
     }
   }
 }
 
 template <int NT16, int MT16, int WAVES, int DEPTH, bool GLU = false>
 static int launch_skinny(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                         int out_stride, int m, int n, int k, int mode, hipStream_t stream) {
+                         int out_stride, int m, int n, int k, int mode, hipStream_t stream, const NormFold& fold) {
   gemm_skinny_kernel<NT16, MT16, WAVES, DEPTH, GLU><<<ceil_div(n, GLU ? 16 : NT16 * 16), WAVES * 64, 0, stream>>>(
-      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode);
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, fold);
   AXK_LAUNCH_CHECK("gemm_skinny");
   return 0;
 }
 
 // Shapes the MFMA kernels take: K a multiple of 64 and 16-byte aligned rows.  Decided by (N, K)
 // and the pointers' alignment, never by M, so a weight matrix always meets the same kernels.
+static bool skinny_takes(int m, int n, int k, int mode) {
+  // a very wide output (the head) with more than 32 rows goes to the tiled kernel, which shares
+  // X through LDS
+  return m <= 64 && !(m > 32 && n >= 65536 && mode != MODE_SWIGLU && (size_t)n * k < (1ull << 32));
+}
+
+// A norm is folded into steps of up to 16 rows: with more, adding up the rows' parts costs a
+// block more than the norm's own pass saves.
+int gemm_norm_fold_ok(int m, int n, int k, int mode) { return k % 64 == 0 && m <= 16 && skinny_takes(m, n, k, mode); }
+
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, bool* handled) {
+                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold_in,
+                     bool* handled) {
   *handled = false;
   if (k % 64 != 0 || x_stride % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return 0;
   *handled = true;
+  NormFold fold = {nullptr, 0.0f, nullptr, 0, nullptr, nullptr};
+  if (fold_in) {
+    fold.in_squares = fold_in->in_squares;
+    fold.in_eps = fold_in->in_eps;
+    fold.norm_gain = fold_in->norm_gain;
+    fold.norm_gain_is_f32 = fold_in->norm_gain_is_f32;
+    fold.norm_values = (bf16_t*)fold_in->norm_values;
+    fold.norm_squares = fold_in->norm_squares;
+  }
 #define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream
   if (m <= 64 && mode == MODE_SWIGLU) {
-    if (m <= 16) return launch_skinny<2, 1, 4, 8, true>(ARGS);
-    if (m <= 32) return launch_skinny<2, 2, 4, 4, true>(ARGS);
-    return launch_skinny<2, 4, 4, 2, true>(ARGS);
+    if (m <= 16) return launch_skinny<2, 1, 4, 8, true>(ARGS, fold);
+    if (m <= 32) return launch_skinny<2, 2, 4, 4, true>(ARGS, fold);
+    return launch_skinny<2, 4, 4, 2, true>(ARGS, fold);
   }
-  if (m <= 64) {
+  if (skinny_takes(m, n, k, mode)) {
     // 32 rows of W per block where that still leaves 128 blocks or more, else 16; four waves
     // split K; the ring is as deep as the registers allow
     const bool wide = n >= 32 * 128;
-    if (m <= 16) return wide ? launch_skinny<2, 1, 4, 8>(ARGS) : launch_skinny<1, 1, 4, 8>(ARGS);
-    if (m <= 32) return wide ? launch_skinny<2, 2, 4, 4>(ARGS) : launch_skinny<1, 2, 4, 8>(ARGS);
-    // a very wide output (the head) with more than 32 rows: the tiled kernel shares X through LDS
-    if (n >= 65536 && mode != MODE_SWIGLU && (size_t)n * k < (1ull << 32)) return launch_tile<128, 128, 2, 2, false>(ARGS);
-    return wide ? launch_skinny<2, 4, 4, 2>(ARGS) : launch_skinny<1, 4, 4, 4>(ARGS);
+    if (m <= 16) return wide ? launch_skinny<2, 1, 4, 8>(ARGS, fold) : launch_skinny<1, 1, 4, 8>(ARGS, fold);
+    if (m <= 32) return wide ? launch_skinny<2, 2, 4, 4>(ARGS, fold) : launch_skinny<1, 2, 4, 8>(ARGS, fold);
+    return wide ? launch_skinny<2, 4, 4, 2>(ARGS, fold) : launch_skinny<1, 4, 4, 4>(ARGS, fold);
   }
+  if (fold_in) {
+    axk_set_error("gemm: M=%d N=%d goes to the tiled kernel, which folds no norm", m, n);
+    return -1;
+  }
+  if (m <= 64) return launch_tile<128, 128, 2, 2, false>(ARGS);
   // offsets inside the kernels are 32-bit element counts
   if ((size_t)n * k * (mode == MODE_SWIGLU ? 2 : 1) >= (1ull << 32) || (size_t)m * x_stride >= (1ull << 32)) {
     *handled = false;

@@ -44,6 +44,9 @@ _SIGNATURES = {
                              c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "axk_attention_fast_ok": [c_int, c_int, c_int, c_int],
     "axk_gemm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "axk_gemm_norm_fold_ok": [c_int, c_int, c_int, c_int],
+    "axk_gemm_norm_fold": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                           c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
     "axk_swiglu": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_argmax": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "axk_topk": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -218,10 +221,21 @@ class Kernels:
             n_heads, n_kv_heads, head_dim, page_size, window, float(scale), _stream()))
         return out
 
+    def gemm_norm_fold_ok(self, m: int, n: int, k: int, mode: int) -> bool:
+        """Whether the product of these sizes can take an RMS norm into itself (see `gemm`)."""
+        return bool(self.lib.axk_gemm_norm_fold_ok(m, n, k, mode))
+
     def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
-             mode: int = MODE_STORE) -> torch.Tensor:
+             mode: int = MODE_STORE, row_squares: Optional[torch.Tensor] = None, eps: float = 0.0,
+             following_norm=None) -> torch.Tensor:
         """out = epilogue(x . w^T + bias); x [M, K] (rows may be strided), w [N, K] contiguous.
-        MODE_SWIGLU: w is [2 N, K], gate rows then up rows; out [M, N] = silu(x gate^T) * (x up^T)."""
+        MODE_SWIGLU: w is [2 N, K], gate rows then up rows; out [M, N] = silu(x gate^T) * (x up^T).
+
+        An RMS norm folded in (where `gemm_norm_fold_ok`): with `row_squares` float32 [M, K / 16],
+        x holds rows times their gain that still lack the scale 1/sqrt(sum(row_squares) / K + eps),
+        which the product applies to its result.  `following_norm` = (gain, values [M, N],
+        squares [M, ceil(N / 16)]) with MODE_ADD_F32: the epilogue also writes out * gain and the
+        sums of out^2 over parts of 16 columns, for the next product's `row_squares` side."""
         self._elem(x, "gemm x"); self._elem(w, "gemm w")
         M, K = x.shape
         N = w.shape[0]
@@ -238,8 +252,27 @@ class Kernels:
             raise KernelError(f"gemm: mode {mode} writes {want}, out is {out.dtype}")
         if bias is not None and bias.numel() != N:
             raise KernelError(f"gemm: bias of {bias.numel()} for {N} columns")
-        self._check(self.lib.axk_gemm(_ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"),
-                                      _ptr(out), out.stride(0), M, N, K, mode, _stream()))
+        if row_squares is None and following_norm is None:
+            self._check(self.lib.axk_gemm(_ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"),
+                                          _ptr(out), out.stride(0), M, N, K, mode, _stream()))
+            return out
+        if row_squares is not None and (row_squares.dtype != torch.float32 or not row_squares.is_contiguous()
+                                        or row_squares.shape != (M, K // 16) or not row_squares.is_cuda):
+            raise KernelError(f"gemm: row_squares {tuple(row_squares.shape)} {row_squares.dtype} is not float32 "
+                              f"[{M}, {K // 16}]")
+        gain = values = squares = None
+        if following_norm is not None:
+            gain, values, squares = following_norm
+            self._elem(values, "gemm norm values")
+            if (gain.numel() != N or values.shape != (M, N) or not values.is_contiguous()
+                    or squares.shape != (M, -(-N // 16)) or squares.dtype != torch.float32 or not squares.is_contiguous()
+                    or not squares.is_cuda):
+                raise KernelError(f"gemm: the following norm's gain {tuple(gain.shape)}, values {tuple(values.shape)} "
+                                  f"or squares {tuple(squares.shape)} do not fit [{M}, {N}]")
+        self._check(self.lib.axk_gemm_norm_fold(
+            _ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"), _ptr(out), out.stride(0), M, N, K,
+            mode, _ptr(row_squares), float(eps), _ptr(gain), self._vec_flag(gain, "gemm norm gain"), _ptr(values),
+            _ptr(squares), _stream()))
         return out
 
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

@@ -104,8 +104,17 @@ class DecoderModel:
     def forward(self, ctx) -> torch.Tensor:
         """The residual stream after every run: float32 [T, hidden]."""
         x = self.embedding.forward(ctx)
-        for run, binding in zip(self.order, self.cache_plan.bindings):
-            self.blocks[run.layer].forward(ctx, binding, x)
+        unscaled = None      # the next block's first norm, where the block before it did its work
+        for i, (run, binding) in enumerate(zip(self.order, self.cache_plan.bindings)):
+            block = self.blocks[run.layer]
+            fold = None
+            if i + 1 < len(self.order) and block.folds_following_norm(ctx):
+                fold = self.blocks[self.order[i + 1].layer].first_norm_fold(ctx, x.shape[0])
+            if unscaled is None and fold is None:
+                block.forward(ctx, binding, x)
+            else:
+                block.forward(ctx, binding, x, unscaled, fold)
+            unscaled = None if fold is None else fold.rows()
         return x
 
     def logits(self, ctx, x: torch.Tensor, rows: torch.Tensor, out=None) -> torch.Tensor:

@@ -21,7 +21,7 @@ import torch
 
 from ..config.base import ConfigError
 from ..kernels import MODE_ADD_F32, MODE_STORE
-from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, build_part, register_mixer
+from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, UnscaledRows, build_part, register_mixer
 
 
 PREFILL_TILE = 128     # tokens of one request per tile of the prompt kernel
@@ -143,9 +143,20 @@ class GQAttention(Mixer):
             self.position.load(store, rt)
 
     # ------------------------------------------------------------------ the step
-    def forward(self, ctx, binding: CacheBinding, h, residual) -> None:
+    def takes_unscaled_rows(self, ctx) -> bool:
+        k = ctx.rt.k
+        return (k.gemm_norm_fold_ok(ctx.n_tokens, self.q_dim + 2 * self.kv_dim, self.hidden, MODE_STORE)
+                and k.gemm_norm_fold_ok(ctx.n_tokens, self.q_dim, self.hidden, MODE_STORE))
+
+    def folds_following_norm(self, ctx) -> bool:
+        return ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.hidden, self.q_dim, MODE_ADD_F32)
+
+    def forward(self, ctx, binding: CacheBinding, h, residual, fold=None) -> None:
         k = ctx.rt.k
         T = h.shape[0]
+        scaled = {}
+        if isinstance(h, UnscaledRows):
+            h, scaled = h.values, {"row_squares": h.squares, "eps": h.eps}
         group = ctx.cache.group(binding.group)
         k_cache, v_cache = group.layer(binding.index)
         # values are kept position-contiguous: a page of them is [heads, head_dim, page_size]
@@ -153,12 +164,12 @@ class GQAttention(Mixer):
         mark = ctx.ws.mark()
         if binding.writes:
             qkv = ctx.ws.take((T, self.q_dim + 2 * self.kv_dim), ctx.rt.dtype)
-            k.gemm(h, self.w_qkv, qkv, self.b_qkv, MODE_STORE)
+            k.gemm(h, self.w_qkv, qkv, self.b_qkv, MODE_STORE, **scaled)
         else:
             # reading another run's cache: only the queries are needed
             qkv = ctx.ws.take((T, self.q_dim + 2 * self.kv_dim), ctx.rt.dtype)
             bias = None if self.b_qkv is None else self.b_qkv[:self.q_dim]
-            k.gemm(h, self.w_qkv[:self.q_dim], qkv[:, :self.q_dim], bias, MODE_STORE)
+            k.gemm(h, self.w_qkv[:self.q_dim], qkv[:, :self.q_dim], bias, MODE_STORE, **scaled)
         if self.position is not None:
             table, rotary = self.position.tables(ctx), self.position.rotary_dim
         else:
@@ -177,7 +188,8 @@ class GQAttention(Mixer):
         else:
             k.attention(qkv, qkv.stride(0), k_cache, v_cache, group.block_table, ctx.positions, ctx.seq_rows, att,
                         self.nh, self.nkv, self.hd, group.page_size, self.window, self.scale)
-        k.gemm(att, self.w_o, residual, self.b_o, MODE_ADD_F32)
+        k.gemm(att, self.w_o, residual, self.b_o, MODE_ADD_F32,
+               following_norm=None if fold is None else fold.following_norm())
         ctx.ws.release(mark)
 
 

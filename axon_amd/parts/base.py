@@ -88,9 +88,44 @@ class Part:
         (device, dtype, kernels)."""
 
 
+class UnscaledRows:
+    """Rows of a norm that still lack their scale: `values` [T, size] in the compute dtype hold
+    x * gain, `squares` float32 [T, size / 16] the sums of x^2 over the 16-column parts of each
+    row, `eps` the norm's constant.  The product that reads them multiplies its result by
+    1 / sqrt(sum(squares) / size + eps): the scale is common to a row, so it commutes with the
+    product, and the norm needs no pass of its own over the rows."""
+
+    def __init__(self, values, squares, eps: float):
+        self.values, self.squares, self.eps = values, squares, eps
+
+    @property
+    def shape(self):
+        return self.values.shape
+
+
+class NormFold:
+    """A norm handed to the part that runs before it: that part's last product, which adds into
+    the residual stream, also writes `values` = residual * gain and `squares` (see UnscaledRows)
+    in its epilogue; `rows()` is then what the part after the norm reads."""
+
+    def __init__(self, gain, eps: float, values, squares):
+        self.gain, self.eps, self.values, self.squares = gain, eps, values, squares
+
+    def following_norm(self):
+        return (self.gain, self.values, self.squares)
+
+    def rows(self) -> UnscaledRows:
+        return UnscaledRows(self.values, self.squares, self.eps)
+
+
 class Norm(Part):
     def forward(self, ctx, x, out=None):
         raise NotImplementedError
+
+    def fold(self, ctx, n_rows: int) -> Optional[NormFold]:
+        """This norm as work for the neighbouring products (with buffers for `n_rows` rows), or
+        None if it has to run on its own."""
+        return None
 
 
 class PositionEncoding(Part):
@@ -112,11 +147,25 @@ class Mixer(Part):
         back in `ctx.decode_shapes[name]`.  None: nothing else matters."""
         return None
 
+    def takes_unscaled_rows(self, ctx) -> bool:
+        """Whether `h` may be UnscaledRows in this step (the first product applies the scale)."""
+        return False
+
+    def folds_following_norm(self, ctx) -> bool:
+        """Whether `forward` takes a NormFold as a further argument in this step and fills it."""
+        return False
+
     def forward(self, ctx, binding: CacheBinding, h, residual) -> None:
         raise NotImplementedError
 
 
 class FeedForward(Part):
+    def takes_unscaled_rows(self, ctx) -> bool:
+        return False
+
+    def folds_following_norm(self, ctx) -> bool:
+        return False
+
     def forward(self, ctx, h, residual) -> None:
         raise NotImplementedError
 
@@ -129,7 +178,20 @@ class Block(Part):
         self.mixer = mixer
         self.feed_forward = feed_forward
 
-    def forward(self, ctx, binding: CacheBinding, x) -> None:
+    def first_norm_fold(self, ctx, n_rows: int) -> Optional[NormFold]:
+        """The block's first norm as work for the block before it (see NormFold), or None: then
+        `forward` is called without `unscaled`."""
+        return None
+
+    def folds_following_norm(self, ctx) -> bool:
+        """Whether `forward` takes the next block's first norm as `fold_next` in this step."""
+        return False
+
+    def forward(self, ctx, binding: CacheBinding, x, unscaled: Optional[UnscaledRows] = None,
+                fold_next: Optional[NormFold] = None) -> None:
+        """Update the residual stream x in place.  `unscaled`: the first norm's rows, already left
+        by the block before; `fold_next`: to be filled for the block after (both only if this
+        block offered it)."""
         raise NotImplementedError
 
 

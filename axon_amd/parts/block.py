@@ -10,6 +10,9 @@ from typing import List
 
 from .base import Block, CacheBinding, TensorDecl, register_block
 
+# A norm between two products can be folded into them where both offer it (short steps in
+# bfloat16: the products then run in kernels that take it): the block asks its parts.
+
 
 class PreNormBlock(Block):
     graph_safe = True
@@ -28,13 +31,28 @@ class PreNormBlock(Block):
         for part in (self.norm1, self.mixer, self.norm2, self.feed_forward):
             part.load(store, rt)
 
-    def forward(self, ctx, binding: CacheBinding, x) -> None:
+    def first_norm_fold(self, ctx, n_rows: int):
+        return self.norm1.fold(ctx, n_rows) if self.mixer.takes_unscaled_rows(ctx) else None
+
+    def folds_following_norm(self, ctx) -> bool:
+        return self.feed_forward.folds_following_norm(ctx)
+
+    def forward(self, ctx, binding: CacheBinding, x, unscaled=None, fold_next=None) -> None:
         mark = ctx.ws.mark()
-        h = self.norm1.forward(ctx, x)
-        self.mixer.forward(ctx, binding, h, x)
-        ctx.ws.release(mark)
-        h = self.norm2.forward(ctx, x)
-        self.feed_forward.forward(ctx, h, x)
+        h = unscaled if unscaled is not None else self.norm1.forward(ctx, x)
+        fold = None
+        if self.mixer.folds_following_norm(ctx) and self.feed_forward.takes_unscaled_rows(ctx):
+            fold = self.norm2.fold(ctx, x.shape[0])
+        if fold is not None:
+            self.mixer.forward(ctx, binding, h, x, fold)
+            h = fold.rows()
+        else:
+            self.mixer.forward(ctx, binding, h, x)
+            h = self.norm2.forward(ctx, x)
+        if fold_next is not None:
+            self.feed_forward.forward(ctx, h, x, fold_next)
+        else:
+            self.feed_forward.forward(ctx, h, x)
         ctx.ws.release(mark)
 
 

@@ -7,7 +7,9 @@ from __future__ import annotations
 
 from typing import List, Optional
 
-from .base import Norm, TensorDecl, register_norm
+import torch
+
+from .base import Norm, NormFold, TensorDecl, register_norm
 
 
 class RMSNorm(Norm):
@@ -31,6 +33,16 @@ class RMSNorm(Norm):
         if out is None:
             out = ctx.ws.take((n, self.size), ctx.rt.dtype)
         return ctx.rt.k.rmsnorm(x, self.gain, self.eps, out, rows)
+
+    def fold(self, ctx, n_rows: int) -> Optional[NormFold]:
+        """The product before the norm leaves x * gain and the sums of squares, the product
+        after it applies 1/sqrt(mean + eps): the same formula, the row's scale moved behind the
+        product (it is common to the row)."""
+        if self.size % 16:
+            return None
+        values = ctx.ws.take((n_rows, self.size), ctx.rt.dtype)
+        squares = ctx.ws.take((n_rows, self.size // 16), torch.float32)
+        return NormFold(self.gain, self.eps, values, squares)
 
 
 register_norm("rmsnorm", RMSNorm)

@@ -217,6 +217,58 @@ def test_gemm_rows_do_not_depend_on_the_batch(dtype):
         assert (small - full[:64]).abs().max() <= 1e-5 * full.abs().max()
 
 
+@pytest.mark.parametrize("M,H,F", [(1, 64, 128), (8, 192, 320), (16, 448, 64), (5, 4608, 64), (13, 128, 192)])
+def test_gemm_with_a_norm_folded_in(M, H, F):
+    """residual += a . Wo^T; h = rmsnorm(residual) * gain; out = h . W^T + bias, with the norm done
+    by the two products: the first leaves residual * gain and the rows' sums of squares, the
+    second scales its result.  Against the plain norm between plain products."""
+    k = kernels("bfloat16")
+    eps = 3e-5
+    a, ar = as_dtype(rnd(M, F, seed=40), "bfloat16")
+    wo, wor = as_dtype(rnd(H, F, seed=41, scale=0.3), "bfloat16")
+    res = rnd(M, H, seed=42, scale=2.0)
+    res[0] *= 40.0                                        # a row of another magnitude: the scale is per row
+    for gain_dt in (torch.float32, torch.bfloat16):
+        gain = (1.0 + 0.3 * rnd(H, seed=43)).to(gain_dt)
+        x_ref = res.double() + ar @ wor.T
+        h_ref = P.rms_norm(x_ref, gain.double(), eps)
+        assert k.gemm_norm_fold_ok(M, H, F, MODE_ADD_F32)
+        x = res.clone().cuda()
+        values = torch.empty(M, H, dtype=torch.bfloat16, device="cuda")
+        squares = torch.full((M, H // 16), float("nan"), dtype=torch.float32, device="cuda")
+        k.gemm(a, wo, x, None, MODE_ADD_F32, following_norm=(gain.cuda(), values, squares))
+        assert (x.cpu().double() - x_ref).abs().max() <= 2e-5 * math.sqrt(F) * x_ref.abs().max()
+        got_sq = squares.cpu().double().sum(1)
+        assert ((got_sq - (x_ref ** 2).sum(1)).abs() <= 1e-5 * (x_ref ** 2).sum(1)).all()
+        # the consumer: a plain product with bias, and the gated one
+        for N in (48, 272):
+            w, wr = as_dtype(rnd(N, H, seed=44, scale=0.2), "bfloat16")
+            bias = rnd(N, seed=45)
+            out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+            k.gemm(values, w, out, bias.cuda(), MODE_STORE, row_squares=squares, eps=eps)
+            want = h_ref @ wr.T + bias.double()
+            assert (out.cpu().double() - want).abs().max() <= tol("bfloat16", want, 0, 1e-2)
+        wg, wgr = as_dtype(rnd(2 * 80, H, seed=46, scale=0.2), "bfloat16")
+        out = torch.empty(M, 80, dtype=torch.bfloat16, device="cuda")
+        k.gemm(values, wg, out, None, MODE_SWIGLU, row_squares=squares, eps=eps)
+        want = P.swiglu(h_ref @ wgr[:80].T, h_ref @ wgr[80:].T)
+        assert (out.cpu().double() - want).abs().max() <= tol("bfloat16", want, 0, 1e-2)
+
+
+def test_gemm_refuses_a_norm_it_cannot_fold():
+    k = kernels("bfloat16")
+    assert not k.gemm_norm_fold_ok(17, 64, 64, MODE_STORE)          # more rows than a folded step takes
+    assert not k.gemm_norm_fold_ok(8, 64, 70, MODE_STORE)           # K that the matrix-core kernels refuse
+    assert not kernels("float32").gemm_norm_fold_ok(8, 64, 64, MODE_STORE)
+    x = torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(KernelError):
+        k.gemm(x, w, out, None, MODE_STORE, row_squares=torch.zeros(17, 4, device="cuda"), eps=1e-6)
+    with pytest.raises(KernelError):                                 # sums of squares of the wrong shape
+        k.gemm(x[:8], w, out[:8], None, MODE_STORE, row_squares=torch.zeros(8, 5, device="cuda"), eps=1e-6)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_strided_rows(dtype):
     k = kernels(dtype)
