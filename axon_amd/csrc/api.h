@@ -102,8 +102,10 @@ int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, const void* b
 int axk_swiglu(const void* gate_up, void* out, int n_tokens, int n_ffn, void* stream);
 
 // picks[r] = index of the largest logit of row r; of equal maxima the last; NaN never
-// (all NaN: n - 1).
-int axk_argmax(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n, void* stream);
+// (all NaN: n - 1).  workspace: axk_argmax_workspace(n_rows, n) bytes, 8-byte aligned.
+long axk_argmax_workspace(int n_rows, int n);
+int axk_argmax(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n, void* workspace,
+               void* stream);
 
 // Repeat penalty on `recent` ids, then the k best as 64-bit keys (order key of the logit <<
 // 32 | id), unsorted, into cands[r, 0..k); the penalty is applied to `logits` in place.  recent is [n_rows, recent_stride] with

@@ -30,32 +30,76 @@ __device__ inline uint64_t wave_max_u64(uint64_t v) {
   return v;
 }
 
-__global__ void __launch_bounds__(PICK_THREADS)
-argmax_kernel(const float* __restrict__ logits, int stride, int32_t* __restrict__ picks, int n) {
-  __shared__ uint64_t partial[PICK_THREADS / AXON_WAVE];
-  const float* row = logits + (size_t)blockIdx.x * stride;
+// Two launches: blocks of 256 threads each take ARGMAX_CHUNK logits of one row and leave the
+// largest key of their chunk; then one wave per row takes the largest of those.  The largest
+// of 64-bit keys does not depend on the order in which they are compared.
+#define ARGMAX_CHUNK 4096
+#define ARGMAX_THREADS 256
+
+__global__ void __launch_bounds__(ARGMAX_THREADS)
+argmax_chunk_kernel(const float* __restrict__ logits, int stride, uint64_t* __restrict__ chunk_best, int n, int vec) {
+  __shared__ uint64_t partial[ARGMAX_THREADS / AXON_WAVE];
+  const float* row = logits + (size_t)blockIdx.y * stride;
+  const int lo = blockIdx.x * ARGMAX_CHUNK, hi = min(n, lo + ARGMAX_CHUNK);
   uint64_t best = 0;
-  for (int i = threadIdx.x; i < n; i += PICK_THREADS) {
-    const uint64_t k = key64(row[i], i);
-    best = k > best ? k : best;
+  if (vec && hi == lo + ARGMAX_CHUNK) {
+#pragma unroll
+    for (int j = 0; j < ARGMAX_CHUNK / (4 * ARGMAX_THREADS); ++j) {
+      const int i = lo + (j * ARGMAX_THREADS + threadIdx.x) * 4;
+      const float4 v = *reinterpret_cast<const float4*>(row + i);
+      uint64_t k = key64(v.x, i);
+      best = k > best ? k : best;
+      k = key64(v.y, i + 1);
+      best = k > best ? k : best;
+      k = key64(v.z, i + 2);
+      best = k > best ? k : best;
+      k = key64(v.w, i + 3);
+      best = k > best ? k : best;
+    }
+  } else {
+    for (int i = lo + threadIdx.x; i < hi; i += ARGMAX_THREADS) {
+      const uint64_t k = key64(row[i], i);
+      best = k > best ? k : best;
+    }
   }
   best = wave_max_u64(best);
   if ((threadIdx.x & (AXON_WAVE - 1)) == 0) partial[threadIdx.x / AXON_WAVE] = best;
   __syncthreads();
   if (threadIdx.x == 0) {
     uint64_t b = partial[0];
-    for (int w = 1; w < PICK_THREADS / AXON_WAVE; ++w) b = partial[w] > b ? partial[w] : b;
-    // every key of an all-NaN row is (0 << 32 | id): the largest id, n - 1, wins
-    picks[blockIdx.x] = (int32_t)(uint32_t)b;
+    for (int w = 1; w < ARGMAX_THREADS / AXON_WAVE; ++w) b = partial[w] > b ? partial[w] : b;
+    chunk_best[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = b;
   }
 }
 
-extern "C" int axk_argmax(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n, void* stream) {
+__global__ void __launch_bounds__(AXON_WAVE)
+argmax_rows_kernel(const uint64_t* __restrict__ chunk_best, int n_chunks, int32_t* __restrict__ picks) {
+  const uint64_t* mine = chunk_best + (size_t)blockIdx.x * n_chunks;
+  uint64_t best = 0;
+  for (int c = threadIdx.x; c < n_chunks; c += AXON_WAVE) best = mine[c] > best ? mine[c] : best;
+  best = wave_max_u64(best);
+  // every key of an all-NaN row is (0 << 32 | id): the largest id, n - 1, wins
+  if (threadIdx.x == 0) picks[blockIdx.x] = (int32_t)(uint32_t)best;
+}
+
+extern "C" long axk_argmax_workspace(int n_rows, int n) {
+  return (long)sizeof(uint64_t) * (long)(n_rows > 0 ? n_rows : 0) * ceil_div(n > 0 ? n : 1, ARGMAX_CHUNK);
+}
+
+extern "C" int axk_argmax(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n, void* workspace,
+                          void* stream) {
   AXK_REQUIRE(n_rows >= 0 && n > 0 && logits_stride >= n, "argmax: bad sizes rows=%d n=%d stride=%d", n_rows, n,
               logits_stride);
+  AXK_REQUIRE(n_rows <= 65535, "argmax: %d rows are more than one launch takes", n_rows);
+  AXK_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 7) == 0, "argmax: needs its workspace, 8-byte aligned");
   if (n_rows == 0) return 0;
-  argmax_kernel<<<n_rows, PICK_THREADS, 0, (hipStream_t)stream>>>(logits, logits_stride, picks, n);
-  AXK_LAUNCH_CHECK("argmax");
+  const int n_chunks = ceil_div(n, ARGMAX_CHUNK);
+  const int vec = logits_stride % 4 == 0 && ((uintptr_t)logits & 15) == 0;
+  argmax_chunk_kernel<<<dim3(n_chunks, n_rows), ARGMAX_THREADS, 0, (hipStream_t)stream>>>(
+      logits, logits_stride, (uint64_t*)workspace, n, vec);
+  AXK_LAUNCH_CHECK("argmax_chunk");
+  argmax_rows_kernel<<<n_rows, AXON_WAVE, 0, (hipStream_t)stream>>>((const uint64_t*)workspace, n_chunks, picks);
+  AXK_LAUNCH_CHECK("argmax_rows");
   return 0;
 }
 

@@ -48,7 +48,7 @@ _SIGNATURES = {
     "axk_gemm_norm_fold": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                            c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
     "axk_swiglu": [c_void_p, c_void_p, c_int, c_int, c_void_p],
-    "axk_argmax": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "axk_argmax": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p],
     "axk_topk": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                  c_void_p],
     "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
@@ -71,6 +71,8 @@ class Kernels:
             fn.restype = c_int
         self.lib.axk_attention_decode_workspace.argtypes = [c_int, c_int, c_int, c_int]
         self.lib.axk_attention_decode_workspace.restype = ctypes.c_long
+        self.lib.axk_argmax_workspace.argtypes = [c_int, c_int]
+        self.lib.axk_argmax_workspace.restype = ctypes.c_long
         if bool(self.lib.axk_is_bf16()) != (dtype_name == "bfloat16"):
             raise KernelError(f"{self.path} was not built for {dtype_name}")
 
@@ -287,8 +289,9 @@ class Kernels:
         self._i32(out, "argmax out")
         if logits.dtype != torch.float32 or not logits.is_cuda or logits.stride(1) != 1 or out.numel() != logits.shape[0]:
             raise KernelError(f"argmax: logits {tuple(logits.shape)} {logits.dtype}, picks {out.numel()}")
-        self._check(self.lib.axk_argmax(_ptr(logits), logits.stride(0), _ptr(out), logits.shape[0], logits.shape[1],
-                                        _stream()))
+        rows, n = logits.shape
+        work = torch.empty(max(1, self.lib.axk_argmax_workspace(rows, n) // 8), dtype=torch.int64, device=logits.device)
+        self._check(self.lib.axk_argmax(_ptr(logits), logits.stride(0), _ptr(out), rows, n, _ptr(work), _stream()))
         return out
 
     def topk(self, logits, recent, n_recent, penalty, k_of_row, cands) -> torch.Tensor:

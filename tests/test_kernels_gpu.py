@@ -309,6 +309,9 @@ def test_argmax_rules_on_the_device():
     out = torch.empty(3, dtype=torch.int32, device="cuda")
     k.argmax(big, out)
     assert out.tolist() == [int(big[0].argmax()), 150000, int(big[2].argmax())]
+    for view in (big[:, 1:9000], big[:, 4096:12288], big[:, :4097]):           # unaligned rows, whole chunks, one over
+        k.argmax(view, out)
+        assert out.tolist() == [P.argmax_last(r) for r in view.cpu().tolist()]
 
 
 def test_topk_with_penalty_on_the_device():
