@@ -278,11 +278,34 @@ struct NormFold {
   float* norm_squares;
 };
 
-template <int NT16, int MT16, int WAVES, int DEPTH, bool GLU>
+// The product of the attention's fused [q; k; v] matrix with the rotary position encoding and the
+// store into the paged cache as its epilogue (EPI_ROPE, NT16 = 2): W's rows are heads of
+// head_dim; a block owns dims d0 .. d0 + 15 of one head and their rotation partners d0 + half ..,
+// so that a lane ends with both values of a pair.  q heads go rotated to `out`, k heads rotated
+// into the request's page of keys, v heads as they are into its page of values (kept
+// position-contiguous, [dim][slot]).  The arithmetic is that of the rotary kernel after a
+// plain product: the sums are rounded to bfloat16 first, and each product and sum of the
+// rotation is rounded on its own.
+struct RopeStore {
+  const float* table;            // [M, half, 2]: sin, cos of each token's angles
+  const int32_t* positions;      // [M]
+  const int32_t* seq_rows;       // [M]: the row of the block table
+  const int32_t* block_table;
+  int table_stride;
+  bf16_t* k_cache;
+  bf16_t* v_cache;
+  int n_heads, n_kv_heads, head_dim, page_size;
+};
+
+enum { EPI_PLAIN = 0, EPI_GLU = 1, EPI_ROPE = 2 };
+
+template <int NT16, int MT16, int WAVES, int DEPTH, int EPI>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w,
                    const void* __restrict__ bias, int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N,
-                   int K, int mode, NormFold fold) {
+                   int K, int mode, NormFold fold, RopeStore rope) {
+  constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE;
+  static_assert(EPI == EPI_PLAIN || NT16 == 2, "the paired epilogues own two tiles of W rows");
   __shared__ float partial[WAVES][NT16 * MT16][64][4];
   __shared__ float row_scale[MT16 * 16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -292,7 +315,12 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
   const bf16_t* wrow[NT16];
 #pragma unroll
   for (int i = 0; i < NT16; ++i) {
-    const int row = GLU ? i * N + min(n0 + r16, N - 1) : min(n0 + i * 16 + r16, N - 1);
+    int row;
+    if (GLU) row = i * N + min(n0 + r16, N - 1);
+    else if (ROPE) {
+      const int half = rope.head_dim / 2, per_head = half / 16;
+      row = (blockIdx.x / per_head) * rope.head_dim + i * half + (blockIdx.x % per_head) * 16 + r16;
+    } else row = min(n0 + i * 16 + r16, N - 1);
     wrow[i] = w + (size_t)row * K + kq;
   }
   const bf16_t* xrow[MT16];
@@ -402,6 +430,73 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
       for (int e = 0; e < 4; ++e) partial[wave][i * MT16 + j][lane][e] = acc[i][j][e];
   __syncthreads();
 
+  if (ROPE) {
+    const int hd = rope.head_dim, half = hd / 2, per_head = half / 16;
+    const int slot = blockIdx.x / per_head;                  // q heads, then k heads, then v heads
+    const int d = (blockIdx.x % per_head) * 16 + (lane >> 4) * 4;
+    for (int j = wave; j < MT16; j += WAVES) {
+      const int m = j * 16 + r16;
+      if (m >= M) continue;
+      const float scale = fold.in_squares ? row_scale[m] : 1.0f;
+      float a[4], b[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float lo = partial[0][j][lane][e], hi = partial[0][MT16 + j][lane][e];
+#pragma unroll
+        for (int q = 1; q < WAVES; ++q) {
+          lo += partial[q][j][lane][e];
+          hi += partial[q][MT16 + j][lane][e];
+        }
+        if (fold.in_squares) {
+          lo *= scale;
+          hi *= scale;
+        }
+        if (bias) {
+          lo += load_vec(bias, bias_is_f32, slot * hd + d + e);
+          hi += load_vec(bias, bias_is_f32, slot * hd + half + d + e);
+        }
+        a[e] = bf16_to_float(float_to_bf16(lo));
+        b[e] = bf16_to_float(float_to_bf16(hi));
+      }
+      bf16_t* dst;
+      if (slot < rope.n_heads) {
+        dst = reinterpret_cast<bf16_t*>(out) + (size_t)m * out_stride + (size_t)slot * hd;
+      } else {
+        const int pos = rope.positions[m];
+        const int page = rope.block_table[(size_t)rope.seq_rows[m] * rope.table_stride + pos / rope.page_size];
+        const int in_page = pos % rope.page_size;
+        if (slot >= rope.n_heads + rope.n_kv_heads) {
+          const int kvh = slot - rope.n_heads - rope.n_kv_heads;
+          bf16_t* vdst = rope.v_cache + ((size_t)page * rope.n_kv_heads + kvh) * hd * rope.page_size + in_page;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            vdst[(size_t)(d + e) * rope.page_size] = float_to_bf16(a[e]);
+            vdst[(size_t)(half + d + e) * rope.page_size] = float_to_bf16(b[e]);
+          }
+          continue;
+        }
+        const int kvh = slot - rope.n_heads;
+        dst = rope.k_cache + (((size_t)page * rope.n_kv_heads + kvh) * rope.page_size + in_page) * hd;
+      }
+      const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * half + d) * 2);
+      const float4 t0 = tab[0], t1 = tab[1];
+      const float sn[4] = {t0.x, t0.z, t1.x, t1.z}, cs[4] = {t0.y, t0.w, t1.y, t1.w};
+      float lo[4], hi[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo[e] = __fsub_rn(__fmul_rn(a[e], cs[e]), __fmul_rn(b[e], sn[e]));
+        hi[e] = __fadd_rn(__fmul_rn(a[e], sn[e]), __fmul_rn(b[e], cs[e]));
+      }
+      uint2 pk;
+      pk.x = pack2_bf16(lo[0], lo[1]);
+      pk.y = pack2_bf16(lo[2], lo[3]);
+      *reinterpret_cast<uint2*>(dst + d) = pk;
+      pk.x = pack2_bf16(hi[0], hi[1]);
+      pk.y = pack2_bf16(hi[2], hi[3]);
+      *reinterpret_cast<uint2*>(dst + half + d) = pk;
+    }
+    return;
+  }
   if (GLU) {
     // a wave takes both tiles of a column block: gate (tile j) and up (tile MT16 + j)
     for (int j = wave; j < MT16; j += WAVES) {
@@ -469,11 +564,12 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
   }
 }
 
-template <int NT16, int MT16, int WAVES, int DEPTH, bool GLU = false>
+template <int NT16, int MT16, int WAVES, int DEPTH, int EPI = EPI_PLAIN>
 static int launch_skinny(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                         int out_stride, int m, int n, int k, int mode, hipStream_t stream, const NormFold& fold) {
-  gemm_skinny_kernel<NT16, MT16, WAVES, DEPTH, GLU><<<ceil_div(n, GLU ? 16 : NT16 * 16), WAVES * 64, 0, stream>>>(
-      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, fold);
+                         int out_stride, int m, int n, int k, int mode, hipStream_t stream, const NormFold& fold,
+                         const RopeStore& rope = RopeStore()) {
+  gemm_skinny_kernel<NT16, MT16, WAVES, DEPTH, EPI><<<ceil_div(n, EPI == EPI_GLU ? 16 : NT16 * 16), WAVES * 64, 0, stream>>>(
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, fold, rope);
   AXK_LAUNCH_CHECK("gemm_skinny");
   return 0;
 }
@@ -507,9 +603,9 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
   }
 #define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream
   if (m <= 64 && mode == MODE_SWIGLU) {
-    if (m <= 16) return launch_skinny<2, 1, 4, 8, true>(ARGS, fold);
-    if (m <= 32) return launch_skinny<2, 2, 4, 4, true>(ARGS, fold);
-    return launch_skinny<2, 4, 4, 2, true>(ARGS, fold);
+    if (m <= 16) return launch_skinny<2, 1, 4, 8, EPI_GLU>(ARGS, fold);
+    if (m <= 32) return launch_skinny<2, 2, 4, 4, EPI_GLU>(ARGS, fold);
+    return launch_skinny<2, 4, 4, 2, EPI_GLU>(ARGS, fold);
   }
   if (skinny_takes(m, n, k, mode)) {
     // 32 rows of W per block where that still leaves 128 blocks or more, else 16; four waves
@@ -536,6 +632,27 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
   }
   if ((long)ceil_div(m, 256) * ceil_div(n, 256) >= 512) return launch_tile<256, 256, 4, 2, false>(ARGS);
   return launch_tile<128, 128, 2, 2, false>(ARGS);
+#undef ARGS
+}
+
+// The [q; k; v] product with rotary encoding and cache store (see RopeStore): up to 64 rows,
+// every head rotated over its whole width, halves of a head a multiple of 16 wide.
+int gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim) {
+  return m >= 1 && m <= 64 && k % 64 == 0 && rotary_dim == head_dim && head_dim % 32 == 0;
+}
+
+int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out,
+                         int out_stride, int m, int n, int k, const float* in_squares, float in_eps,
+                         const float* table, const int32_t* positions, const int32_t* seq_rows,
+                         const int32_t* block_table, int table_stride, bf16_t* k_cache, bf16_t* v_cache, int n_heads,
+                         int n_kv_heads, int head_dim, int page_size, hipStream_t stream) {
+  const NormFold fold = {in_squares, in_eps, nullptr, 0, nullptr, nullptr};
+  const RopeStore rope = {table, positions, seq_rows, block_table, table_stride, k_cache, v_cache,
+                          n_heads, n_kv_heads, head_dim, page_size};
+#define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream, fold, rope
+  if (m <= 16) return launch_skinny<2, 1, 4, 8, EPI_ROPE>(ARGS);
+  if (m <= 32) return launch_skinny<2, 2, 4, 4, EPI_ROPE>(ARGS);
+  return launch_skinny<2, 4, 4, 2, EPI_ROPE>(ARGS);
 #undef ARGS
 }
 

@@ -36,6 +36,10 @@ _SIGNATURES = {
     "axk_rope_table": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_rope_kv_write": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "axk_gemm_qkv_rope_ok": [c_int, c_int, c_int, c_int],
+    "axk_gemm_qkv_rope": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_float,
+                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                          c_int, c_void_p],
     "axk_attention": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
                       c_int, c_int, c_int, c_int, c_float, c_void_p],
     "axk_attention_prefill": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
@@ -166,6 +170,39 @@ class Kernels:
             _ptr(qkv), _ptr(table), _ptr(positions), _ptr(seq_rows), _ptr(block_table), block_table.shape[-1],
             _ptr(k_cache if write_kv else None), _ptr(v_cache if write_kv else None), T, n_heads, n_kv_heads, head_dim,
             rotary_dim, page_size, 1 if write_kv else 0, _stream()))
+
+    def gemm_qkv_rope_ok(self, m: int, k: int, head_dim: int, rotary_dim: int) -> bool:
+        """Whether `gemm_qkv_rope` takes a step of m tokens and these sizes."""
+        return bool(self.lib.axk_gemm_qkv_rope_ok(m, k, head_dim, rotary_dim))
+
+    def gemm_qkv_rope(self, x, w, bias, qkv, table, positions, seq_rows, block_table, k_cache, v_cache, n_heads,
+                      n_kv_heads, head_dim, page_size, write_kv=True, row_squares=None, eps=0.0) -> None:
+        """The [q; k; v] product, the rotary encoding and the store into the pages in one launch:
+        the same bits as `gemm` into qkv followed by `rope_kv_write`.  q lands in qkv[:, :n_heads *
+        head_dim]; the k and v columns of qkv are not written.  Without write_kv, w holds the q
+        rows only.  row_squares, eps: as in `gemm`."""
+        self._elem(x, "qkv x"); self._elem(w, "qkv w"); self._elem(qkv, "qkv out"); self._f32(table, "rope table")
+        self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
+        M, K = x.shape
+        rows = (n_heads + (2 * n_kv_heads if write_kv else 0)) * head_dim
+        if w.shape != (rows, K) or not w.is_contiguous() or x.stride(1) != 1:
+            raise KernelError(f"gemm_qkv_rope: x {tuple(x.shape)} w {tuple(w.shape)}, expected w [{rows}, {K}]")
+        if qkv.shape[0] != M or qkv.shape[1] < n_heads * head_dim or qkv.stride(1) != 1:
+            raise KernelError(f"gemm_qkv_rope: qkv {tuple(qkv.shape)} does not hold [{M}, {n_heads * head_dim}]")
+        if table.shape != (M, head_dim // 2, 2) or positions.numel() != M or seq_rows.numel() != M:
+            raise KernelError(f"gemm_qkv_rope: table {tuple(table.shape)} or positions do not fit {M} tokens")
+        if bias is not None and bias.numel() != rows:
+            raise KernelError(f"gemm_qkv_rope: bias of {bias.numel()} for {rows} rows")
+        if row_squares is not None and (row_squares.dtype != torch.float32 or not row_squares.is_contiguous()
+                                        or row_squares.shape != (M, K // 16) or not row_squares.is_cuda):
+            raise KernelError(f"gemm_qkv_rope: row_squares {tuple(row_squares.shape)} is not float32 [{M}, {K // 16}]")
+        if write_kv:
+            self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
+        self._check(self.lib.axk_gemm_qkv_rope(
+            _ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "qkv bias"), _ptr(qkv), qkv.stride(0), M, K,
+            _ptr(row_squares), float(eps), _ptr(table), _ptr(positions), _ptr(seq_rows), _ptr(block_table),
+            block_table.shape[-1], _ptr(k_cache if write_kv else None), _ptr(v_cache if write_kv else None), n_heads,
+            n_kv_heads, head_dim, page_size, 1 if write_kv else 0, _stream()))
 
     def attention(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, n_heads, n_kv_heads,
                   head_dim, page_size, window, scale) -> torch.Tensor:

@@ -162,20 +162,24 @@ class GQAttention(Mixer):
         # values are kept position-contiguous: a page of them is [heads, head_dim, page_size]
         v_cache = v_cache.view(v_cache.shape[0], self.nkv, self.hd, group.page_size)
         mark = ctx.ws.mark()
-        if binding.writes:
-            qkv = ctx.ws.take((T, self.q_dim + 2 * self.kv_dim), ctx.rt.dtype)
-            k.gemm(h, self.w_qkv, qkv, self.b_qkv, MODE_STORE, **scaled)
-        else:
-            # reading another run's cache: only the queries are needed
-            qkv = ctx.ws.take((T, self.q_dim + 2 * self.kv_dim), ctx.rt.dtype)
-            bias = None if self.b_qkv is None else self.b_qkv[:self.q_dim]
-            k.gemm(h, self.w_qkv[:self.q_dim], qkv[:, :self.q_dim], bias, MODE_STORE, **scaled)
+        qkv = ctx.ws.take((T, self.q_dim + 2 * self.kv_dim), ctx.rt.dtype)
         if self.position is not None:
             table, rotary = self.position.tables(ctx), self.position.rotary_dim
         else:
             table, rotary = ctx.no_rotation(), 0
-        k.rope_kv_write(qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache, self.nh, self.nkv,
-                        self.hd, rotary, group.page_size, binding.writes)
+        if binding.writes:
+            w, bias = self.w_qkv, self.b_qkv
+        else:
+            # reading another run's cache: only the queries are needed
+            w, bias = self.w_qkv[:self.q_dim], None if self.b_qkv is None else self.b_qkv[:self.q_dim]
+        if k.gemm_qkv_rope_ok(T, self.hidden, self.hd, rotary):
+            # a short step: product, rotation and the store into the pages in one launch
+            k.gemm_qkv_rope(h, w, bias, qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache,
+                            self.nh, self.nkv, self.hd, group.page_size, binding.writes, **scaled)
+        else:
+            k.gemm(h, w, qkv[:, :w.shape[0]], bias, MODE_STORE, **scaled)
+            k.rope_kv_write(qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache, self.nh,
+                            self.nkv, self.hd, rotary, group.page_size, binding.writes)
         att = ctx.ws.take((T, self.q_dim), ctx.rt.dtype)
         if k.attention_fast_ok(self.hd, group.page_size, self.nh, self.nkv):
             plan = attention_plan(ctx, self.window, self.nh, self.hd)

@@ -255,6 +255,50 @@ def test_gemm_with_a_norm_folded_in(M, H, F):
         assert (out.cpu().double() - want).abs().max() <= tol("bfloat16", want, 0, 1e-2)
 
 
+@pytest.mark.parametrize("M,nh,nkv,hd,hidden,page", [(1, 4, 2, 32, 64, 8), (8, 6, 2, 64, 192, 16), (16, 7, 1, 128, 256, 8),
+                                                      (17, 3, 3, 96, 128, 4), (40, 4, 1, 64, 320, 32),
+                                                      (64, 2, 2, 128, 64, 16)])
+def test_qkv_product_with_rotation_and_cache_store_in_one(M, nh, nkv, hd, hidden, page):
+    """The fused launch against the product followed by the rotary kernel: the same bits in q, in
+    the pages of keys and in the pages of values; other pages untouched."""
+    k = kernels("bfloat16")
+    assert k.gemm_qkv_rope_ok(M, hidden, hd, hd)
+    assert not k.gemm_qkv_rope_ok(M, hidden, hd, hd // 2) and not k.gemm_qkv_rope_ok(65, hidden, hd, hd)
+    assert not k.gemm_qkv_rope_ok(M, hidden, 48, 48) and not kernels("float32").gemm_qkv_rope_ok(M, hidden, hd, hd)
+    width = (nh + 2 * nkv) * hd
+    x, _ = as_dtype(rnd(M, hidden, seed=50), "bfloat16")
+    w, _ = as_dtype(rnd(width, hidden, seed=51, scale=0.2), "bfloat16")
+    g = torch.Generator().manual_seed(52)
+    # tokens of three requests at scattered positions, every (request, position) once
+    n_pages, max_pages = 40, 8
+    slots = torch.randperm(3 * max_pages * page, generator=g)[:M]
+    rows = (slots // (max_pages * page)).to(torch.int32)
+    pos = (slots % (max_pages * page)).to(torch.int32)
+    table_of_pages = torch.randperm(n_pages, generator=g)[:3 * max_pages].view(3, max_pages).to(torch.int32).cuda()
+    freqs = P.rope_freqs(hd, 10000.0).cuda()
+    table = torch.empty(M, hd // 2, 2, dtype=torch.float32, device="cuda")
+    k.rope_table(pos.cuda(), freqs, table)
+    for bias_dt, write_kv in ((None, True), (torch.float32, True), (torch.bfloat16, False)):
+        bias = None if bias_dt is None else rnd(width, seed=53).to(bias_dt).cuda()
+        n_rows = width if write_kv else nh * hd
+        ww, bb = w[:n_rows], (None if bias is None else bias[:n_rows])
+        got, want = [], []
+        for fused in (True, False):
+            kc = torch.full((n_pages, nkv, page, hd), 7.0, dtype=torch.bfloat16, device="cuda")
+            vc = torch.full((n_pages, nkv, hd, page), 7.0, dtype=torch.bfloat16, device="cuda")
+            qkv = torch.zeros(M, width, dtype=torch.bfloat16, device="cuda")
+            if fused:
+                k.gemm_qkv_rope(x, ww, bb, qkv, table, pos.cuda(), rows.cuda(), table_of_pages, kc, vc, nh, nkv, hd, page,
+                                write_kv)
+            else:
+                k.gemm(x, ww, qkv[:, :n_rows], bb, MODE_STORE)
+                k.rope_kv_write(qkv, table, pos.cuda(), rows.cuda(), table_of_pages, kc, vc, nh, nkv, hd, hd, page, write_kv)
+            (got if fused else want).extend([qkv[:, :nh * hd].clone(), kc, vc])
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+        assert write_kv == bool((got[1] != 7.0).any())
+
+
 def test_gemm_refuses_a_norm_it_cannot_fold():
     k = kernels("bfloat16")
     assert not k.gemm_norm_fold_ok(17, 64, 64, MODE_STORE)          # more rows than a folded step takes
