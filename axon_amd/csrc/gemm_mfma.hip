@@ -44,6 +44,33 @@ __device__ inline void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+template <int N>
+__device__ inline void wait_lgkmcnt() {
+  asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// COUNT reads of 16 bytes a lane from LDS, STEP bytes apart, written as instructions (see
+// gemm_tile_kernel).  Their results may be used only after wait_lgkmcnt and use_frags.
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+
+template <int COUNT, int STEP>
+__device__ inline void read_frags(u32x4 (&dst)[COUNT], unsigned lds_address) {
+  static_assert((COUNT - 1) * STEP < 65536, "the offset field of an LDS read");
+#pragma unroll
+  for (int i = 0; i < COUNT; ++i)
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst[i]) : "v"(lds_address), "n"(i * STEP));
+}
+
+// Ties the registers to this point of the program: what uses them afterwards stays behind
+// the wait that precedes this.
+template <int COUNT>
+__device__ inline void use_frags(u32x4 (&regs)[COUNT]) {
+#pragma unroll
+  for (int i = 0; i < COUNT; ++i) asm volatile("" : "+v"(regs[i]));
+}
+
+__device__ inline bf16x8 as_frag(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+
 // ---------------------------------------------------------------------------- gemm_tile
 // LDS holds STAGES stages; a stage is BM rows of X and BN rows of W, BK k each, written by
 // direct global -> LDS loads of 16 bytes per lane (a wave instruction fills 1024 bytes of
@@ -143,48 +170,67 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
 
   // fragment addresses: row = tile row + lane % 32, k chunk = 2 ks + lane / 32, slot = chunk ^ SWZ(row)
   const int frow = lane & 31, fhalf = lane >> 5, fsw = SWZ(frow);
-  const int xbase = (wm * WM + frow) * ROW;
-  const int wbase = (BM + wn * WN + frow) * ROW;
+  const unsigned lds0 = (unsigned)(size_t)(lds_ptr_t)smem;
+  const unsigned xbase = lds0 + (wm * WM + frow) * ROW;
+  const unsigned wbase = lds0 + (BM + wn * WN + frow) * ROW;
+  // The fragments of k step ks of a stage into one of two register sets.  The reads are written
+  // as instructions: the compiler, which cannot tell the stage being read from the stage a
+  // direct load is filling, would wait for every load in flight before each of its own reads,
+  // and the loads of the next tile would never overlap the products of this one.
+  u32x4 a[2][TM], b[2][TN];
+  auto read_step = [&](int set, int stage_index, int ks) {
+    const unsigned at = stage_index * STAGE + ((((ks * 2 + fhalf) ^ fsw)) << 4);
+    read_frags<TM, 32 * ROW>(a[set], xbase + at);
+    read_frags<TN, 32 * ROW>(b[set], wbase + at);
+  };
+  auto multiply = [&](int set, int j_from, int j_to) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = j_from; j < j_to; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(a[set][i]), as_frag(b[set][j]), acc[i][j], 0, 0, 0);
+  };
 
+  // Every stage is filled before the loop; tile kt + STAGES is fetched into tile kt's stage as
+  // soon as every wave has read that tile's last fragments, which is during its last k step:
+  // the wait for the next tile, the barrier and the first reads of the next tile are hidden
+  // behind that step's products (half of them before the barrier, half after the reads).
   const int nk = K / BK;
+  constexpr int KS = BK / 16;
+  static_assert(KS % 2 == 0, "the register sets alternate and start a tile at set 0");
 #pragma unroll
-  for (int d = 0; d < STAGES - 1; ++d)
+  for (int d = 0; d < STAGES; ++d)
     if (d < nk) issue(d);
+  if (nk >= STAGES) wait_vmcnt<(STAGES - 1) * (XQ + WQ)>();
+  else wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();   // tile 0 is in LDS for every wave
+  read_step(0, 0, 0);
   for (int kt = 0; kt < nk; ++kt) {
-    // tile kt has landed when only the loads of the STAGES - 2 younger tiles are outstanding
-    if (kt + STAGES - 2 < nk) wait_vmcnt<(STAGES - 2) * (XQ + WQ)>();
-    else wait_vmcnt<0>();
-    __syncthreads();  // tile kt is in LDS for every wave, and every wave is done with tile kt - 1
-    if (kt + STAGES - 1 < nk) issue(kt + STAGES - 1);  // into the stage that tile kt - 1 has left
-    const unsigned char* stage = smem + (kt % STAGES) * STAGE;
-    bf16x8 a[2][TM], b[2][TN];
-    {
-      const int slot = ((0 + fhalf) ^ fsw) << 4;
+    const int stage_index = kt % STAGES;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a[0][i] = as_frag(*reinterpret_cast<const uint4*>(stage + xbase + i * 32 * ROW + slot));
-#pragma unroll
-      for (int j = 0; j < TN; ++j) b[0][j] = as_frag(*reinterpret_cast<const uint4*>(stage + wbase + j * 32 * ROW + slot));
-    }
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
+    for (int ks = 0; ks < KS; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks + 1 < BK / 16) {
-        const int slot = (((ks + 1) * 2 + fhalf) ^ fsw) << 4;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-          a[nxt][i] = as_frag(*reinterpret_cast<const uint4*>(stage + xbase + i * 32 * ROW + slot));
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          b[nxt][j] = as_frag(*reinterpret_cast<const uint4*>(stage + wbase + j * 32 * ROW + slot));
+      if (ks + 1 < KS) {
+        read_step(nxt, stage_index, ks + 1);
+        wait_lgkmcnt<TM + TN>();          // this step's fragments (reads return in order)
+        use_frags<TM>(a[cur]);
+        use_frags<TN>(b[cur]);
+        multiply(cur, 0, TN);
+      } else {
+        wait_lgkmcnt<0>();                // the last fragments of this tile: its stage is free
+        use_frags<TM>(a[cur]);
+        use_frags<TN>(b[cur]);
+        multiply(cur, 0, TN / 2);
+        if (kt + 1 < nk) {
+          // this wave's part of tile kt + 1 has landed when only younger tiles are outstanding
+          if (kt + STAGES < nk) wait_vmcnt<(STAGES - 2) * (XQ + WQ)>();
+          else wait_vmcnt<0>();
+          __builtin_amdgcn_s_barrier();   // tile kt + 1 is in LDS for every wave; nobody reads tile kt any more
+          if (kt + STAGES < nk) issue(kt + STAGES);
+          read_step(nxt, (kt + 1) % STAGES, 0);
+        }
+        multiply(cur, TN / 2, TN);
       }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
-      // let the scheduler interleave the next step's fragment reads with this step's MFMAs (its
-      // strategy for small matrix-multiply loops measured best here)
-      __builtin_amdgcn_iglp_opt(1);
     }
   }
 #undef SWZ
@@ -625,12 +671,18 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
     *handled = false;
     return 0;
   }
-  // 256 x 256 tiles (8 waves) when they still give every CU two blocks; else 128 x 128
+  // 256 x 256 tiles (8 waves) where they fill the chip: one round of at least 140 blocks (on 256
+  // CUs), or several rounds of which the last is not mostly idle; else 128 x 128 tiles, four times
+  // as many blocks at twice the traffic from L2 per product.  Thresholds are measured ones.
+  const int n_per_block = mode == MODE_SWIGLU ? 128 : 256;
+  const long big = (long)ceil_div(m, 256) * ceil_div(n, n_per_block);
+  const long rounds = (big + 255) / 256;
+  const bool use_big = big <= 256 ? big >= 140 : big * 10 >= rounds * 256 * 7;
   if (mode == MODE_SWIGLU) {
-    if ((long)ceil_div(m, 256) * ceil_div(n, 128) >= 512) return launch_tile<256, 256, 4, 2, true>(ARGS);
+    if (use_big) return launch_tile<256, 256, 4, 2, true>(ARGS);
     return launch_tile<128, 128, 2, 2, true>(ARGS);
   }
-  if ((long)ceil_div(m, 256) * ceil_div(n, 256) >= 512) return launch_tile<256, 256, 4, 2, false>(ARGS);
+  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS);
   return launch_tile<128, 128, 2, 2, false>(ARGS);
 #undef ARGS
 }
