@@ -53,7 +53,7 @@ __device__ inline uint32_t pack_bf16(float a, float b) { return pack2_bf16(a, b)
 #define PF_BLOCK 64
 
 template <int HD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
                          const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
@@ -98,6 +98,23 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
   }
 
   const size_t kv_head_stride = (size_t)HD * page_size;           // elements of one (page, kv head)
+  // The pages a block of positions lies in are looked up one block ahead of the loads that use
+  // them, so that no load waits for a table entry behind the loads issued just before it.
+  int k_page[K_INSTR], v_page[V_INSTR];
+  auto lookup = [&](int b) {
+    const int p0 = first_block + b * PF_BLOCK;
+#pragma unroll
+    for (int n = 0; n < K_INSTR; ++n) {
+      const int row = (n * 4 + wave) * K_ROWS_PER_INSTR + lane / KCH;
+      k_page[n] = table_row[min(p0 + row, hi) / page_size];       // rows past the tile's last position: any valid row
+    }
+#pragma unroll
+    for (int n = 0; n < V_INSTR; ++n) {
+      const int d = (n * 4 + wave) * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ (d & 7);
+      v_page[n] = table_row[min(p0 + chunk * 8, hi) / page_size];
+    }
+  };
   auto issue = [&](int b) {
     unsigned char* stage = smem + (b & 1) * STAGE;
     const int p0 = first_block + b * PF_BLOCK;
@@ -107,8 +124,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
       const int instr = n * 4 + wave;
       const int row = instr * K_ROWS_PER_INSTR + lane / KCH;
       const int chunk = (lane % KCH) ^ (row & 7);
-      const int p = min(p0 + row, hi);                            // rows past the tile's last position: any valid row
-      const bf16_t* src = k_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * kv_head_stride +
+      const int p = min(p0 + row, hi);
+      const bf16_t* src = k_cache + ((size_t)k_page[n] * n_kv_heads + kvh) * kv_head_stride +
                           (size_t)(p % page_size) * HD + chunk * 8;
       __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + instr * 1024), 16, 0, 0);
     }
@@ -119,7 +136,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
       const int d = instr * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ (d & 7);
       const int p = min(p0 + chunk * 8, hi);
-      const bf16_t* src = v_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * kv_head_stride +
+      const bf16_t* src = v_cache + ((size_t)v_page[n] * n_kv_heads + kvh) * kv_head_stride +
                           (size_t)d * page_size + ((p % page_size) & ~7);
       __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + K_BYTES + instr * 1024), 16, 0, 0);
     }
@@ -133,12 +150,26 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
   float m_run = -INFINITY, l_run = 0.0f;
   const float c = scale * LOG2E;
 
+  // Fragment reads are written as instructions (see common.h).  Row r of an S^T tile is key
+  // position pi(r) of the tile, pi swapping bits 2 and 3 of r: a lane then ends with weights of
+  // 8 CONSECUTIVE positions per k step of O^T, which are one 16-byte read of a V^T row.
+  const unsigned lds0 = (unsigned)(size_t)(lds_ptr_t)smem;
+  const int k_row = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);
+  const unsigned k_at = lds0 + k_row * KROW, k_swz = k_row & 7;
+  const unsigned v_at = lds0 + K_BYTES + l32 * 128, v_swz = l32 & 7;
+
+  lookup(0);
   issue(0);
+  if (n_blocks > 1) lookup(1);
   for (int b = 0; b < n_blocks; ++b) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (b + 1 < n_blocks) issue(b + 1);
+    wait_vmcnt<0>();                  // this wave's part of block b has landed
+    __builtin_amdgcn_s_barrier();     // so has everyone's, and everyone is done with block b - 1
+    if (b + 1 < n_blocks) {
+      issue(b + 1);                   // into the stage block b - 1 has left, under way during block b's products
+      if (b + 2 < n_blocks) lookup(b + 2);
+    }
     unsigned char* stage = smem + (b & 1) * STAGE;
+    const unsigned st = (b & 1) * STAGE;
     const int p0 = first_block + b * PF_BLOCK;
     if (p0 + PF_BLOCK - 1 > hi) {
       // the last block: positions past `hi` were never written for this request.  Their
@@ -155,25 +186,49 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
     }
     if (!wave_live || p0 > wave_hi) continue;  // nothing for this wave's rows in this block (all waves reach the barriers)
 
-    // S^T [64 positions][32 queries] = K Q^T: two tiles of 32 positions
+    // S^T [64 positions][32 queries] = K Q^T: two tiles of 32 positions, two k steps a group
     f32x16 s_acc[2];
 #pragma unroll
     for (int pt = 0; pt < 2; ++pt)
 #pragma unroll
       for (int e = 0; e < 16; ++e) s_acc[pt][e] = 0.0f;
+    u32x4 kf[2][4];
+    auto read_k = [&](u32x4 (&dst)[4], int ks0) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-      for (int pt = 0; pt < 2; ++pt) {
-        const int row = pt * 32 + l32;
-        const int slot = (ks * 2 + half) ^ (row & 7);
-        const bf16x8 kf = frag_of(*reinterpret_cast<const uint4*>(stage + row * KROW + slot * 16));
-        s_acc[pt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s_acc[pt], 0, 0, 0);
+      for (int kk = 0; kk < 2; ++kk) {
+        const unsigned at = k_at + st + ((((ks0 + kk) * 2 + half) ^ k_swz) << 4);
+        lds_read16<0>(dst[kk * 2 + 0], at);
+        lds_read16<32 * KROW>(dst[kk * 2 + 1], at);
       }
+    };
+    read_k(kf[0], 0);
+#pragma unroll
+    for (int g = 0; g < KS / 2; ++g) {
+      if (g + 1 < KS / 2) {
+        read_k(kf[(g + 1) & 1], 2 * (g + 1));
+        wait_lgkmcnt<4>();
+      } else {
+        wait_lgkmcnt<0>();
+      }
+      use_frags<4>(kf[g & 1]);
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int pt = 0; pt < 2; ++pt)
+          s_acc[pt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[g & 1][kk * 2 + pt]),
+                                                              qf[2 * g + kk], s_acc[pt], 0, 0, 0);
     }
-    // this lane: query my_row; positions p0 + pt*32 + (e/4)*8 + half*4 + e%4.  A block that every
-    // row of the wave sees whole needs no mask (all but the blocks on the diagonal and at the
-    // window's edge).
+    // V^T fragments of the first k step of O^T: on their way during the softmax
+    u32x4 vf[2][DT];
+    auto read_v = [&](u32x4 (&dst)[DT], int s2) {
+      const unsigned chunk = (s2 >> 1) * 4 + (s2 & 1) * 2 + half;
+      read_frags<DT, 32 * 128>(dst, v_at + st + ((chunk ^ v_swz) << 4));
+    };
+    read_v(vf[0], 0);
+
+    // this lane: query my_row; register e of tile pt is position
+    // p0 + 32 pt + 16 (e / 8) + 8 half + (e % 8).  A block that every row of the wave sees whole
+    // needs no mask (all but the blocks on the diagonal and at the window's edge).
     const bool whole = p0 + PF_BLOCK - 1 <= pos0 + wave * 32 && p0 >= wave_lo;
     float mloc = -INFINITY;
     if (whole) {
@@ -190,7 +245,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
       for (int pt = 0; pt < 2; ++pt)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const int p = p0 + pt * 32 + (e >> 2) * 8 + half * 4 + (e & 3);
+          const int p = p0 + pt * 32 + (e >> 3) * 16 + half * 8 + (e & 7);
           const bool seen = p <= my_pos && p >= my_lo;
           const float v = seen ? s_acc[pt][e] * c : -INFINITY;
           s_acc[pt][e] = v;
@@ -220,24 +275,25 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
         for (int e = 0; e < 16; ++e) o_acc[i][e] *= alpha;
     }
 
-    // O^T [HD][32 queries] += V^T P^T.  k step s2 (16 positions) takes registers e = 8 (s2 % 2) ..
-    // + 7 of tile s2 / 2: positions (s2/2)*32 + (s2%2)*16 + half*4 + {0..3} and the same + 8.
+    // O^T [HD][32 queries] += V^T P^T.  k step s2 (16 positions) takes registers 8 (s2 % 2) .. + 7
+    // of tile s2 / 2: the 8 consecutive positions 32 (s2 / 2) + 16 (s2 % 2) + 8 half + {0..7}.
 #pragma unroll
     for (int s2 = 0; s2 < 4; ++s2) {
+      if (s2 + 1 < 4) {
+        read_v(vf[(s2 + 1) & 1], s2 + 1);
+        wait_lgkmcnt<DT>();
+      } else {
+        wait_lgkmcnt<0>();
+      }
+      use_frags<DT>(vf[s2 & 1]);
       const int pt = s2 >> 1, e0 = (s2 & 1) * 8;
       union { uint32_t u[4]; bf16x8 f; } pf;
 #pragma unroll
       for (int j = 0; j < 4; ++j) pf.u[j] = pack_bf16(s_acc[pt][e0 + 2 * j], s_acc[pt][e0 + 2 * j + 1]);
-      const int col = pt * 32 + (s2 & 1) * 16 + half * 4;   // first of the lane's 4 + 4 positions
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const int d = dt * 32 + l32;
-        const unsigned char* vrow = stage + K_BYTES + d * 128 + (col & 7) * 2;
-        const int ch = col >> 3;
-        const uint2 v0 = *reinterpret_cast<const uint2*>(vrow + ((ch ^ (d & 7)) << 4));
-        const uint2 v1 = *reinterpret_cast<const uint2*>(vrow + (((ch + 1) ^ (d & 7)) << 4));
-        o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_of2(v0, v1), pf.f, o_acc[dt], 0, 0, 0);
-      }
+      for (int dt = 0; dt < DT; ++dt)
+        o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[s2 & 1][dt]), pf.f, o_acc[dt], 0,
+                                                            0, 0);
     }
   }
 

@@ -105,6 +105,47 @@ __device__ inline float wave_max(float v) {
   return v;
 }
 
+// ---------------------------------------------------------------------------- LDS reads as instructions
+// A kernel that fills LDS with direct global -> LDS loads while it reads other parts of LDS has
+// to write those reads as instructions: the compiler cannot tell the part being read from the
+// part a load is filling, and would wait for every load in flight before each read of its own,
+// so that loads never overlap the work on what has landed.  The kernel then counts its reads
+// itself: wait_lgkmcnt<N> returns when at most N of them are outstanding (they return in
+// order), and use_frags ties registers to that point, so that what uses them stays behind it.
+template <int N>
+__device__ inline void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int N>
+__device__ inline void wait_lgkmcnt() {
+  asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+}
+
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+
+// 16 bytes a lane from LDS byte address `lds_address` + OFFSET.
+template <int OFFSET>
+__device__ inline void lds_read16(u32x4& dst, unsigned lds_address) {
+  static_assert(OFFSET >= 0 && OFFSET < 65536, "the offset field of an LDS read");
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(lds_address), "n"(OFFSET));
+}
+
+// COUNT such reads, STEP bytes apart.
+template <int COUNT, int STEP, int I = 0>
+__device__ inline void read_frags(u32x4 (&dst)[COUNT], unsigned lds_address) {
+  if constexpr (I < COUNT) {
+    lds_read16<I * STEP>(dst[I], lds_address);
+    read_frags<COUNT, STEP, I + 1>(dst, lds_address);
+  }
+}
+
+template <int COUNT>
+__device__ inline void use_frags(u32x4 (&regs)[COUNT]) {
+#pragma unroll
+  for (int i = 0; i < COUNT; ++i) asm volatile("" : "+v"(regs[i]));
+}
+
 // ---------------------------------------------------------------------------- errors
 // Every entry point returns 0, or a negative code after recording a message that
 // axk_last_error() returns.  Shapes are checked on the host before anything is launched.

@@ -39,36 +39,6 @@ __device__ inline bf16x8 as_frag(uint4 v) {
 typedef const __attribute__((address_space(1))) void* global_ptr_t;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-template <int N>
-__device__ inline void wait_vmcnt() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-template <int N>
-__device__ inline void wait_lgkmcnt() {
-  asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
-}
-
-// COUNT reads of 16 bytes a lane from LDS, STEP bytes apart, written as instructions (see
-// gemm_tile_kernel).  Their results may be used only after wait_lgkmcnt and use_frags.
-typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
-
-template <int COUNT, int STEP>
-__device__ inline void read_frags(u32x4 (&dst)[COUNT], unsigned lds_address) {
-  static_assert((COUNT - 1) * STEP < 65536, "the offset field of an LDS read");
-#pragma unroll
-  for (int i = 0; i < COUNT; ++i)
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst[i]) : "v"(lds_address), "n"(i * STEP));
-}
-
-// Ties the registers to this point of the program: what uses them afterwards stays behind
-// the wait that precedes this.
-template <int COUNT>
-__device__ inline void use_frags(u32x4 (&regs)[COUNT]) {
-#pragma unroll
-  for (int i = 0; i < COUNT; ++i) asm volatile("" : "+v"(regs[i]));
-}
-
 __device__ inline bf16x8 as_frag(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
 // ---------------------------------------------------------------------------- gemm_tile
