@@ -72,9 +72,12 @@ int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const
 // out = epilogue(X [M, K] . W [N, K]^T + bias).  mode 0: store elem [M, N]; 1: add into
 // float32 [M, N] (the residual stream); 2: store float32 [M, N] (logits); 3: W holds 2 N rows,
 // gate rows then up rows, and out elem [M, N] = silu(X . gate^T) * (X . up^T) (no bias).
-// x_stride / out_stride: elements between rows.
+// x_stride / out_stride: elements between rows.  workspace: axk_gemm_workspace(m, n, k, mode) bytes
+// (0 for most shapes: then it may be null), 16-byte aligned; products of 17 to 64 rows split K
+// between blocks and add the blocks' sums through it.
+long axk_gemm_workspace(int m, int n, int k, int mode);
 int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
-             int out_stride, int m, int n, int k, int mode, void* stream);
+             int out_stride, int m, int n, int k, int mode, void* workspace, long workspace_bytes, void* stream);
 
 // The same product with an RMS norm folded into it on either side, so that the norm needs no
 // pass of its own (bfloat16 build, shapes for which axk_gemm_norm_fold_ok says 1):

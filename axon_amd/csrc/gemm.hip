@@ -145,7 +145,8 @@ static int launch_fma(const elem_t* x, int x_stride, const elem_t* w, const void
 #if AXON_BF16
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                      int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold,
-                     bool* handled);
+                     void* workspace, size_t workspace_bytes, bool* handled);
+size_t gemm_workspace_bytes(int m, int n, int k, int mode);
 int gemm_norm_fold_ok(int m, int n, int k, int mode);
 int gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim);
 int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out,
@@ -156,7 +157,8 @@ int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const v
 #endif
 
 static int gemm_checked(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
-                        int out_stride, int m, int n, int k, int mode, const GemmNormFold* fold, void* stream) {
+                        int out_stride, int m, int n, int k, int mode, const GemmNormFold* fold, void* workspace,
+                        long workspace_bytes, void* stream) {
   AXK_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
   AXK_REQUIRE(x_stride >= k && out_stride >= n, "gemm: strides x=%d (K=%d) out=%d (N=%d) too small", x_stride, k,
               out_stride, n);
@@ -167,7 +169,8 @@ static int gemm_checked(const void* x, int x_stride, const void* w, const void* 
 #if AXON_BF16
   bool handled = false;
   int rc = launch_gemm_mfma((const bf16_t*)x, x_stride, (const bf16_t*)w, bias, bias_is_f32, out, out_stride, m, n, k,
-                            mode, (hipStream_t)stream, fold, &handled);
+                            mode, (hipStream_t)stream, fold, workspace, workspace_bytes > 0 ? (size_t)workspace_bytes : 0,
+                            &handled);
   if (rc != 0 || handled) return rc;
 #endif
   AXK_REQUIRE(fold == nullptr, "gemm: no kernel folds a norm into M=%d N=%d K=%d of these strides and alignments", m, n,
@@ -176,9 +179,19 @@ static int gemm_checked(const void* x, int x_stride, const void* w, const void* 
                     (hipStream_t)stream);
 }
 
+extern "C" long axk_gemm_workspace(int m, int n, int k, int mode) {
+#if AXON_BF16
+  return m > 0 && n > 0 && k > 0 ? (long)gemm_workspace_bytes(m, n, k, mode) : 0;
+#else
+  return 0;
+#endif
+}
+
 extern "C" int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
-                        int out_stride, int m, int n, int k, int mode, void* stream) {
-  return gemm_checked(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, nullptr, stream);
+                        int out_stride, int m, int n, int k, int mode, void* workspace, long workspace_bytes,
+                        void* stream) {
+  return gemm_checked(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, nullptr, workspace,
+                      workspace_bytes, stream);
 }
 
 extern "C" int axk_gemm_norm_fold_ok(int m, int n, int k, int mode) {
@@ -199,7 +212,7 @@ extern "C" int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, co
               "gemm: the following norm needs the add-into-residual epilogue and both of its outputs");
   AXK_REQUIRE(((uintptr_t)in_squares & 15) == 0, "gemm: the rows' sums of squares must be 16-byte aligned");
   const GemmNormFold fold = {in_squares, in_eps, norm_gain, norm_gain_is_f32, norm_values, norm_squares};
-  return gemm_checked(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, &fold, stream);
+  return gemm_checked(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, &fold, nullptr, 0, stream);
 }
 
 extern "C" int axk_gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim) {

@@ -62,7 +62,7 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK, int STAGES
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const void* __restrict__ bias,
                  int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode, int m_blocks,
-                 int n_blocks) {
+                 int n_blocks, float* __restrict__ partial) {
   extern __shared__ __align__(16) unsigned char smem[];
   static_assert(BK == 32 || BK == 64, "K steps of 32 or 64");
   constexpr int NW = WAVES_M * WAVES_N;
@@ -117,9 +117,13 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
     woff[q] = (unsigned)grow * (unsigned)K + (lslot ^ SWZ(r)) * 8;
   }
 
-  auto issue = [&](int kt) {
+  // Split K (gridDim.y > 1): this block multiplies the K tiles kt_begin .. kt_begin + nk - 1 and
+  // leaves its sums in `partial`; gemm_split_reduce_kernel adds the blocks' sums in block order.
+  const int kt_begin = (int)((long)blockIdx.y * (K / BK) / gridDim.y);
+  const int nk = (int)((long)(blockIdx.y + 1) * (K / BK) / gridDim.y) - kt_begin;
+  auto issue = [&](int kt) {     // kt counts from kt_begin
     unsigned char* stage = smem + (kt % STAGES) * STAGE;
-    const int koff = kt * BK;
+    const int koff = (kt_begin + kt) * BK;
 #pragma unroll
     for (int q = 0; q < XQ; ++q)
       __builtin_amdgcn_global_load_lds((global_ptr_t)(x + xoff[q] + koff), (lds_ptr_t)(stage + (q * NW + wave) * 1024), 16,
@@ -165,7 +169,6 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   // soon as every wave has read that tile's last fragments, which is during its last k step:
   // the wait for the next tile, the barrier and the first reads of the next tile are hidden
   // behind that step's products (half of them before the barrier, half after the reads).
-  const int nk = K / BK;
   constexpr int KS = BK / 16;
   static_assert(KS % 2 == 0, "the register sets alternate and start a tile at set 0");
 #pragma unroll
@@ -206,6 +209,25 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
 #undef SWZ
 
   // epilogue: lane holds column n = lane % 32 of each tile and rows (e/4)*8 + (lane/32)*4 + e%4
+  if (partial) {
+    // [split][gate | up][M][N] (one part without GLU), 32-bit sums as they are
+    constexpr int PARTS = GLU ? 2 : 1;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int part = GLU ? j / (TN / 2) : 0;
+      const int n = GLU ? n0 + wn * (WN / 2) + (j % (TN / 2)) * 32 + (lane & 31) : n0 + wn * WN + j * 32 + (lane & 31);
+      if (n >= N) continue;
+      float* dst = partial + ((size_t)blockIdx.y * PARTS + part) * M * N + n;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m0 + wm * WM + i * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+          if (m < M) dst[(size_t)m * N] = acc[i][j][e];
+        }
+    }
+    return;
+  }
   if (GLU) {
 #pragma unroll
     for (int j = 0; j < TN / 2; ++j) {
@@ -245,9 +267,48 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   }
 }
 
+// The sums of the split-K blocks, added in block order, then the epilogue of the product.
+// One thread per 4 consecutive columns of a row (N is a multiple of 4 on this path).
+__global__ void __launch_bounds__(256)
+gemm_split_reduce_kernel(const float* __restrict__ partial, int splits, int M, int N, const void* __restrict__ bias,
+                         int bias_is_f32, void* __restrict__ out, int out_stride, int mode) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  const int n4 = N / 4;
+  if (idx >= M * n4) return;
+  const int m = idx / n4, n = (idx % n4) * 4;
+  const size_t plane = (size_t)M * N, at_in = (size_t)m * N + n;
+  const int parts = mode == MODE_SWIGLU ? 2 : 1;
+  float4 g = *reinterpret_cast<const float4*>(partial + at_in), u = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  if (parts == 2) u = *reinterpret_cast<const float4*>(partial + plane + at_in);
+  for (int z = 1; z < splits; ++z) {
+    const float4 a = *reinterpret_cast<const float4*>(partial + (size_t)z * parts * plane + at_in);
+    g.x += a.x; g.y += a.y; g.z += a.z; g.w += a.w;
+    if (parts == 2) {
+      const float4 b = *reinterpret_cast<const float4*>(partial + ((size_t)z * parts + 1) * plane + at_in);
+      u.x += b.x; u.y += b.y; u.z += b.z; u.w += b.w;
+    }
+  }
+  float v[4] = {g.x, g.y, g.z, g.w};
+  const size_t at = (size_t)m * out_stride + n;
+  if (mode == MODE_SWIGLU) {
+    const float uu[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) reinterpret_cast<bf16_t*>(out)[at + e] = float_to_bf16(swiglu1(v[e], uu[e]));
+    return;
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (bias) v[e] += load_vec(bias, bias_is_f32, n + e);
+    if (mode == MODE_STORE) reinterpret_cast<bf16_t*>(out)[at + e] = float_to_bf16(v[e]);
+    else if (mode == MODE_ADD_F32) reinterpret_cast<float*>(out)[at + e] += v[e];
+    else reinterpret_cast<float*>(out)[at + e] = v[e];
+  }
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK = 64, int STAGES = 2>
 static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                       int out_stride, int m, int n, int k, int mode, hipStream_t stream) {
+                       int out_stride, int m, int n, int k, int mode, hipStream_t stream, int splits = 1,
+                       float* partial = nullptr) {
   static bool configured = false;
   constexpr int lds_bytes = STAGES * (BM + BN) * BK * 2;
   static_assert(lds_bytes <= 160 * 1024, "the stages do not fit the LDS of a CU");
@@ -262,9 +323,14 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
     configured = true;
   }
   const int m_blocks = ceil_div(m, BM), n_blocks = ceil_div(n, GLU ? BN / 2 : BN);
-  kernel<<<m_blocks * n_blocks, WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(x, x_stride, w, bias, bias_is_f32, out, out_stride,
-                                                                           m, n, k, mode, m_blocks, n_blocks);
+  kernel<<<dim3(m_blocks * n_blocks, splits), WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks, splits > 1 ? partial : nullptr);
   AXK_LAUNCH_CHECK("gemm_tile");
+  if (splits > 1) {
+    gemm_split_reduce_kernel<<<ceil_div(m * (n / 4), 256), 256, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, out,
+                                                                            out_stride, mode);
+    AXK_LAUNCH_CHECK("gemm_split_reduce");
+  }
   return 0;
 }
 
@@ -592,19 +658,33 @@ static int launch_skinny(const bf16_t* x, int x_stride, const bf16_t* w, const v
 
 // Shapes the MFMA kernels take: K a multiple of 64 and 16-byte aligned rows.  Decided by (N, K)
 // and the pointers' alignment, never by M, so a weight matrix always meets the same kernels.
-static bool skinny_takes(int m, int n, int k, int mode) {
-  // a very wide output (the head) with more than 32 rows goes to the tiled kernel, which shares
-  // X through LDS
-  return m <= 64 && !(m > 32 && n >= 65536 && mode != MODE_SWIGLU && (size_t)n * k < (1ull << 32));
+static bool skinny_takes(int m, int n, int k, int mode) { return m <= 16; }
+
+// 17 to 64 rows: one tile of rows (gemm_tile with a 64-row block), K split between blocks so
+// that the chip is full although the output is small; the blocks' sums go through a workspace
+// and are added in block order.  The number of splits depends on (N, K) alone: a row's bits do
+// not depend on how many rows ride along.
+static int mid_splits(int n, int k, int mode) {
+  if (n % 4 != 0) return 1;
+  const int per_block = mode == MODE_SWIGLU ? 128 : (n >= 8192 ? 256 : 128);
+  const int n_blocks = ceil_div(n, per_block), nk = k / 64;
+  int s = 512 / n_blocks;                      // two blocks a CU
+  if (s > nk / 4) s = nk / 4;                  // at least four K tiles a block
+  if (s > 32) s = 32;
+  return s < 1 ? 1 : s;
 }
 
-// A norm is folded into steps of up to 16 rows: with more, adding up the rows' parts costs a
-// block more than the norm's own pass saves.
-int gemm_norm_fold_ok(int m, int n, int k, int mode) { return k % 64 == 0 && m <= 16 && skinny_takes(m, n, k, mode); }
+size_t gemm_workspace_bytes(int m, int n, int k, int mode) {
+  if (m <= 16 || m > 64 || k % 64 != 0) return 0;
+  const int s = mid_splits(n, k, mode);
+  return s > 1 ? (size_t)s * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float) : 0;
+}
+
+int gemm_norm_fold_ok(int m, int n, int k, int mode) { return k % 64 == 0 && skinny_takes(m, n, k, mode); }
 
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                      int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold_in,
-                     bool* handled) {
+                     void* workspace, size_t workspace_bytes, bool* handled) {
   *handled = false;
   if (k % 64 != 0 || x_stride % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return 0;
   *handled = true;
@@ -618,28 +698,33 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
     fold.norm_squares = fold_in->norm_squares;
   }
 #define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream
-  if (m <= 64 && mode == MODE_SWIGLU) {
-    if (m <= 16) return launch_skinny<2, 1, 4, 8, EPI_GLU>(ARGS, fold);
-    if (m <= 32) return launch_skinny<2, 2, 4, 4, EPI_GLU>(ARGS, fold);
-    return launch_skinny<2, 4, 4, 2, EPI_GLU>(ARGS, fold);
-  }
   if (skinny_takes(m, n, k, mode)) {
+    if (mode == MODE_SWIGLU) return launch_skinny<2, 1, 4, 8, EPI_GLU>(ARGS, fold);
     // 32 rows of W per block where that still leaves 128 blocks or more, else 16; four waves
     // split K; the ring is as deep as the registers allow
-    const bool wide = n >= 32 * 128;
-    if (m <= 16) return wide ? launch_skinny<2, 1, 4, 8>(ARGS, fold) : launch_skinny<1, 1, 4, 8>(ARGS, fold);
-    if (m <= 32) return wide ? launch_skinny<2, 2, 4, 4>(ARGS, fold) : launch_skinny<1, 2, 4, 8>(ARGS, fold);
-    return wide ? launch_skinny<2, 4, 4, 2>(ARGS, fold) : launch_skinny<1, 4, 4, 4>(ARGS, fold);
+    return n >= 32 * 128 ? launch_skinny<2, 1, 4, 8>(ARGS, fold) : launch_skinny<1, 1, 4, 8>(ARGS, fold);
   }
   if (fold_in) {
     axk_set_error("gemm: M=%d N=%d goes to the tiled kernel, which folds no norm", m, n);
     return -1;
   }
-  if (m <= 64) return launch_tile<128, 128, 2, 2, false>(ARGS);
   // offsets inside the kernels are 32-bit element counts
   if ((size_t)n * k * (mode == MODE_SWIGLU ? 2 : 1) >= (1ull << 32) || (size_t)m * x_stride >= (1ull << 32)) {
     *handled = false;
     return 0;
+  }
+  if (m <= 64) {
+    const int splits = mid_splits(n, k, mode);
+    const size_t need = gemm_workspace_bytes(m, n, k, mode);
+    if (need > workspace_bytes || (need > 0 && (workspace == nullptr || ((uintptr_t)workspace & 15)))) {
+      axk_set_error("gemm: M=%d N=%d K=%d needs a workspace of %zu bytes, 16-byte aligned (got %zu)", m, n, k, need,
+                    workspace_bytes);
+      return -1;
+    }
+    float* ws = (float*)workspace;
+    if (mode == MODE_SWIGLU) return launch_tile<64, 256, 1, 4, true, 64, 2>(ARGS, splits, ws);
+    if (n >= 8192) return launch_tile<64, 256, 1, 4, false, 64, 2>(ARGS, splits, ws);
+    return launch_tile<64, 128, 1, 4, false, 64, 3>(ARGS, splits, ws);
   }
   // 256 x 256 tiles (8 waves) where they fill the chip: one round of at least 140 blocks (on 256
   // CUs), or several rounds of which the last is not mostly idle; else 128 x 128 tiles, four times
@@ -657,10 +742,11 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
 #undef ARGS
 }
 
-// The [q; k; v] product with rotary encoding and cache store (see RopeStore): up to 64 rows,
-// every head rotated over its whole width, halves of a head a multiple of 16 wide.
+// The [q; k; v] product with rotary encoding and cache store (see RopeStore): up to 16 rows
+// (what gemm_skinny takes), every head rotated over its whole width, halves of a head a
+// multiple of 16 wide.
 int gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim) {
-  return m >= 1 && m <= 64 && k % 64 == 0 && rotary_dim == head_dim && head_dim % 32 == 0;
+  return m >= 1 && m <= 16 && k % 64 == 0 && rotary_dim == head_dim && head_dim % 32 == 0;
 }
 
 int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out,
@@ -672,9 +758,7 @@ int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const v
   const RopeStore rope = {table, positions, seq_rows, block_table, table_stride, k_cache, v_cache,
                           n_heads, n_kv_heads, head_dim, page_size};
 #define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream, fold, rope
-  if (m <= 16) return launch_skinny<2, 1, 4, 8, EPI_ROPE>(ARGS);
-  if (m <= 32) return launch_skinny<2, 2, 4, 4, EPI_ROPE>(ARGS);
-  return launch_skinny<2, 4, 4, 2, EPI_ROPE>(ARGS);
+  return launch_skinny<2, 1, 4, 8, EPI_ROPE>(ARGS);
 #undef ARGS
 }
 

@@ -47,7 +47,8 @@ _SIGNATURES = {
     "axk_attention_decode": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                              c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "axk_attention_fast_ok": [c_int, c_int, c_int, c_int],
-    "axk_gemm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "axk_gemm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
+                 ctypes.c_long, c_void_p],
     "axk_gemm_norm_fold_ok": [c_int, c_int, c_int, c_int],
     "axk_gemm_norm_fold": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                            c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
@@ -75,6 +76,8 @@ class Kernels:
             fn.restype = c_int
         self.lib.axk_attention_decode_workspace.argtypes = [c_int, c_int, c_int, c_int]
         self.lib.axk_attention_decode_workspace.restype = ctypes.c_long
+        self.lib.axk_gemm_workspace.argtypes = [c_int, c_int, c_int, c_int]
+        self.lib.axk_gemm_workspace.restype = ctypes.c_long
         self.lib.axk_argmax_workspace.argtypes = [c_int, c_int]
         self.lib.axk_argmax_workspace.restype = ctypes.c_long
         if bool(self.lib.axk_is_bf16()) != (dtype_name == "bfloat16"):
@@ -292,8 +295,10 @@ class Kernels:
         if bias is not None and bias.numel() != N:
             raise KernelError(f"gemm: bias of {bias.numel()} for {N} columns")
         if row_squares is None and following_norm is None:
+            need = self.lib.axk_gemm_workspace(M, N, K, mode)
+            work = torch.empty(need // 4, dtype=torch.float32, device=x.device) if need > 0 else None
             self._check(self.lib.axk_gemm(_ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"),
-                                          _ptr(out), out.stride(0), M, N, K, mode, _stream()))
+                                          _ptr(out), out.stride(0), M, N, K, mode, _ptr(work), need, _stream()))
             return out
         if row_squares is not None and (row_squares.dtype != torch.float32 or not row_squares.is_contiguous()
                                         or row_squares.shape != (M, K // 16) or not row_squares.is_cuda):
