@@ -668,8 +668,9 @@ static int mid_splits(int n, int k, int mode) {
   if (n % 4 != 0) return 1;
   const int per_block = mode == MODE_SWIGLU ? 128 : (n >= 8192 ? 256 : 128);
   const int n_blocks = ceil_div(n, per_block), nk = k / 64;
-  int s = 512 / n_blocks;                      // two blocks a CU
-  if (s > nk / 4) s = nk / 4;                  // at least four K tiles a block
+  // a block a CU for the narrow tile, two for the wide one (measured); at least four K tiles a block
+  int s = (per_block == 128 && mode != MODE_SWIGLU ? 256 : 512) / n_blocks;
+  if (s > nk / 4) s = nk / 4;
   if (s > 32) s = 32;
   return s < 1 ? 1 : s;
 }
