@@ -675,9 +675,20 @@ static int mid_splits(int n, int k, int mode) {
   return s < 1 ? 1 : s;
 }
 
+// 65 to 256 rows: one or two rows of 128 x 128 tiles, which leave most CUs idle when N is small;
+// K is split so that about a block a CU runs.  Again by (N, K) alone.
+static int small_splits(int n, int k, int mode) {
+  if (n % 4 != 0) return 1;
+  const int n_blocks = ceil_div(n, mode == MODE_SWIGLU ? 64 : 128), nk = k / 64;
+  int s = 256 / (2 * n_blocks);
+  if (s > nk / 4) s = nk / 4;
+  if (s > 16) s = 16;
+  return s < 1 ? 1 : s;
+}
+
 size_t gemm_workspace_bytes(int m, int n, int k, int mode) {
-  if (m <= 16 || m > 64 || k % 64 != 0) return 0;
-  const int s = mid_splits(n, k, mode);
+  if (m <= 16 || m > 256 || k % 64 != 0) return 0;
+  const int s = m <= 64 ? mid_splits(n, k, mode) : small_splits(n, k, mode);
   return s > 1 ? (size_t)s * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float) : 0;
 }
 
@@ -714,8 +725,8 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
     *handled = false;
     return 0;
   }
-  if (m <= 64) {
-    const int splits = mid_splits(n, k, mode);
+  if (m <= 256) {
+    const int splits = m <= 64 ? mid_splits(n, k, mode) : small_splits(n, k, mode);
     const size_t need = gemm_workspace_bytes(m, n, k, mode);
     if (need > workspace_bytes || (need > 0 && (workspace == nullptr || ((uintptr_t)workspace & 15)))) {
       axk_set_error("gemm: M=%d N=%d K=%d needs a workspace of %zu bytes, 16-byte aligned (got %zu)", m, n, k, need,
@@ -723,6 +734,10 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
       return -1;
     }
     float* ws = (float*)workspace;
+    if (m > 64) {
+      if (mode == MODE_SWIGLU) return launch_tile<128, 128, 2, 2, true>(ARGS, splits, ws);
+      return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws);
+    }
     if (mode == MODE_SWIGLU) return launch_tile<64, 256, 1, 4, true, 64, 2>(ARGS, splits, ws);
     if (n >= 8192) return launch_tile<64, 256, 1, 4, false, 64, 2>(ARGS, splits, ws);
     return launch_tile<64, 128, 1, 4, false, 64, 3>(ARGS, splits, ws);

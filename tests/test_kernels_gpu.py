@@ -158,7 +158,7 @@ def test_attention_finds_a_far_key_and_respects_the_windows_edge(dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (3, 100, 70), (17, 259, 130), (70, 96, 33), (130, 48, 257),
                                    (5, 1000, 512), (64, 256, 256), (200, 384, 1024), (33, 152, 3584), (64, 1000, 2048),
-                                   (20, 8200, 512), (48, 130, 1024)])
+                                   (20, 8200, 512), (48, 130, 1024), (100, 132, 2048), (256, 260, 1024)])
 def test_gemm_every_epilogue(dtype, M, N, K):
     k = kernels(dtype)
     x, xr = as_dtype(rnd(M, K, seed=10), dtype)
@@ -184,7 +184,7 @@ def test_gemm_every_epilogue(dtype, M, N, K):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,F,K", [(1, 96, 64), (9, 176, 64), (40, 320, 192), (64, 130, 128), (70, 300, 128),
                                    (300, 512, 256), (600, 1000, 128), (5, 100, 70), (33, 19, 33), (2100, 384, 64),
-                                   (40, 320, 1024), (17, 132, 2048), (64, 96, 4096)])
+                                   (40, 320, 1024), (17, 132, 2048), (64, 96, 4096), (130, 96, 2048)])
 def test_gemm_with_the_gated_epilogue(dtype, M, F, K):
     """One product over [gate; up] whose epilogue is silu(gate) * up."""
     k = kernels(dtype)
@@ -202,23 +202,23 @@ def test_gemm_with_the_gated_epilogue(dtype, M, F, K):
 def test_gemm_rows_do_not_depend_on_the_batch(dtype):
     """The same row of x gives the same bits whatever rows ride along.  float32: for any number
     of rows.  bfloat16: among batches of up to 16 rows (the decoding kernel), among those of 17
-    to 64 (one tile of rows, K split between blocks) and among larger ones (the tiled kernel);
-    between the three a row differs by the rounding of 32-bit sums."""
+    to 64 and of 65 to 256 (tiles with K split between blocks, by (N, K) alone) and among larger
+    ones (the tiled kernel); between the classes a row differs by the rounding of 32-bit sums."""
     k = kernels(dtype)
     for N, K in [(96, 80), (256, 512), (130, 1000), (512, 1024), (300, 4096)]:
         x, _ = as_dtype(rnd(400, K, seed=14), dtype)
         w, _ = as_dtype(rnd(N, K, seed=15, scale=0.2), dtype)
         whole = {}
-        for rows in (16, 64, 400):
+        for rows in (16, 64, 256, 400):
             whole[rows] = torch.empty(rows, N, dtype=torch.float32, device="cuda")
             k.gemm(x[:rows], w, whole[rows], None, MODE_STORE_F32)
-        for m in (1, 3, 16, 17, 33, 64, 65, 130, 257, 300):
+        for m in (1, 3, 16, 17, 33, 64, 65, 130, 256, 257, 300):
             part = torch.empty(m, N, dtype=torch.float32, device="cuda")
             k.gemm(x[:m], w, part, None, MODE_STORE_F32)
-            same_as = whole[400] if dtype == "float32" else whole[16 if m <= 16 else 64 if m <= 64 else 400]
+            same_as = whole[400] if dtype == "float32" else whole[16 if m <= 16 else 64 if m <= 64 else 256 if m <= 256 else 400]
             assert torch.equal(part, same_as[:m]), (N, K, m)
-        assert (whole[16] - whole[400][:16]).abs().max() <= 1e-5 * whole[400].abs().max()
-        assert (whole[64] - whole[400][:64]).abs().max() <= 1e-5 * whole[400].abs().max()
+        for rows in (16, 64, 256):
+            assert (whole[rows] - whole[400][:rows]).abs().max() <= 1e-5 * whole[400].abs().max()
 
 
 @pytest.mark.parametrize("M,H,F", [(1, 64, 128), (8, 192, 320), (16, 448, 64), (5, 4608, 64), (13, 128, 192)])
