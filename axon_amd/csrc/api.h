@@ -73,7 +73,7 @@ int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const
 // float32 [M, N] (the residual stream); 2: store float32 [M, N] (logits); 3: W holds 2 N rows,
 // gate rows then up rows, and out elem [M, N] = silu(X . gate^T) * (X . up^T) (no bias).
 // x_stride / out_stride: elements between rows.  workspace: axk_gemm_workspace(m, n, k, mode) bytes
-// (0 for most shapes: then it may be null), 16-byte aligned; products of 17 to 256 rows split K
+// (0 for most shapes: then it may be null), 16-byte aligned; products of 17 to 2048 rows may split K
 // between blocks and add the blocks' sums through it.
 long axk_gemm_workspace(int m, int n, int k, int mode);
 int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,

@@ -686,9 +686,22 @@ static int small_splits(int n, int k, int mode) {
   return s < 1 ? 1 : s;
 }
 
+// 257 to 2048 rows: a narrow output over a long K (the feed-forward's down projection) gives too
+// few tiles for 256 CUs; K is halved.  By (N, K) alone.
+static int long_k_splits(int n, int k, int mode) {
+  if (n % 4 != 0) return 1;
+  const int n_blocks = ceil_div(n, mode == MODE_SWIGLU ? 128 : 256), nk = k / 64;
+  return nk >= 128 && n_blocks <= 18 ? 2 : 1;
+}
+
+static int splits_of(int m, int n, int k, int mode) {
+  if (m <= 16 || m > 2048) return 1;
+  return m <= 64 ? mid_splits(n, k, mode) : m <= 256 ? small_splits(n, k, mode) : long_k_splits(n, k, mode);
+}
+
 size_t gemm_workspace_bytes(int m, int n, int k, int mode) {
-  if (m <= 16 || m > 256 || k % 64 != 0) return 0;
-  const int s = m <= 64 ? mid_splits(n, k, mode) : small_splits(n, k, mode);
+  if (k % 64 != 0) return 0;
+  const int s = splits_of(m, n, k, mode);
   return s > 1 ? (size_t)s * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float) : 0;
 }
 
@@ -725,15 +738,15 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
     *handled = false;
     return 0;
   }
+  const int splits = splits_of(m, n, k, mode);
+  const size_t need = gemm_workspace_bytes(m, n, k, mode);
+  if (need > workspace_bytes || (need > 0 && (workspace == nullptr || ((uintptr_t)workspace & 15)))) {
+    axk_set_error("gemm: M=%d N=%d K=%d needs a workspace of %zu bytes, 16-byte aligned (got %zu)", m, n, k, need,
+                  workspace_bytes);
+    return -1;
+  }
+  float* ws = (float*)workspace;
   if (m <= 256) {
-    const int splits = m <= 64 ? mid_splits(n, k, mode) : small_splits(n, k, mode);
-    const size_t need = gemm_workspace_bytes(m, n, k, mode);
-    if (need > workspace_bytes || (need > 0 && (workspace == nullptr || ((uintptr_t)workspace & 15)))) {
-      axk_set_error("gemm: M=%d N=%d K=%d needs a workspace of %zu bytes, 16-byte aligned (got %zu)", m, n, k, need,
-                    workspace_bytes);
-      return -1;
-    }
-    float* ws = (float*)workspace;
     if (m > 64) {
       if (mode == MODE_SWIGLU) return launch_tile<128, 128, 2, 2, true>(ARGS, splits, ws);
       return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws);
@@ -746,15 +759,15 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
   // CUs), or several rounds of which the last is not mostly idle; else 128 x 128 tiles, four times
   // as many blocks at twice the traffic from L2 per product.  Thresholds are measured ones.
   const int n_per_block = mode == MODE_SWIGLU ? 128 : 256;
-  const long big = (long)ceil_div(m, 256) * ceil_div(n, n_per_block);
+  const long big = (long)ceil_div(m, 256) * ceil_div(n, n_per_block) * splits;
   const long rounds = (big + 255) / 256;
   const bool use_big = big <= 256 ? big >= 140 : big * 10 >= rounds * 256 * 7;
   if (mode == MODE_SWIGLU) {
-    if (use_big) return launch_tile<256, 256, 4, 2, true>(ARGS);
-    return launch_tile<128, 128, 2, 2, true>(ARGS);
+    if (use_big) return launch_tile<256, 256, 4, 2, true>(ARGS, splits, ws);
+    return launch_tile<128, 128, 2, 2, true>(ARGS, splits, ws);
   }
-  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS);
-  return launch_tile<128, 128, 2, 2, false>(ARGS);
+  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS, splits, ws);
+  return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws);
 #undef ARGS
 }
 

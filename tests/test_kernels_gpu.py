@@ -202,23 +202,23 @@ def test_gemm_with_the_gated_epilogue(dtype, M, F, K):
 def test_gemm_rows_do_not_depend_on_the_batch(dtype):
     """The same row of x gives the same bits whatever rows ride along.  float32: for any number
     of rows.  bfloat16: among batches of up to 16 rows (the decoding kernel), among those of 17
-    to 64 and of 65 to 256 (tiles with K split between blocks, by (N, K) alone) and among larger
-    ones (the tiled kernel); between the classes a row differs by the rounding of 32-bit sums."""
+    to 64, of 65 to 256 and of 257 to 2048 (tiles with K split between blocks, by (N, K) alone)
+    and among larger ones; between the classes a row differs by the rounding of 32-bit sums."""
     k = kernels(dtype)
-    for N, K in [(96, 80), (256, 512), (130, 1000), (512, 1024), (300, 4096)]:
-        x, _ = as_dtype(rnd(400, K, seed=14), dtype)
+    for N, K in [(96, 80), (256, 512), (130, 1000), (512, 1024), (300, 4096), (200, 8192)]:
+        x, _ = as_dtype(rnd(2100, K, seed=14), dtype)
         w, _ = as_dtype(rnd(N, K, seed=15, scale=0.2), dtype)
         whole = {}
-        for rows in (16, 64, 256, 400):
+        for rows in (16, 64, 256, 2048, 2100):
             whole[rows] = torch.empty(rows, N, dtype=torch.float32, device="cuda")
             k.gemm(x[:rows], w, whole[rows], None, MODE_STORE_F32)
-        for m in (1, 3, 16, 17, 33, 64, 65, 130, 256, 257, 300):
+        for m in (1, 3, 16, 17, 33, 64, 65, 130, 256, 257, 300, 1000, 2049):
             part = torch.empty(m, N, dtype=torch.float32, device="cuda")
             k.gemm(x[:m], w, part, None, MODE_STORE_F32)
-            same_as = whole[400] if dtype == "float32" else whole[16 if m <= 16 else 64 if m <= 64 else 256 if m <= 256 else 400]
-            assert torch.equal(part, same_as[:m]), (N, K, m)
-        for rows in (16, 64, 256):
-            assert (whole[rows] - whole[400][:rows]).abs().max() <= 1e-5 * whole[400].abs().max()
+            cls = 2100 if dtype == "float32" else 16 if m <= 16 else 64 if m <= 64 else 256 if m <= 256 else 2048 if m <= 2048 else 2100
+            assert torch.equal(part, whole[cls][:m]), (N, K, m)
+        for rows in (16, 64, 256, 2048):
+            assert (whole[rows] - whole[2100][:rows]).abs().max() <= 1e-5 * whole[2100].abs().max()
 
 
 @pytest.mark.parametrize("M,H,F", [(1, 64, 128), (8, 192, 320), (16, 448, 64), (5, 4608, 64), (13, 128, 192)])
