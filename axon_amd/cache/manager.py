@@ -183,9 +183,12 @@ class CacheManager:
         """Pages for positions [0, n_tokens) in every group, or OutOfPages and nothing taken."""
         if n_tokens > self.max_seq_len:
             raise CacheError(f"{n_tokens} positions exceed the {self.max_seq_len} a request may reach")
+        held = [self.lib.axh_cache_pages_of(self._h, g, slot) for g in range(len(self.groups))]
         rc = self.lib.axh_cache_reserve(self._h, slot, n_tokens)
         if rc == 0:
-            self._dirty.add(slot)
+            # only a row that took a page has to be uploaded again
+            if any(self.lib.axh_cache_pages_of(self._h, g, slot) != held[g] for g in range(len(self.groups))):
+                self._dirty.add(slot)
         elif rc <= -1000000:
             raise CacheError(self._error())
         else:
