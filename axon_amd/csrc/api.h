@@ -19,8 +19,9 @@ int axk_is_bf16(void);
 int axk_elem_size(void);
 
 // x[t, :] = table[tokens[t], :] widened to float32.  A token outside [0, vocab) is an error
-// raised by the caller; the kernel clamps nothing.
-int axk_embed(const int32_t* tokens, const void* table, float* x, int n_tokens, int dim, int vocab,
+// raised by the caller; the kernel clamps nothing.  packed: the table is a packed matrix (see
+// axk_pack_matrix; a tied head's), else row-major.
+int axk_embed(const int32_t* tokens, const void* table, int packed, float* x, int n_tokens, int dim, int vocab,
               void* stream);
 
 // out[r, :] = (x[row(r), :] * inv_rms) * gain, row(r) = rows ? rows[r] : r.
@@ -69,18 +70,27 @@ int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const
                          float* partial, int max_chunks, int n_heads, int n_kv_heads, int head_dim,
                          int page_size, int window, float scale, void* stream);
 
-// out = epilogue(X [M, K] . W [N, K]^T + bias).  mode 0: store elem [M, N]; 1: add into
+// The matrix-core products (bfloat16 build) read W packed: blocks of 16 rows x 32 k of 1 KB in
+// the order in which a wave holds them as an MFMA operand, [row tile][k block], rows padded with
+// zeros to a multiple of 16 (axk_packed_elems elements).  axk_pack_ok: whether a [rows, k] matrix
+// (gated: [gate; up] halves for the SwiGLU epilogue) can be packed; what cannot is multiplied
+// row-major by the 32-bit FMA kernel.
+int axk_pack_ok(int rows, int k, int gated);
+long axk_packed_elems(int rows, int k);
+int axk_pack_matrix(const void* src, void* dst, int rows, int k, void* stream);
+
+// out = epilogue(X [M, K] . W [N, K]^T + bias).  w_packed: W is packed (see above), else row-major.  mode 0: store elem [M, N]; 1: add into
 // float32 [M, N] (the residual stream); 2: store float32 [M, N] (logits); 3: W holds 2 N rows,
 // gate rows then up rows, and out elem [M, N] = silu(X . gate^T) * (X . up^T) (no bias).
 // x_stride / out_stride: elements between rows.  workspace: axk_gemm_workspace(m, n, k, mode) bytes
 // (0 for most shapes: then it may be null), 16-byte aligned; products of 17 to 2048 rows may split K
 // between blocks and add the blocks' sums through it.
 long axk_gemm_workspace(int m, int n, int k, int mode);
-int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
+int axk_gemm(const void* x, int x_stride, const void* w, int w_packed, const void* bias, int bias_is_f32, void* out,
              int out_stride, int m, int n, int k, int mode, void* workspace, long workspace_bytes, void* stream);
 
 // The same product with an RMS norm folded into it on either side, so that the norm needs no
-// pass of its own (bfloat16 build, shapes for which axk_gemm_norm_fold_ok says 1):
+// pass of its own (bfloat16 build, W packed, shapes for which axk_gemm_norm_fold_ok says 1):
 // * in_squares [M, K / 16] (or null): X holds x * gain without the row's scale and in_squares
 //   the sums of x^2 over the 16-column parts of each row; the product's result is multiplied
 //   by 1 / sqrt(sum(in_squares[m]) / K + in_eps) before the bias is added.
@@ -101,7 +111,7 @@ int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, const void* b
                        const void* norm_gain, int norm_gain_is_f32, void* norm_values, float* norm_squares,
                        void* stream);
 
-// The attention's [q; k; v] product (W [(n_heads + 2 n_kv_heads) head_dim, K], or the q rows alone
+// The attention's [q; k; v] product (W packed, [(n_heads + 2 n_kv_heads) head_dim, K], or the q rows alone
 // if write_kv is 0) with what follows it as its epilogue: bias, the rotary encoding of q and k
 // heads over their whole width (table [M, head_dim / 2, 2]: sin, cos), q into qkv [M, >= n_heads
 // head_dim], k and v into the request's pages (as axk_rope_kv_write stores them).  in_squares as in

@@ -24,19 +24,29 @@ extern "C" int axk_elem_size(void) { return (int)sizeof(elem_t); }
 // One block per token; the row is widened exactly (bf16 -> f32) or copied.
 // Reference twin: embed_b (src/cuda/prefill.cu:52-56); no scaling for this architecture
 // (src/model.rs:2657-2675).
-__global__ void embed_kernel(const int32_t* __restrict__ tokens, const elem_t* __restrict__ table,
+// A tied head's matrix is kept packed for the products (see axk_pack_matrix): element (row, i) is
+// then at ((row / 16 * dim / 32 + i / 32) * 64 + row % 16 + 16 (i % 32 / 8)) * 8 + i % 8.
+__global__ void embed_kernel(const int32_t* __restrict__ tokens, const elem_t* __restrict__ table, int packed,
                              float* __restrict__ x, int dim) {
   const int t = blockIdx.x;
-  const elem_t* row = table + (size_t)tokens[t] * dim;
+  const int token = tokens[t];
   float* dst = x + (size_t)t * dim;
+  if (packed) {
+    const elem_t* tile = table + (size_t)(token / 16) * (dim / 32) * 512 + (token % 16) * 8;
+    for (int i = threadIdx.x; i < dim; i += blockDim.x)
+      dst[i] = to_float(tile[(size_t)(i / 32) * 512 + ((i % 32) / 8) * 128 + i % 8]);
+    return;
+  }
+  const elem_t* row = table + (size_t)token * dim;
   for (int i = threadIdx.x; i < dim; i += blockDim.x) dst[i] = to_float(row[i]);
 }
 
-extern "C" int axk_embed(const int32_t* tokens, const void* table, float* x, int n_tokens, int dim,
+extern "C" int axk_embed(const int32_t* tokens, const void* table, int packed, float* x, int n_tokens, int dim,
                          int vocab, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && dim > 0 && vocab > 0, "embed: bad sizes T=%d dim=%d vocab=%d", n_tokens, dim, vocab);
+  AXK_REQUIRE(!packed || dim % 32 == 0, "embed: a packed table has rows of whole blocks of 32, not %d", dim);
   if (n_tokens == 0) return 0;
-  embed_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(tokens, (const elem_t*)table, x, dim);
+  embed_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(tokens, (const elem_t*)table, packed, x, dim);
   AXK_LAUNCH_CHECK("embed");
   return 0;
 }

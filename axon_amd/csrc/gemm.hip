@@ -145,7 +145,9 @@ static int launch_fma(const elem_t* x, int x_stride, const elem_t* w, const void
 #if AXON_BF16
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                      int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold,
-                     void* workspace, size_t workspace_bytes, bool* handled);
+                     void* workspace, size_t workspace_bytes);
+int gemm_pack_ok(int rows, int k, int gated);
+int launch_pack_matrix(const bf16_t* src, bf16_t* dst, int rows, int k, hipStream_t stream);
 size_t gemm_workspace_bytes(int m, int n, int k, int mode);
 int gemm_norm_fold_ok(int m, int n, int k, int mode);
 int gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim);
@@ -156,9 +158,9 @@ int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const v
                          int n_kv_heads, int head_dim, int page_size, hipStream_t stream);
 #endif
 
-static int gemm_checked(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
-                        int out_stride, int m, int n, int k, int mode, const GemmNormFold* fold, void* workspace,
-                        long workspace_bytes, void* stream) {
+static int gemm_checked(const void* x, int x_stride, const void* w, int w_packed, const void* bias, int bias_is_f32,
+                        void* out, int out_stride, int m, int n, int k, int mode, const GemmNormFold* fold,
+                        void* workspace, long workspace_bytes, void* stream) {
   AXK_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
   AXK_REQUIRE(x_stride >= k && out_stride >= n, "gemm: strides x=%d (K=%d) out=%d (N=%d) too small", x_stride, k,
               out_stride, n);
@@ -166,15 +168,16 @@ static int gemm_checked(const void* x, int x_stride, const void* w, const void* 
   AXK_REQUIRE(mode != MODE_SWIGLU || bias == nullptr, "gemm: the gated epilogue takes no bias");
   AXK_REQUIRE(ceil_div(m, 16) <= 65535, "gemm: M=%d is more rows than one launch takes", m);
   if (m == 0) return 0;
+  if (w_packed) {
 #if AXON_BF16
-  bool handled = false;
-  int rc = launch_gemm_mfma((const bf16_t*)x, x_stride, (const bf16_t*)w, bias, bias_is_f32, out, out_stride, m, n, k,
-                            mode, (hipStream_t)stream, fold, workspace, workspace_bytes > 0 ? (size_t)workspace_bytes : 0,
-                            &handled);
-  if (rc != 0 || handled) return rc;
+    return launch_gemm_mfma((const bf16_t*)x, x_stride, (const bf16_t*)w, bias, bias_is_f32, out, out_stride, m, n, k, mode,
+                            (hipStream_t)stream, fold, workspace, workspace_bytes > 0 ? (size_t)workspace_bytes : 0);
+#else
+    axk_set_error("gemm: packed matrices exist only in the bfloat16 build");
+    return -1;
 #endif
-  AXK_REQUIRE(fold == nullptr, "gemm: no kernel folds a norm into M=%d N=%d K=%d of these strides and alignments", m, n,
-              k);
+  }
+  AXK_REQUIRE(fold == nullptr, "gemm: a norm is folded only into products with a packed matrix");
   return launch_fma((const elem_t*)x, x_stride, (const elem_t*)w, bias, bias_is_f32, out, out_stride, m, n, k, mode,
                     (hipStream_t)stream);
 }
@@ -187,11 +190,32 @@ extern "C" long axk_gemm_workspace(int m, int n, int k, int mode) {
 #endif
 }
 
-extern "C" int axk_gemm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
-                        int out_stride, int m, int n, int k, int mode, void* workspace, long workspace_bytes,
+extern "C" int axk_gemm(const void* x, int x_stride, const void* w, int w_packed, const void* bias, int bias_is_f32,
+                        void* out, int out_stride, int m, int n, int k, int mode, void* workspace, long workspace_bytes,
                         void* stream) {
-  return gemm_checked(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, nullptr, workspace,
+  return gemm_checked(x, x_stride, w, w_packed, bias, bias_is_f32, out, out_stride, m, n, k, mode, nullptr, workspace,
                       workspace_bytes, stream);
+}
+
+extern "C" int axk_pack_ok(int rows, int k, int gated) {
+#if AXON_BF16
+  return gemm_pack_ok(rows, k, gated);
+#else
+  return 0;   // the 32-bit build multiplies row-major matrices
+#endif
+}
+
+extern "C" long axk_packed_elems(int rows, int k) { return (long)((rows + 15) / 16 * 16) * k; }
+
+extern "C" int axk_pack_matrix(const void* src, void* dst, int rows, int k, void* stream) {
+#if AXON_BF16
+  AXK_REQUIRE(gemm_pack_ok(rows, k, 0), "pack_matrix: [%d, %d] cannot be packed", rows, k);
+  AXK_REQUIRE(((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0, "pack_matrix: operands must be 16-byte aligned");
+  return launch_pack_matrix((const bf16_t*)src, (bf16_t*)dst, rows, k, (hipStream_t)stream);
+#else
+  axk_set_error("pack_matrix: only in the bfloat16 build");
+  return -1;
+#endif
 }
 
 extern "C" int axk_gemm_norm_fold_ok(int m, int n, int k, int mode) {
@@ -212,7 +236,7 @@ extern "C" int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, co
               "gemm: the following norm needs the add-into-residual epilogue and both of its outputs");
   AXK_REQUIRE(((uintptr_t)in_squares & 15) == 0, "gemm: the rows' sums of squares must be 16-byte aligned");
   const GemmNormFold fold = {in_squares, in_eps, norm_gain, norm_gain_is_f32, norm_values, norm_squares};
-  return gemm_checked(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, &fold, nullptr, 0, stream);
+  return gemm_checked(x, x_stride, w, 1, bias, bias_is_f32, out, out_stride, m, n, k, mode, &fold, nullptr, 0, stream);
 }
 
 extern "C" int axk_gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim) {

@@ -1,5 +1,12 @@
-// bfloat16 matrix products on the matrix cores: out = X [M, K] . W [N, K]^T, both operands
-// K-major, 32-bit accumulation.  Only in the bfloat16 build.
+// bfloat16 matrix products on the matrix cores: out = X [M, K] . W [N, K]^T, 32-bit accumulation.
+// Only in the bfloat16 build.
+//
+// W is PACKED (axk_pack_matrix, once, when the weights are loaded): blocks of 16 rows x 32 k, each
+// 1 KB in the order in which a wave holds them as an MFMA operand (lane l: row l % 16, the 8
+// consecutive k from 8 (l / 16)); blocks ordered [row tile][k block]; rows padded to a multiple
+// of 16 with zeros.  A wave instruction then reads 1 KB of consecutive memory (measured: 10 to 35 %
+// more bandwidth than 16 rows x 64 bytes of a row-major matrix), lands in LDS without a
+// permutation, and the same bytes serve the 16x16x32 and the 32x32x16 MFMA.
 //
 // Two kernels, chosen by M alone so that a given (N, K) always meets the same pair:
 //
@@ -71,9 +78,11 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   constexpr int ROW = BK * 2;                          // bytes of a row
   constexpr int SLOTS = BK / 8;                        // 16-byte slots of a row
   constexpr int RPI = 1024 / ROW;                      // rows one wave instruction fills
-  constexpr int XQ = BM / RPI / NW, WQ = BN / RPI / NW;  // load instructions per wave and stage
+  constexpr int KBT = BK / 32;                         // packed k blocks of a K tile
+  constexpr int XQ = BM / RPI / NW, WQ = BN / 16 * KBT / NW;  // load instructions per wave and stage
   constexpr int STAGE = (BM + BN) * ROW;               // bytes per stage
   static_assert(XQ >= 1 && WQ >= 1 && (STAGES - 2) * (XQ + WQ) < 64, "tile too small or too many loads in flight");
+  static_assert(BN / 16 * KBT % NW == 0 && WN % 32 == 0, "the 1 KB chunks of W are shared out evenly");
 #define SWZ(row) (BK == 64 ? (((row) >> 1) & 7) : (((row) >> 2) & 3))
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -103,18 +112,24 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
     const int r = (q * NW + wave) * RPI + lrow;
     xoff[q] = (unsigned)min(m0 + r, M - 1) * (unsigned)x_stride + (lslot ^ SWZ(r)) * 8;
   }
+  // W: chunk c = q * NW + wave of a stage is the packed block (row tile c / KBT, k block c % KBT)
+  // of the tile, 1 KB as it lies in memory.  Row tiles past the matrix: its last one (the
+  // epilogue drops those columns).
+  const int KB = K / 32;
+  const int row_tiles = GLU ? N / 16 : (N + 15) / 16;          // GLU: per half, N a multiple of 16
 #pragma unroll
   for (int q = 0; q < WQ; ++q) {
-    const int r = (q * NW + wave) * RPI + lrow;  // row of the LDS tile
-    int grow;
+    const int c = q * NW + wave;
+    const int r = (c / KBT) * 16;                               // first row of the chunk in the LDS tile
+    int tile;
     if (GLU) {
-      const int owner = r / WN, within = r % WN;             // the wave whose columns these are
+      const int owner = r / WN, within = r % WN;                // the wave whose columns these are
       const int col = n0 + owner * (WN / 2) + within % (WN / 2);
-      grow = (within >= WN / 2 ? N : 0) + min(col, N - 1);   // up rows follow the N gate rows
+      tile = (within >= WN / 2 ? row_tiles : 0) + min(col / 16, row_tiles - 1);   // up rows follow the N gate rows
     } else {
-      grow = min(n0 + r, N - 1);
+      tile = min((n0 + r) / 16, row_tiles - 1);
     }
-    woff[q] = (unsigned)grow * (unsigned)K + (lslot ^ SWZ(r)) * 8;
+    woff[q] = ((unsigned)tile * (unsigned)KB + (c % KBT)) * 512 + lane * 8;
   }
 
   // Split K (gridDim.y > 1): this block multiplies the K tiles kt_begin .. kt_begin + nk - 1 and
@@ -130,7 +145,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
                                        0, 0);
 #pragma unroll
     for (int q = 0; q < WQ; ++q)
-      __builtin_amdgcn_global_load_lds((global_ptr_t)(w + woff[q] + koff),
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(w + woff[q] + (kt_begin + kt) * (KBT * 512)),
                                        (lds_ptr_t)(stage + BM * ROW + (q * NW + wave) * 1024), 16, 0, 0);
   };
 
@@ -146,16 +161,17 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   const int frow = lane & 31, fhalf = lane >> 5, fsw = SWZ(frow);
   const unsigned lds0 = (unsigned)(size_t)(lds_ptr_t)smem;
   const unsigned xbase = lds0 + (wm * WM + frow) * ROW;
-  const unsigned wbase = lds0 + (BM + wn * WN + frow) * ROW;
+  // W fragment of k step ks: block (row tile of the lane's row, k block ks / 2), lane slot
+  // 16 (2 (ks % 2) + lane / 32) + row % 16 of it: no permutation, 16 lanes read 256 consecutive bytes
+  const unsigned wbase = lds0 + BM * ROW + ((wn * WN + frow) / 16) * KBT * 1024 + (fhalf * 16 + (frow & 15)) * 16;
   // The fragments of k step ks of a stage into one of two register sets.  The reads are written
   // as instructions: the compiler, which cannot tell the stage being read from the stage a
   // direct load is filling, would wait for every load in flight before each of its own reads,
   // and the loads of the next tile would never overlap the products of this one.
   u32x4 a[2][TM], b[2][TN];
   auto read_step = [&](int set, int stage_index, int ks) {
-    const unsigned at = stage_index * STAGE + ((((ks * 2 + fhalf) ^ fsw)) << 4);
-    read_frags<TM, 32 * ROW>(a[set], xbase + at);
-    read_frags<TN, 32 * ROW>(b[set], wbase + at);
+    read_frags<TM, 32 * ROW>(a[set], xbase + stage_index * STAGE + ((((ks * 2 + fhalf) ^ fsw)) << 4));
+    read_frags<TN, 2 * KBT * 1024>(b[set], wbase + stage_index * STAGE + (ks / 2) * 1024 + (ks % 2) * 512);
   };
   auto multiply = [&](int set, int j_from, int j_to) {
 #pragma unroll
@@ -335,9 +351,9 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
 }
 
 // ---------------------------------------------------------------------------- gemm_skinny
-// A block of WAVES waves owns NT16 * 16 rows of W; wave v takes the k steps (of 64) v, v + WAVES,
-// ...  C[n][m] tiles of 16 x 16: the MFMA's A operand is W (lane: row n = lane % 16, 8
-// consecutive k from (lane / 16) * 8), its B operand X (lane: row m = lane % 16, the same k).
+// A block of WAVES waves owns NT16 row tiles (of 16) of W; wave v takes the k steps (of 64) v,
+// v + WAVES, ...  C[n][m] tiles of 16 x 16: the MFMA's A operand is W (a packed block as it lies
+// in memory), its B operand X (lane: row m = lane % 16, 8 consecutive k from (lane / 16) * 8).
 // A lane ends with 4 consecutive n of one m: one vector store.
 // GLU (NT16 = 2): the block's two tiles are the gate rows n0 .. n0 + 15 and the up rows of the
 // same columns (W holds 2 N rows), and the output is silu(gate) * up.
@@ -394,16 +410,18 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
   const int n0 = blockIdx.x * (GLU ? 16 : NT16 * 16);
   const int r16 = lane & 15, kq = (lane >> 4) * 8;
 
-  const bf16_t* wrow[NT16];
+  // the packed blocks of this block's row tiles: [row tile][k block of 32][lane][8]
+  const int KB = K / 32;
+  const bf16_t* wtile[NT16];
 #pragma unroll
   for (int i = 0; i < NT16; ++i) {
-    int row;
-    if (GLU) row = i * N + min(n0 + r16, N - 1);
+    int tile;
+    if (GLU) tile = i * (N / 16) + blockIdx.x;                 // gate rows, then the up rows of the same columns
     else if (ROPE) {
       const int half = rope.head_dim / 2, per_head = half / 16;
-      row = (blockIdx.x / per_head) * rope.head_dim + i * half + (blockIdx.x % per_head) * 16 + r16;
-    } else row = min(n0 + i * 16 + r16, N - 1);
-    wrow[i] = w + (size_t)row * K + kq;
+      tile = ((blockIdx.x / per_head) * rope.head_dim + i * half) / 16 + blockIdx.x % per_head;
+    } else tile = min(n0 / 16 + i, (N + 15) / 16 - 1);         // past the matrix: its last tile (columns dropped below)
+    wtile[i] = w + (size_t)tile * KB * 512 + lane * 8;
   }
   const bf16_t* xrow[MT16];
 #pragma unroll
@@ -425,8 +443,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
     const int k0 = (wave + local * WAVES) * 64;
 #pragma unroll
     for (int i = 0; i < NT16; ++i) {
-      wf[slot][i][0] = *reinterpret_cast<const uint4*>(wrow[i] + k0);
-      wf[slot][i][1] = *reinterpret_cast<const uint4*>(wrow[i] + k0 + 32);
+      wf[slot][i][0] = *reinterpret_cast<const uint4*>(wtile[i] + k0 * 16);          // k block k0 / 32: 512 elements each
+      wf[slot][i][1] = *reinterpret_cast<const uint4*>(wtile[i] + k0 * 16 + 512);
     }
 #pragma unroll
     for (int j = 0; j < MT16; ++j) {
@@ -658,6 +676,37 @@ static int launch_skinny(const bf16_t* x, int x_stride, const bf16_t* w, const v
 
 // Shapes the MFMA kernels take: K a multiple of 64 and 16-byte aligned rows.  Decided by (N, K)
 // and the pointers' alignment, never by M, so a weight matrix always meets the same kernels.
+// What can be packed: K in whole steps of 64, offsets inside the kernels in 32 bits, and for a
+// [gate; up] matrix halves that are whole row tiles.
+int gemm_pack_ok(int rows, int k, int gated) {
+  if (rows <= 0 || k <= 0 || k % 64 != 0) return 0;
+  if ((size_t)((rows + 15) / 16 * 16) * k >= (1ull << 32)) return 0;
+  return !gated || (rows % 32 == 0);
+}
+
+// One thread per 16 bytes of the packed matrix: lane slot (row % 16) + 16 ((k % 32) / 8) of block
+// (row / 16, k / 32).  Rows past the matrix are zeros.
+__global__ void __launch_bounds__(256)
+pack_matrix_kernel(const bf16_t* __restrict__ src, bf16_t* __restrict__ dst, int rows, int K) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;     // 16-byte slot of the packed matrix
+  const int KB = K / 32;
+  const size_t block = idx / 64;
+  const int lane = (int)(idx % 64);
+  const int tile = (int)(block / KB), kb = (int)(block % KB);
+  if (tile >= (rows + 15) / 16) return;
+  const int row = tile * 16 + (lane & 15), k = kb * 32 + (lane >> 4) * 8;
+  uint4 v = uint4{0, 0, 0, 0};
+  if (row < rows) v = *reinterpret_cast<const uint4*>(src + (size_t)row * K + k);
+  *reinterpret_cast<uint4*>(dst + idx * 8) = v;
+}
+
+int launch_pack_matrix(const bf16_t* src, bf16_t* dst, int rows, int k, hipStream_t stream) {
+  const size_t slots = (size_t)((rows + 15) / 16) * (k / 32) * 64;
+  pack_matrix_kernel<<<(unsigned)((slots + 255) / 256), 256, 0, stream>>>(src, dst, rows, k);
+  AXK_LAUNCH_CHECK("pack_matrix");
+  return 0;
+}
+
 static bool skinny_takes(int m, int n, int k, int mode) { return m <= 16; }
 
 // 17 to 64 rows: one tile of rows (gemm_tile with a 64-row block), K split between blocks so
@@ -705,14 +754,22 @@ size_t gemm_workspace_bytes(int m, int n, int k, int mode) {
   return s > 1 ? (size_t)s * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float) : 0;
 }
 
-int gemm_norm_fold_ok(int m, int n, int k, int mode) { return k % 64 == 0 && skinny_takes(m, n, k, mode); }
+int gemm_norm_fold_ok(int m, int n, int k, int mode) {
+  return gemm_pack_ok(mode == MODE_SWIGLU ? 2 * n : n, k, mode == MODE_SWIGLU) && skinny_takes(m, n, k, mode);
+}
 
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                      int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold_in,
-                     void* workspace, size_t workspace_bytes, bool* handled) {
-  *handled = false;
-  if (k % 64 != 0 || x_stride % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15)) return 0;
-  *handled = true;
+                     void* workspace, size_t workspace_bytes) {
+  if (!gemm_pack_ok(mode == MODE_SWIGLU ? 2 * n : n, k, mode == MODE_SWIGLU)) {
+    axk_set_error("gemm: N=%d K=%d is no shape of a packed matrix", n, k);
+    return -1;
+  }
+  if (x_stride % 8 != 0 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15) || (size_t)m * x_stride >= (1ull << 32)) {
+    axk_set_error("gemm: with a packed matrix the rows of X must be 16-byte aligned and X below 2^32 elements "
+                  "(stride %d, M=%d)", x_stride, m);
+    return -1;
+  }
   NormFold fold = {nullptr, 0.0f, nullptr, 0, nullptr, nullptr};
   if (fold_in) {
     fold.in_squares = fold_in->in_squares;
@@ -732,11 +789,6 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
   if (fold_in) {
     axk_set_error("gemm: M=%d N=%d goes to the tiled kernel, which folds no norm", m, n);
     return -1;
-  }
-  // offsets inside the kernels are 32-bit element counts
-  if ((size_t)n * k * (mode == MODE_SWIGLU ? 2 : 1) >= (1ull << 32) || (size_t)m * x_stride >= (1ull << 32)) {
-    *handled = false;
-    return 0;
   }
   const int splits = splits_of(m, n, k, mode);
   const size_t need = gemm_workspace_bytes(m, n, k, mode);

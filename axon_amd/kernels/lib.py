@@ -31,7 +31,7 @@ def _stream() -> c_void_p:
 
 
 _SIGNATURES = {
-    "axk_embed": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "axk_embed": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
     "axk_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p],
     "axk_rope_table": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_rope_kv_write": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
@@ -47,8 +47,10 @@ _SIGNATURES = {
     "axk_attention_decode": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                              c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "axk_attention_fast_ok": [c_int, c_int, c_int, c_int],
-    "axk_gemm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
+    "axk_gemm": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
                  ctypes.c_long, c_void_p],
+    "axk_pack_ok": [c_int, c_int, c_int],
+    "axk_pack_matrix": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_gemm_norm_fold_ok": [c_int, c_int, c_int, c_int],
     "axk_gemm_norm_fold": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                            c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
@@ -59,6 +61,35 @@ _SIGNATURES = {
     "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
     "axk_fill_f32": [c_void_p, c_float, c_int, c_void_p],
 }
+
+
+class PackedMatrix:
+    """A [rows, cols] matrix in the layout the matrix-core products read: blocks of 16 rows x 32
+    columns, each 1 KB in the order in which a wave holds them as an MFMA operand, ordered
+    [row tile][column block]; rows padded with zeros to a multiple of 16.  `data` is the flat
+    storage.  A leading slice of whole row tiles is a view."""
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int):
+        self.data, self.rows, self.cols = data, rows, cols
+
+    @property
+    def shape(self):
+        return (self.rows, self.cols)
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr()
+
+    def __getitem__(self, rows) -> "PackedMatrix":
+        if not isinstance(rows, slice) or rows.start not in (None, 0) or rows.step not in (None, 1):
+            raise KernelError("a packed matrix gives only its leading rows")
+        n = self.rows if rows.stop is None else int(rows.stop)
+        if not 0 < n <= self.rows or (n % 16 and n != self.rows):
+            raise KernelError(f"a packed matrix of {self.rows} rows is cut at multiples of 16, not at {n}")
+        return PackedMatrix(self.data[:-(-n // 16) * 16 * self.cols], n, self.cols)
 
 
 class Kernels:
@@ -76,6 +107,8 @@ class Kernels:
             fn.restype = c_int
         self.lib.axk_attention_decode_workspace.argtypes = [c_int, c_int, c_int, c_int]
         self.lib.axk_attention_decode_workspace.restype = ctypes.c_long
+        self.lib.axk_packed_elems.argtypes = [c_int, c_int]
+        self.lib.axk_packed_elems.restype = ctypes.c_long
         self.lib.axk_gemm_workspace.argtypes = [c_int, c_int, c_int, c_int]
         self.lib.axk_gemm_workspace.restype = ctypes.c_long
         self.lib.axk_argmax_workspace.argtypes = [c_int, c_int]
@@ -123,11 +156,14 @@ class Kernels:
 
     # ------------------------------------------------------------------ ops
     def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-        self._i32(tokens, "embed tokens"); self._elem(table, "embed table"); self._f32(out, "embed out")
+        packed = isinstance(table, PackedMatrix)
+        self._i32(tokens, "embed tokens"); self._elem(table.data if packed else table, "embed table")
+        self._f32(out, "embed out")
         vocab, dim = table.shape
-        if out.shape != (tokens.numel(), dim) or not table.is_contiguous():
+        if out.shape != (tokens.numel(), dim) or not (packed or table.is_contiguous()):
             raise KernelError(f"embed: out {tuple(out.shape)} does not fit {tokens.numel()} tokens of width {dim}")
-        self._check(self.lib.axk_embed(_ptr(tokens), _ptr(table), _ptr(out), tokens.numel(), dim, vocab, _stream()))
+        self._check(self.lib.axk_embed(_ptr(tokens), _ptr(table), 1 if packed else 0, _ptr(out), tokens.numel(), dim,
+                                       vocab, _stream()))
         return out
 
     def rmsnorm(self, x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
@@ -184,11 +220,13 @@ class Kernels:
         the same bits as `gemm` into qkv followed by `rope_kv_write`.  q lands in qkv[:, :n_heads *
         head_dim]; the k and v columns of qkv are not written.  Without write_kv, w holds the q
         rows only.  row_squares, eps: as in `gemm`."""
-        self._elem(x, "qkv x"); self._elem(w, "qkv w"); self._elem(qkv, "qkv out"); self._f32(table, "rope table")
+        if not isinstance(w, PackedMatrix):
+            raise KernelError("gemm_qkv_rope: needs a packed matrix")
+        self._elem(x, "qkv x"); self._elem(w.data, "qkv w"); self._elem(qkv, "qkv out"); self._f32(table, "rope table")
         self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
         M, K = x.shape
         rows = (n_heads + (2 * n_kv_heads if write_kv else 0)) * head_dim
-        if w.shape != (rows, K) or not w.is_contiguous() or x.stride(1) != 1:
+        if w.shape != (rows, K) or x.stride(1) != 1:
             raise KernelError(f"gemm_qkv_rope: x {tuple(x.shape)} w {tuple(w.shape)}, expected w [{rows}, {K}]")
         if qkv.shape[0] != M or qkv.shape[1] < n_heads * head_dim or qkv.stride(1) != 1:
             raise KernelError(f"gemm_qkv_rope: qkv {tuple(qkv.shape)} does not hold [{M}, {n_heads * head_dim}]")
@@ -263,6 +301,27 @@ class Kernels:
             n_heads, n_kv_heads, head_dim, page_size, window, float(scale), _stream()))
         return out
 
+    def pack_ok(self, rows: int, cols: int, gated: bool = False) -> bool:
+        """Whether a [rows, cols] matrix can be packed for the matrix-core products (gated: a
+        [gate; up] matrix for the SwiGLU epilogue).  Never in the float32 build."""
+        return bool(self.lib.axk_pack_ok(rows, cols, 1 if gated else 0))
+
+    def pack_matrix(self, w: torch.Tensor) -> PackedMatrix:
+        self._elem(w, "pack_matrix")
+        if w.dim() != 2 or not w.is_contiguous() or not self.pack_ok(w.shape[0], w.shape[1]):
+            raise KernelError(f"pack_matrix: {tuple(w.shape)} cannot be packed")
+        rows, cols = w.shape
+        out = torch.empty(self.lib.axk_packed_elems(rows, cols), dtype=w.dtype, device=w.device)
+        self._check(self.lib.axk_pack_matrix(_ptr(w), _ptr(out), rows, cols, _stream()))
+        return PackedMatrix(out, rows, cols)
+
+    def prepare_weight(self, w: torch.Tensor, gated: bool = False):
+        """A weight matrix as the products want it: packed where that is possible (then the
+        row-major tensor is no longer needed), else as it is."""
+        if isinstance(w, torch.Tensor) and w.dim() == 2 and self.pack_ok(w.shape[0], w.shape[1], gated):
+            return self.pack_matrix(w.contiguous())
+        return w
+
     def gemm_norm_fold_ok(self, m: int, n: int, k: int, mode: int) -> bool:
         """Whether the product of these sizes can take an RMS norm into itself (see `gemm`)."""
         return bool(self.lib.axk_gemm_norm_fold_ok(m, n, k, mode))
@@ -270,7 +329,8 @@ class Kernels:
     def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
              mode: int = MODE_STORE, row_squares: Optional[torch.Tensor] = None, eps: float = 0.0,
              following_norm=None) -> torch.Tensor:
-        """out = epilogue(x . w^T + bias); x [M, K] (rows may be strided), w [N, K] contiguous.
+        """out = epilogue(x . w^T + bias); x [M, K] (rows may be strided), w [N, K] contiguous or
+        a PackedMatrix (the matrix-core kernels; a row-major w goes to the 32-bit FMA kernel).
         MODE_SWIGLU: w is [2 N, K], gate rows then up rows; out [M, N] = silu(x gate^T) * (x up^T).
 
         An RMS norm folded in (where `gemm_norm_fold_ok`): with `row_squares` float32 [M, K / 16],
@@ -278,14 +338,15 @@ class Kernels:
         which the product applies to its result.  `following_norm` = (gain, values [M, N],
         squares [M, ceil(N / 16)]) with MODE_ADD_F32: the epilogue also writes out * gain and the
         sums of out^2 over parts of 16 columns, for the next product's `row_squares` side."""
-        self._elem(x, "gemm x"); self._elem(w, "gemm w")
+        packed = isinstance(w, PackedMatrix)
+        self._elem(x, "gemm x"); self._elem(w.data if packed else w, "gemm w")
         M, K = x.shape
         N = w.shape[0]
         if mode == MODE_SWIGLU:
             if N % 2 or bias is not None:
                 raise KernelError("gemm: the gated epilogue needs gate and up rows and takes no bias")
             N //= 2
-        if w.shape[1] != K or not w.is_contiguous() or x.stride(1) != 1 or out.stride(1) != 1:
+        if w.shape[1] != K or not (packed or w.is_contiguous()) or x.stride(1) != 1 or out.stride(1) != 1:
             raise KernelError(f"gemm: x {tuple(x.shape)} w {tuple(w.shape)} do not multiply, or are not row-major")
         if out.shape != (M, N) or not out.is_cuda:
             raise KernelError(f"gemm: out {tuple(out.shape)} is not [{M}, {N}]")
@@ -295,11 +356,14 @@ class Kernels:
         if bias is not None and bias.numel() != N:
             raise KernelError(f"gemm: bias of {bias.numel()} for {N} columns")
         if row_squares is None and following_norm is None:
-            need = self.lib.axk_gemm_workspace(M, N, K, mode)
+            need = self.lib.axk_gemm_workspace(M, N, K, mode) if packed else 0
             work = torch.empty(need // 4, dtype=torch.float32, device=x.device) if need > 0 else None
-            self._check(self.lib.axk_gemm(_ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"),
-                                          _ptr(out), out.stride(0), M, N, K, mode, _ptr(work), need, _stream()))
+            self._check(self.lib.axk_gemm(_ptr(x), x.stride(0), _ptr(w), 1 if packed else 0, _ptr(bias),
+                                          self._vec_flag(bias, "gemm bias"), _ptr(out), out.stride(0), M, N, K, mode,
+                                          _ptr(work), need, _stream()))
             return out
+        if not packed:
+            raise KernelError("gemm: a norm is folded only into products with a packed matrix")
         if row_squares is not None and (row_squares.dtype != torch.float32 or not row_squares.is_contiguous()
                                         or row_squares.shape != (M, K // 16) or not row_squares.is_cuda):
             raise KernelError(f"gemm: row_squares {tuple(row_squares.shape)} {row_squares.dtype} is not float32 "

@@ -99,6 +99,12 @@ class DecoderModel:
             b.load(store, rt)
         self.final_norm.load(store, rt)
         self.head.load(store, rt)
+        # a head tied to the embedding may have repacked the matrix for its product: the embedding
+        # then reads that copy, and the row-major one is dropped
+        if (getattr(self.head, "source_name", None) == getattr(self.embedding, "name", None)
+                and not isinstance(self.head.weight, torch.Tensor)):
+            self.embedding.table = self.head.weight
+            store.forget(self.embedding.name)
 
     # ------------------------------------------------------------------ the step
     def forward(self, ctx) -> torch.Tensor:

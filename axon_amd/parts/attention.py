@@ -20,7 +20,7 @@ from typing import List, Optional
 import torch
 
 from ..config.base import ConfigError
-from ..kernels import MODE_ADD_F32, MODE_STORE
+from ..kernels import MODE_ADD_F32, MODE_STORE, PackedMatrix
 from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, UnscaledRows, build_part, register_mixer
 
 
@@ -129,7 +129,7 @@ class GQAttention(Mixer):
         return ("attention_chunks", self.window), 1 << (most - 1).bit_length()
 
     def load(self, store, rt) -> None:
-        self.w_qkv = store.fused_matrix([self.n[k] + ".weight" for k in ("q", "k", "v")])
+        self.w_qkv = rt.k.prepare_weight(store.fused_matrix([self.n[k] + ".weight" for k in ("q", "k", "v")]))
         biases = [store.vector(self.n[k] + ".bias", optional=True) for k in ("q", "k", "v")] if self.qkv_bias else []
         present = [b is not None for b in biases]
         if any(present):
@@ -137,7 +137,8 @@ class GQAttention(Mixer):
                 raise ConfigError(f"{self.prefix}: q, k and v biases must all be present or all absent")
             dt = torch.float32 if any(b.dtype == torch.float32 for b in biases) else biases[0].dtype
             self.b_qkv = torch.cat([b.to(dt) for b in biases]).contiguous()
-        self.w_o = store.matrix(self.n["o"] + ".weight")
+        self.w_o = rt.k.prepare_weight(store.matrix(self.n["o"] + ".weight"))
+        store.forget(self.n["o"] + ".weight")
         self.b_o = store.vector(self.n["o"] + ".bias") if self.out_bias else None
         if self.position is not None:
             self.position.load(store, rt)
@@ -145,11 +146,13 @@ class GQAttention(Mixer):
     # ------------------------------------------------------------------ the step
     def takes_unscaled_rows(self, ctx) -> bool:
         k = ctx.rt.k
-        return (k.gemm_norm_fold_ok(ctx.n_tokens, self.q_dim + 2 * self.kv_dim, self.hidden, MODE_STORE)
+        return (isinstance(self.w_qkv, PackedMatrix)
+                and k.gemm_norm_fold_ok(ctx.n_tokens, self.q_dim + 2 * self.kv_dim, self.hidden, MODE_STORE)
                 and k.gemm_norm_fold_ok(ctx.n_tokens, self.q_dim, self.hidden, MODE_STORE))
 
     def folds_following_norm(self, ctx) -> bool:
-        return ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.hidden, self.q_dim, MODE_ADD_F32)
+        return (isinstance(self.w_o, PackedMatrix)
+                and ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.hidden, self.q_dim, MODE_ADD_F32))
 
     def forward(self, ctx, binding: CacheBinding, h, residual, fold=None) -> None:
         k = ctx.rt.k
@@ -172,7 +175,7 @@ class GQAttention(Mixer):
         else:
             # reading another run's cache: only the queries are needed
             w, bias = self.w_qkv[:self.q_dim], None if self.b_qkv is None else self.b_qkv[:self.q_dim]
-        if k.gemm_qkv_rope_ok(T, self.hidden, self.hd, rotary):
+        if isinstance(w, PackedMatrix) and k.gemm_qkv_rope_ok(T, self.hidden, self.hd, rotary):
             # a short step: product, rotation and the store into the pages in one launch
             k.gemm_qkv_rope(h, w, bias, qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache,
                             self.nh, self.nkv, self.hd, group.page_size, binding.writes, **scaled)

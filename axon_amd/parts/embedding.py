@@ -22,7 +22,7 @@ class TokenEmbedding(Part):
         self.vocab = int(params["vocab_size"])
         self.hidden = int(params["hidden_size"])
         self.name = prefix + params["tensor"]
-        self.table = None
+        self.table = None            # row-major, or a head's packed matrix (see LMHead.load)
 
     def tensors(self) -> List[TensorDecl]:
         return [TensorDecl(self.name, (self.vocab, self.hidden), "matrix")]
@@ -46,15 +46,21 @@ class LMHead(Part):
         self.tied_to = params.get("tied_to")
         self.tied = bool(params.get("tied", False))
         self.weight = None
+        self.source_name = None      # the tensor the head was loaded from
 
     def tensors(self) -> List[TensorDecl]:
         # tied: the head's own tensor is used if the checkpoint has one
         return [TensorDecl(self.name, (self.vocab, self.hidden), "matrix", optional=self.tied)]
 
     def load(self, store, rt) -> None:
-        self.weight = store.matrix(self.name, optional=self.tied)
-        if self.weight is None:
-            self.weight = store.matrix(self.tied_to)
+        self.source_name = self.name
+        weight = store.matrix(self.name, optional=self.tied)
+        if weight is None:
+            self.source_name = self.tied_to
+            weight = store.matrix(self.tied_to)
+        # packed for the matrix-core products where it can be; a tied embedding then reads the
+        # packed matrix too (the model hands it over), so that the matrix is in memory once
+        self.weight = rt.k.prepare_weight(weight)
 
     def forward(self, ctx, h, out=None):
         """h: [rows, hidden] in the compute dtype -> float32 logits [rows, vocab]."""

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 from typing import List
 
-from ..kernels import MODE_ADD_F32, MODE_SWIGLU
+from ..kernels import MODE_ADD_F32, MODE_SWIGLU, PackedMatrix
 from .base import FeedForward, TensorDecl, UnscaledRows, register_feed_forward
 
 
@@ -29,14 +29,17 @@ class SwiGLUMLP(FeedForward):
                 TensorDecl(self.n["down"], (self.hidden, self.ffn))]
 
     def load(self, store, rt) -> None:
-        self.w_gate_up = store.fused_matrix([self.n["gate"], self.n["up"]])
-        self.w_down = store.matrix(self.n["down"])
+        self.w_gate_up = rt.k.prepare_weight(store.fused_matrix([self.n["gate"], self.n["up"]]), gated=True)
+        self.w_down = rt.k.prepare_weight(store.matrix(self.n["down"]))
+        store.forget(self.n["down"])
 
     def takes_unscaled_rows(self, ctx) -> bool:
-        return ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.ffn, self.hidden, MODE_SWIGLU)
+        return (isinstance(self.w_gate_up, PackedMatrix)
+                and ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.ffn, self.hidden, MODE_SWIGLU))
 
     def folds_following_norm(self, ctx) -> bool:
-        return ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.hidden, self.ffn, MODE_ADD_F32)
+        return (isinstance(self.w_down, PackedMatrix)
+                and ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.hidden, self.ffn, MODE_ADD_F32))
 
     def forward(self, ctx, h, residual, fold=None) -> None:
         k = ctx.rt.k

@@ -90,6 +90,10 @@ class WeightStore:
         self._matrices[name] = t
         return t
 
+    def forget(self, name: str) -> None:
+        """Drop the store's reference to a matrix (its user keeps another form of it)."""
+        self._matrices.pop(name, None)
+
     def fused_matrix(self, names: List[str]) -> torch.Tensor:
         """The named [rows_i, K] matrices stacked into one [sum rows_i, K]."""
         shapes = [tuple(self.source.shape(n)) for n in names]

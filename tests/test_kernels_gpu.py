@@ -155,6 +155,12 @@ def test_attention_finds_a_far_key_and_respects_the_windows_edge(dtype):
         assert ((got[2] - vr[far, 1]).abs().max() < 1e-2) == seen
 
 
+def packed(k, w, gated=False):
+    """The matrix as a model's weights reach the products: packed for the matrix cores where it can
+    be (never in the float32 build), else row-major."""
+    return k.prepare_weight(w, gated)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (3, 100, 70), (17, 259, 130), (70, 96, 33), (130, 48, 257),
                                    (5, 1000, 512), (64, 256, 256), (200, 384, 1024), (33, 152, 3584), (64, 1000, 2048),
@@ -163,6 +169,7 @@ def test_gemm_every_epilogue(dtype, M, N, K):
     k = kernels(dtype)
     x, xr = as_dtype(rnd(M, K, seed=10), dtype)
     w, wr = as_dtype(rnd(N, K, seed=11, scale=0.2), dtype)
+    w = packed(k, w)
     ref = xr @ wr.T
     for bias_dt in (None, torch.float32, torch.bfloat16):
         bias = None if bias_dt is None else rnd(N, seed=12).to(bias_dt)
@@ -190,6 +197,7 @@ def test_gemm_with_the_gated_epilogue(dtype, M, F, K):
     k = kernels(dtype)
     x, xr = as_dtype(rnd(M, K, seed=30), dtype)
     w, wr = as_dtype(rnd(2 * F, K, seed=31, scale=0.3), dtype)
+    w = packed(k, w, gated=True)
     out = torch.empty(M, F, dtype=TORCH[dtype], device="cuda")
     k.gemm(x, w, out, None, MODE_SWIGLU)
     ref = P.swiglu(xr @ wr[:F].T, xr @ wr[F:].T)
@@ -208,6 +216,7 @@ def test_gemm_rows_do_not_depend_on_the_batch(dtype):
     for N, K in [(96, 80), (256, 512), (130, 1000), (512, 1024), (300, 4096), (200, 8192)]:
         x, _ = as_dtype(rnd(2100, K, seed=14), dtype)
         w, _ = as_dtype(rnd(N, K, seed=15, scale=0.2), dtype)
+        w = packed(k, w)
         whole = {}
         for rows in (16, 64, 256, 2048, 2100):
             whole[rows] = torch.empty(rows, N, dtype=torch.float32, device="cuda")
@@ -240,7 +249,7 @@ def test_gemm_with_a_norm_folded_in(M, H, F):
         x = res.clone().cuda()
         values = torch.empty(M, H, dtype=torch.bfloat16, device="cuda")
         squares = torch.full((M, H // 16), float("nan"), dtype=torch.float32, device="cuda")
-        k.gemm(a, wo, x, None, MODE_ADD_F32, following_norm=(gain.cuda(), values, squares))
+        k.gemm(a, packed(k, wo), x, None, MODE_ADD_F32, following_norm=(gain.cuda(), values, squares))
         assert (x.cpu().double() - x_ref).abs().max() <= 2e-5 * math.sqrt(F) * x_ref.abs().max()
         got_sq = squares.cpu().double().sum(1)
         assert ((got_sq - (x_ref ** 2).sum(1)).abs() <= 1e-5 * (x_ref ** 2).sum(1)).all()
@@ -249,12 +258,12 @@ def test_gemm_with_a_norm_folded_in(M, H, F):
             w, wr = as_dtype(rnd(N, H, seed=44, scale=0.2), "bfloat16")
             bias = rnd(N, seed=45)
             out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
-            k.gemm(values, w, out, bias.cuda(), MODE_STORE, row_squares=squares, eps=eps)
+            k.gemm(values, packed(k, w), out, bias.cuda(), MODE_STORE, row_squares=squares, eps=eps)
             want = h_ref @ wr.T + bias.double()
             assert (out.cpu().double() - want).abs().max() <= tol("bfloat16", want, 0, 1e-2)
         wg, wgr = as_dtype(rnd(2 * 80, H, seed=46, scale=0.2), "bfloat16")
         out = torch.empty(M, 80, dtype=torch.bfloat16, device="cuda")
-        k.gemm(values, wg, out, None, MODE_SWIGLU, row_squares=squares, eps=eps)
+        k.gemm(values, packed(k, wg, gated=True), out, None, MODE_SWIGLU, row_squares=squares, eps=eps)
         want = P.swiglu(h_ref @ wgr[:80].T, h_ref @ wgr[80:].T)
         assert (out.cpu().double() - want).abs().max() <= tol("bfloat16", want, 0, 1e-2)
 
@@ -285,7 +294,7 @@ def test_qkv_product_with_rotation_and_cache_store_in_one(M, nh, nkv, hd, hidden
     for bias_dt, write_kv in ((None, True), (torch.float32, True), (torch.bfloat16, False)):
         bias = None if bias_dt is None else rnd(width, seed=53).to(bias_dt).cuda()
         n_rows = width if write_kv else nh * hd
-        ww, bb = w[:n_rows], (None if bias is None else bias[:n_rows])
+        ww, bb = k.pack_matrix(w[:n_rows].contiguous()), (None if bias is None else bias[:n_rows])
         got, want = [], []
         for fused in (True, False):
             kc = torch.full((n_pages, nkv, page, hd), 7.0, dtype=torch.bfloat16, device="cuda")
@@ -309,7 +318,7 @@ def test_gemm_refuses_a_norm_it_cannot_fold():
     assert not k.gemm_norm_fold_ok(8, 64, 70, MODE_STORE)           # K that the matrix-core kernels refuse
     assert not kernels("float32").gemm_norm_fold_ok(8, 64, 64, MODE_STORE)
     x = torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda")
-    w = torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda")
+    w = k.pack_matrix(torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda"))
     out = torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(KernelError):
         k.gemm(x, w, out, None, MODE_STORE, row_squares=torch.zeros(17, 4, device="cuda"), eps=1e-6)

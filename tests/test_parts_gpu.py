@@ -193,3 +193,32 @@ def test_prenorm_block_with_the_norms_folded_into_the_products():
     # more rows than a folded step takes: the parts say so and the block runs its norms itself
     big = PartHarness(dtype, mixer.cache_spec())
     assert not mixer.takes_unscaled_rows(big.ctx([0] * 17)) and block.first_norm_fold(big.ctx([0] * 17), 17) is None
+
+
+def test_tied_head_and_embedding_share_the_packed_matrix(tmp_path):
+    """bfloat16, widths the matrix cores take: the head's matrix is repacked for its product and
+    the embedding reads rows out of that same copy (one matrix in memory); the rows are exact."""
+    from axon_amd.engine import Runtime
+    from axon_amd.engine.loading import load_model
+    from axon_amd.kernels import PackedMatrix
+    from helpers import make_model_dir
+    from axon_amd.weights.safetensors_io import Checkpoint
+    d = make_model_dir(str(tmp_path / "m"), "D", storage="bfloat16")            # tied, hidden 192
+    rt = Runtime("bfloat16")
+    model = load_model(d, rt)
+    assert isinstance(model.head.weight, PackedMatrix) and model.embedding.table is model.head.weight
+    table = Checkpoint(d).tensor("model.embed_tokens.weight")
+    toks = torch.tensor([0, 1, 15, 16, 17, 299, 150], dtype=torch.int32).cuda()
+    out = torch.empty(7, 192, dtype=torch.float32, device="cuda")
+    rt.k.embed(toks, model.embedding.table, out)
+    assert torch.equal(out.cpu(), table[toks.cpu().long()].float())
+    # a leading slice of whole row tiles is a view of the same storage; other cuts are refused
+    part = model.head.weight[:32]
+    assert part.shape == (32, 192) and part.data.data_ptr() == model.head.weight.data.data_ptr()
+    x = torch.randn(5, 192, device="cuda").bfloat16()
+    got = torch.empty(5, 32, dtype=torch.float32, device="cuda")
+    rt.k.gemm(x, part, got, None, 2)
+    ref = x.float().cpu().double() @ table[:32].double().T
+    assert (got.cpu().double() - ref).abs().max() <= 1e-4 * max(1.0, float(ref.abs().max()))
+    with pytest.raises(Exception):
+        model.head.weight[:40]
