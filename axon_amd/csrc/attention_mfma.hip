@@ -44,16 +44,18 @@ __device__ inline bf16x8 frag_of2(uint2 lo, uint2 hi) {
 __device__ inline uint32_t pack_bf16(float a, float b) { return pack2_bf16(a, b); }
 
 // ============================================================================ prompt portions
-// grid (tiles, query heads); a tile is up to 128 consecutive tokens of one request.  4 waves,
-// each owning 32 query rows.  Per block of 64 key positions the waves bring K [64][HD] and
+// grid (tiles, kv heads x groups of HPB query heads); a tile is up to 128 consecutive tokens of
+// one request.  4 waves per query head, each owning 32 query rows; with HPB = 2 two query heads of
+// the same kv head share every K and V^T block in LDS (the path from L2 into LDS carries about 32
+// bytes a cycle and CU, which is what one head's products use up).  Per block of 64 key positions the waves bring K [64][HD] and
 // V^T [HD][64] into LDS with direct global -> LDS loads (two stages: the next block's loads are
 // in flight while this one is multiplied).  16-byte slots of an LDS row are permuted
 // (slot ^ row & 7) so that fragment reads of neighbouring rows fall into different banks.
 #define PF_TOKENS 128
 #define PF_BLOCK 64
 
-template <int HD>
-__global__ void __launch_bounds__(256, 2)
+template <int HD, int HPB>
+__global__ void __launch_bounds__(256 * HPB, 2)
 attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
                          const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
@@ -66,14 +68,21 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
   constexpr int KROW = HD * 2;                    // bytes per K row
   constexpr int KCH = HD / 8;                     // 16-byte slots per K row
   constexpr int K_ROWS_PER_INSTR = 1024 / KROW;
-  constexpr int K_INSTR = PF_BLOCK / K_ROWS_PER_INSTR / 4;  // per wave
-  constexpr int V_INSTR = HD / 8 / 4;                       // V^T: 8 rows per instruction
+  constexpr int NW = 4 * HPB;                               // waves of the block
+  constexpr int K_INSTR = PF_BLOCK / K_ROWS_PER_INSTR / NW;  // per wave
+  constexpr int V_INSTR = HD / 8 / NW;                       // V^T: 8 rows per instruction
+  static_assert(K_INSTR >= 1 && V_INSTR >= 1, "more waves than load instructions");
   constexpr int DT = HD / 32;                     // output tiles (32 dims each)
   constexpr int KS = HD / 16;                     // k steps of S^T
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, block_wave = tid >> 6;
+  const int wave = block_wave & 3;                 // which 32 query rows of the tile
   const int t0 = tiles[2 * blockIdx.x], count = tiles[2 * blockIdx.x + 1];
-  const int head = blockIdx.y, kvh = head / (n_heads / n_kv_heads);
+  const int group = n_heads / n_kv_heads, sets = (group + HPB - 1) / HPB;   // sets of HPB query heads per kv head
+  const int kvh = blockIdx.y / sets;
+  const int in_group = (blockIdx.y % sets) * HPB + (block_wave >> 2);
+  const bool head_live = in_group < group;         // an odd group leaves the last set's second half idle
+  const int head = kvh * group + min(in_group, group - 1);
   const int pos0 = positions[t0];
   const int32_t* table_row = block_table + (size_t)seq_rows[t0] * table_stride;
   const int hi = pos0 + count - 1;                               // last position any row of the tile sees
@@ -87,7 +96,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
   const int my_lo = window > 0 ? max(0, my_pos + 1 - window) : 0;
   const int wave_hi = pos0 + min(wave * 32 + 31, count - 1);     // last position this wave's rows see
   const int wave_lo = window > 0 ? max(0, wave_hi + 1 - window) : 0;  // the latest window start among them
-  const bool wave_live = wave * 32 < count;
+  const bool wave_live = head_live && wave * 32 < count;
 
   // Q^T fragments (B operand): column = query row, 8 consecutive dims from 16 ks + 8 half
   bf16x8 qf[KS];
@@ -105,12 +114,12 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
     const int p0 = first_block + b * PF_BLOCK;
 #pragma unroll
     for (int n = 0; n < K_INSTR; ++n) {
-      const int row = (n * 4 + wave) * K_ROWS_PER_INSTR + lane / KCH;
+      const int row = (n * NW + block_wave) * K_ROWS_PER_INSTR + lane / KCH;
       k_page[n] = table_row[min(p0 + row, hi) / page_size];       // rows past the tile's last position: any valid row
     }
 #pragma unroll
     for (int n = 0; n < V_INSTR; ++n) {
-      const int d = (n * 4 + wave) * 8 + (lane >> 3);
+      const int d = (n * NW + block_wave) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ (d & 7);
       v_page[n] = table_row[min(p0 + chunk * 8, hi) / page_size];
     }
@@ -121,7 +130,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
     // K: lane i of an instruction brings row i / KCH, slot i % KCH holding chunk slot ^ (row & 7)
 #pragma unroll
     for (int n = 0; n < K_INSTR; ++n) {
-      const int instr = n * 4 + wave;
+      const int instr = n * NW + block_wave;
       const int row = instr * K_ROWS_PER_INSTR + lane / KCH;
       const int chunk = (lane % KCH) ^ (row & 7);
       const int p = min(p0 + row, hi);
@@ -132,7 +141,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
     // V^T: lane i brings row (dim) i / 8, slot i % 8 holding the 8 positions of chunk slot ^ (row & 7)
 #pragma unroll
     for (int n = 0; n < V_INSTR; ++n) {
-      const int instr = n * 4 + wave;
+      const int instr = n * NW + block_wave;
       const int d = instr * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ (d & 7);
       const int p = min(p0 + chunk * 8, hi);
@@ -175,7 +184,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
       // the last block: positions past `hi` were never written for this request.  Their
       // weights are zero, but zero times whatever the page holds must stay zero: clear them.
       const int first_bad = hi - p0 + 1;
-      for (int idx = tid; idx < HD * PF_BLOCK; idx += 256) {
+      for (int idx = tid; idx < HD * PF_BLOCK; idx += 64 * NW) {
         const int d = idx / PF_BLOCK, col = idx % PF_BLOCK;
         if (col >= first_bad) {
           const int slot = (col >> 3) ^ (d & 7);
@@ -230,16 +239,14 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
     // p0 + 32 pt + 16 (e / 8) + 8 half + (e % 8).  A block that every row of the wave sees whole
     // needs no mask (all but the blocks on the diagonal and at the window's edge).
     const bool whole = p0 + PF_BLOCK - 1 <= pos0 + wave * 32 && p0 >= wave_lo;
+    // the largest raw score first (the scale is positive), then exp2(score * c - max * c) in one
+    // multiply-add each
     float mloc = -INFINITY;
     if (whole) {
 #pragma unroll
       for (int pt = 0; pt < 2; ++pt)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const float v = s_acc[pt][e] * c;
-          s_acc[pt][e] = v;
-          mloc = fmaxf(mloc, v);
-        }
+        for (int e = 0; e < 16; ++e) mloc = fmaxf(mloc, s_acc[pt][e]);
     } else {
 #pragma unroll
       for (int pt = 0; pt < 2; ++pt)
@@ -247,13 +254,13 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
         for (int e = 0; e < 16; ++e) {
           const int p = p0 + pt * 32 + (e >> 3) * 16 + half * 8 + (e & 7);
           const bool seen = p <= my_pos && p >= my_lo;
-          const float v = seen ? s_acc[pt][e] * c : -INFINITY;
+          const float v = seen ? s_acc[pt][e] : -INFINITY;
           s_acc[pt][e] = v;
           mloc = fmaxf(mloc, v);
         }
     }
     mloc = fmaxf(mloc, __shfl_xor(mloc, 32, AXON_WAVE));
-    const float mn = fmaxf(m_run, mloc);
+    const float mn = fmaxf(m_run, mloc * c);
     const float mref = mn == -INFINITY ? 0.0f : mn;     // a row that has seen nothing yet
     const float alpha = __builtin_amdgcn_exp2f(m_run - mref);
     float lsum = 0.0f;
@@ -261,7 +268,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
     for (int pt = 0; pt < 2; ++pt)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const float pv = __builtin_amdgcn_exp2f(s_acc[pt][e] - mref);
+        const float pv = __builtin_amdgcn_exp2f(fmaf(s_acc[pt][e], c, -mref));
         s_acc[pt][e] = pv;
         lsum += pv;
       }
@@ -552,13 +559,14 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
               "attention_prefill: bad arguments (tiles %d, heads %d, window %d, q stride %d)", n_tiles, n_heads, window,
               q_stride);
   if (n_tiles == 0) return 0;
-  dim3 grid(n_tiles, n_heads);
-#define LAUNCH(HD)                                                                                                  \
+  const int group = n_heads / n_kv_heads;
+#define LAUNCH(HD, HPB)                                                                                             \
   {                                                                                                                 \
     static bool configured = false;                                                                                 \
     constexpr int lds = 2 * (PF_BLOCK * HD * 2 + HD * PF_BLOCK * 2);                                                \
+    const dim3 grid(n_tiles, n_kv_heads * ((group + HPB - 1) / HPB));                                               \
     if (!configured) {                                                                                              \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<HD>),              \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<HD, HPB>),         \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);                          \
       if (e != hipSuccess) {                                                                                        \
         axk_set_error("attention_prefill: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));          \
@@ -566,11 +574,16 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
       }                                                                                                             \
       configured = true;                                                                                            \
     }                                                                                                               \
-    attention_prefill_kernel<HD><<<grid, 256, lds, (hipStream_t)stream>>>(                                          \
+    attention_prefill_kernel<HD, HPB><<<grid, 256 * HPB, lds, (hipStream_t)stream>>>(                               \
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,      \
         positions, seq_rows, (bf16_t*)out, tiles, n_heads, n_kv_heads, page_size, window, scale);                   \
   }
-  if (head_dim == 64) LAUNCH(64) else LAUNCH(128)
+  // two query heads a block where a kv head has more than one
+  if (group >= 2) {
+    if (head_dim == 64) LAUNCH(64, 2) else LAUNCH(128, 2)
+  } else {
+    if (head_dim == 64) LAUNCH(64, 1) else LAUNCH(128, 1)
+  }
 #undef LAUNCH
   AXK_LAUNCH_CHECK("attention_prefill");
   return 0;
