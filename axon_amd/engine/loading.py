@@ -32,6 +32,7 @@ def load_model(model_dir: str, rt: Runtime) -> DecoderModel:
     source = CheckpointSource(ck)
     check_tensors(model.tensors(), source)
     model.load(WeightStore(source, rt.device, rt.dtype), rt)
+    _release_staging(rt)
     return model
 
 
@@ -41,4 +42,13 @@ def random_model(config: ModelConfig, rt: Runtime, seed: int = 0, std: float = 0
     storage = torch.bfloat16 if rt.dtype == torch.bfloat16 else torch.float32
     source = RandomSource(model.tensors(), seed, std=std, storage=storage)
     model.load(WeightStore(source, rt.device, rt.dtype), rt)
+    _release_staging(rt)
     return model
+
+
+def _release_staging(rt: Runtime) -> None:
+    """The row-major copies that were repacked are gone; give their memory back to the device,
+    so that the cache pool, which is sized from what is free, can have it."""
+    if rt.device is not None and torch.cuda.is_available():
+        torch.cuda.synchronize(rt.device)
+        torch.cuda.empty_cache()

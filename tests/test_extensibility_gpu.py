@@ -1,6 +1,7 @@
 """(c)'s generality, shown with toy parts that exist only in this file: a mixer with state of
-its own, another position encoding, windowed attention layers with pages of their own, a layer
-that runs twice and a run that reads another run's cache.  The toy architecture is registered,
+its own, a feed-forward that routes between experts, another position encoding, windowed
+attention layers with pages of their own, a layer that runs twice and a run that reads another
+run's cache.  The toy architecture is registered,
 built, loaded from a folder written by the random-weights mode and stepped, without a change
 to the framework's files, and compared with a plain implementation written here."""
 import json
@@ -13,7 +14,8 @@ import axon_amd
 from axon_amd.config import (LayerSpec, ModelConfig, ModelSpec, PartSpec, Run, register_architecture)
 from axon_amd.config.base import get_number, get_whole
 from axon_amd.engine import StepEntry
-from axon_amd.parts import Mixer, StateSpec, TensorDecl, register_mixer, register_position
+from axon_amd.parts import (FeedForward, Mixer, StateSpec, TensorDecl, build_part, register_feed_forward, register_mixer,
+                            register_position)
 from axon_amd.parts.rope import RotaryEncoding
 from axon_amd.weights import write_random_model
 from helpers import tolerance
@@ -61,8 +63,38 @@ class HalvedRope(RotaryEncoding):
         return super().frequencies() * 0.5
 
 
+class RoutedFFN(FeedForward):
+    """A toy mixture of experts: router logits (32-bit) -> softmax -> the experts' outputs weighted
+    by it.  Each expert is the framework's own dense feed-forward under a scope of its own; every
+    expert sees every token here (a soft router: no token changes expert by rounding)."""
+
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        self.hidden, self.n = int(params["hidden_size"]), int(params["experts"])
+        self.router_name = prefix + "mlp.router.weight"
+        self.experts = [build_part("feed_forward", PartSpec("swiglu_mlp", {
+            "hidden_size": self.hidden, "intermediate_size": int(params["intermediate_size"]),
+            "names": {"scope": f"mlp.experts.{e}."}}), prefix) for e in range(self.n)]
+
+    def tensors(self):
+        return [TensorDecl(self.router_name, (self.n, self.hidden))] + [d for e in self.experts for d in e.tensors()]
+
+    def load(self, store, rt):
+        self.router = store.matrix(self.router_name).float()
+        for e in self.experts:
+            e.load(store, rt)
+
+    def forward(self, ctx, h, residual):
+        weights = torch.softmax(h.float() @ self.router.T, dim=-1)          # [T, experts], 32-bit
+        for e, expert in enumerate(self.experts):
+            out = torch.zeros_like(residual)
+            expert.forward(ctx, h, out)                                     # adds its output into `out`
+            residual += weights[:, e:e + 1] * out
+
+
 register_mixer("toy_decay", DecayMixer)
 register_position("toy_halved_rope", HalvedRope)
+register_feed_forward("toy_routed", RoutedFFN)
 
 
 class ToyConfig(ModelConfig):
@@ -94,8 +126,9 @@ class ToyConfig(ModelConfig):
         rope = PartSpec("rope", {"head_dim": self.head_dim, "theta": 1000.0})
         halved = PartSpec("toy_halved_rope", {"head_dim": self.head_dim, "theta": 1000.0})
         decay = PartSpec("toy_decay", {"hidden_size": self.hidden, "state_size": self.state, "decay": self.decay})
+        routed = PartSpec("toy_routed", {"hidden_size": self.hidden, "intermediate_size": self.ffn, "experts": 3})
         layers = [LayerSpec("prenorm", attn(self.window, rope), ffn, norm, "layers.0."),     # windowed attention
-                  LayerSpec("prenorm", decay, ffn, norm, "layers.1."),                      # state of its own
+                  LayerSpec("prenorm", decay, routed, norm, "layers.1."),                   # state of its own; routed experts
                   LayerSpec("prenorm", attn(0, halved), ffn, norm, "layers.2.")]            # full, other positions
         # layer 0 runs twice (each run its own cache); the last run reads what layer 2 stored
         order = [Run(0, cache=0), Run(1, cache=1), Run(2, cache=2), Run(0, cache=3), Run(2, cache=2, writes_cache=False)]
@@ -149,8 +182,13 @@ def toy_plain(w, tokens):
             s = c["decay"] * s + u[t]
             outs.append(s)
         x = x + torch.stack(outs) @ w[p + "mixer.out.weight"].T
-        return x + P.mlp_block({k2.replace(p, "model.layers.0."): v2 for k2, v2 in w.items() if k2.startswith(p + "mlp")}, 0,
-                               P.rms_norm(x, w[p + "post_attention_layernorm.weight"], c["eps"]))
+        h = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], c["eps"])
+        weights = torch.softmax(h @ w[p + "mlp.router.weight"].T, dim=-1)
+        for e in range(3):
+            scope = f"{p}mlp.experts.{e}."
+            expert = {k2.replace(scope, "model.layers.0.mlp."): v2 for k2, v2 in w.items() if k2.startswith(scope)}
+            x = x + weights[:, e:e + 1] * P.mlp_block(expert, 0, h)
+        return x
 
     x = attention(x, 0, c["window"], 1.0)
     x = decay(x, 1)
@@ -179,6 +217,7 @@ def test_the_toy_architecture_is_described_by_its_parts(toy_dir):
         (0, 0, True, -1), (-1, -1, True, 0), (1, 0, True, -1), (0, 1, True, -1), (1, 0, False, -1)]
     names = {d.name for d in model.tensors()}
     assert "layers.1.mixer.in.weight" in names and "layers.0.self_attn.q_proj.bias" in names
+    assert "layers.1.mlp.router.weight" in names and "layers.1.mlp.experts.2.down_proj.weight" in names
     assert json.load(open(os.path.join(toy_dir, "config.json")))["architectures"] == ["ToyForCausalLM"]
 
 
