@@ -8,26 +8,31 @@
 // more bandwidth than 16 rows x 64 bytes of a row-major matrix), lands in LDS without a
 // permutation, and the same bytes serve the 16x16x32 and the 32x32x16 MFMA.
 //
-// Two kernels, chosen by M alone so that a given (N, K) always meets the same pair:
+// Two kernels, chosen by the number of rows M alone, so that a given (N, K) always meets the same
+// kernel and the same grouping of k for a given class of M:
 //
-// * gemm_tile (M > 64): a block of 4 or 8 waves owns a BM x BN tile of the output (256 x 256,
-//   or 128 x 128 when that would leave CUs without work), walks K in steps of 64 through two
-//   LDS stages filled by direct global -> LDS loads (the next step's loads in flight while
-//   this one multiplies), and each wave keeps a tile of 32x32x16 MFMA accumulators.  The
-//   16-byte slots of an LDS row are permuted so that fragment reads of neighbouring rows fall
-//   into different banks.  Blocks are numbered so that the blocks of one XCD (every eighth
-//   block) share weight tiles in that XCD's L2.
+// * gemm_skinny (M <= 16, decoding): bound by reading W once.  A block owns one or two row tiles
+//   of W; its four waves split K between them and stream their share from memory straight into
+//   MFMA operands (16x16x32), keeping a ring of steps in flight so that the memory pipe never
+//   drains; each multiplies with up to 16 rows of X, and the waves' sums are added in wave
+//   order through LDS.  No atomics, so the result does not depend on timing.  Epilogues: bias /
+//   residual add / SwiGLU, an RMS norm folded in on either side, and the attention's qkv product
+//   with the rotary encoding and the store into the paged cache.
 //
-// * gemm_skinny (M <= 64, decoding): bound by reading W once.  A block owns 16 or 32 rows of
-//   W; its four waves split K between them and stream their share from memory straight into
-//   MFMA fragments (16x16x32: a lane's 8 consecutive k are one 16-byte load), keeping a ring
-//   of steps in flight so that the memory pipe never drains; each multiplies with up to 64
-//   rows of X, and the waves' partial sums are added in wave order through LDS.  No atomics,
-//   so the result does not depend on timing.
+// * gemm_tile (M > 16): a block of 4 or 8 waves owns a BM x BN tile of the output, walks K in
+//   steps of 64 through LDS stages filled by direct global -> LDS loads (the next step's loads
+//   in flight while this one multiplies), and each wave keeps a tile of 32x32x16 MFMA
+//   accumulators.  X rows land in LDS with their 16-byte slots permuted so that fragment reads
+//   of neighbouring rows fall into different banks; W blocks land as they are.  Blocks are
+//   numbered so that the blocks of one XCD (every eighth block) share weight tiles in that
+//   XCD's L2.  Tiles: 64 x 128 / 64 x 256 for 17 to 64 rows, 128 x 128 for 65 to 256, and 256 x 256
+//   or 128 x 128 beyond, by how they fill the chip.  Where the output gives too few tiles for
+//   256 CUs, K is split between blocks (by (N, K) alone within a class of M), the blocks' sums go
+//   through a workspace and gemm_split_reduce adds them in block order and applies the epilogue.
 //
-// The two kernels sum k in different groupings, so a row's bits differ between M <= 64 and
-// M > 64 by rounding (and only by rounding); within one kernel a row does not depend on the
-// other rows of the batch.
+// Classes of M: <= 16, 17..64, 65..256, 257..2048, > 2048.  Within a class a row's bits do not
+// depend on the other rows of the batch; between classes they differ by the rounding of 32-bit
+// sums (and only by that).
 #include "api.h"
 #include "common.h"
 
@@ -49,14 +54,15 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 __device__ inline bf16x8 as_frag(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
 // ---------------------------------------------------------------------------- gemm_tile
-// LDS holds STAGES stages; a stage is BM rows of X and BN rows of W, BK k each, written by
-// direct global -> LDS loads of 16 bytes per lane (a wave instruction fills 1024 bytes of
-// consecutive rows).  The loads of step kt + STAGES - 1 are issued while step kt is multiplied,
-// so the latency of L2 and of the path into LDS is covered by STAGES - 1 steps of MFMAs.
+// LDS holds STAGES stages; a stage is BM rows of X and the BN / 16 x BK / 32 packed blocks of W,
+// written by direct global -> LDS loads of 16 bytes per lane (a wave instruction fills 1024
+// bytes: 8 rows of X, or one block of W).  Every stage is filled before the loop, and the loads
+// of step kt + STAGES go out as soon as step kt's stage is free, so the latency of L2 and of
+// the path into LDS is covered by STAGES - 1 steps of MFMAs.
 //
-// A row of a stage is BK / 8 slots of 16 bytes, permuted so that fragment reads of neighbouring
-// rows at one k chunk fall into different banks without padding (which direct loads could
-// not skip).  LDS serves 256 bytes a cycle (64 banks): a 16-byte read of 16 consecutive lanes
+// A row of X in a stage is BK / 8 slots of 16 bytes, permuted so that fragment reads of
+// neighbouring rows at one k chunk fall into different banks without padding (which direct
+// loads could not skip).  LDS serves 256 bytes a cycle (64 banks): a 16-byte read of 16 consecutive lanes
 // (16 consecutive rows, the same k chunk) is conflict-free when the rows' 16-byte positions
 // modulo 256 differ.  With 128-byte rows (BK 64) that is slot = chunk ^ ((row >> 1) & 7); with
 // 64-byte rows (BK 32) slot = chunk ^ ((row >> 2) & 3).
