@@ -1,7 +1,7 @@
 """The benchmark: decode tokens per second of the Qwen2.5-7B-sized model (random weights,
 bfloat16) on one MI355X, plus prefill throughput and the decode step's memory roofline.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--prompt N]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--prompt N] [--sizes 7b|14b|32b]
 
 A "step" is one decode step of the whole batch: every live request advances by one token
 through the engine's own step function (HIP graph replay) and its device argmax.  Before the
@@ -25,6 +25,12 @@ PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 SIZES_7B = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=28, hidden_size=3584,
                 intermediate_size=18944, num_attention_heads=28, num_key_value_heads=4, head_dim=128, vocab_size=152064,
                 max_position_embeddings=8192, rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
+# the further sizes of the same architecture (--sizes): layers, width, heads, feed-forward width, eps
+SIZES = {"7b": SIZES_7B,
+         "14b": dict(SIZES_7B, num_hidden_layers=48, hidden_size=5120, intermediate_size=13824, num_attention_heads=40,
+                     num_key_value_heads=8, rms_norm_eps=1e-5),
+         "32b": dict(SIZES_7B, num_hidden_layers=64, hidden_size=5120, intermediate_size=27648, num_attention_heads=40,
+                     num_key_value_heads=8, rms_norm_eps=1e-5)}
 
 
 def main() -> int:
@@ -36,6 +42,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0: all)")
     ap.add_argument("--prompt", type=int, default=2048, help="prompt tokens of every request")
     ap.add_argument("--dtype", default="bfloat16")
+    ap.add_argument("--sizes", default="7b", choices=sorted(SIZES), help="layer sizes of Qwen2.5-7B (the default), 14B or 32B")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
                     help="for profiling: time only the prefill step (repeated --steps times) or only decoding")
@@ -49,7 +56,8 @@ def main() -> int:
     import axon_amd
     from axon_amd.engine import StepEntry
 
-    cfg = dict(SIZES_7B)
+    cfg = dict(SIZES[args.sizes])
+    name = f"Qwen2.5-{args.sizes.upper()} sizes"
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -126,11 +134,11 @@ def main() -> int:
                 points[f"decode_b{b}"] = round(decode(b, max(8, args.steps // 2), args.warmup)[0], 1)
     achieved = bytes_read / step_s / 1e9
     line = {
-        "metric": f"decode tok/s (Qwen2.5-7B sizes, {args.dtype}, batch {args.batch}, {args.prompt}-token prompts)",
+        "metric": f"decode tok/s ({name}, {args.dtype}, batch {args.batch}, {args.prompt}-token prompts)",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random N(0, 0.02) weights, uniform random token ids",
-        "config": {"model": "Qwen2.5-7B sizes", "layers": L, "layers_of_config": full_layers, "hidden": dim,
+        "config": {"model": name, "layers": L, "layers_of_config": full_layers, "hidden": dim,
                    "heads": nh, "kv_heads": nkv, "head_dim": hd, "intermediate": ffn, "vocab": V, "batch": args.batch,
                    "global_batch": args.batch, "seq_len": args.prompt, "context": ctx_len, "page_size": page,
                    "parallelism": "single GPU", "graphs": bool(eng.graphs_ok)},
