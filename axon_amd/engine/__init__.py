@@ -1,4 +1,4 @@
 from .runtime import Runtime, Workspace
-from .step import Engine, LiveRequest, Span, StepContext, StepEntry, StepError
+from .step import Engine, LiveRequest, PendingPicks, Span, StepContext, StepEntry, StepError
 
-__all__ = ["Runtime", "Workspace", "Engine", "LiveRequest", "Span", "StepContext", "StepEntry", "StepError"]
+__all__ = ["Runtime", "Workspace", "Engine", "LiveRequest", "PendingPicks", "Span", "StepContext", "StepEntry", "StepError"]

@@ -96,23 +96,54 @@ class LLM:
         stop = set(int(s) for s in stop)
         cache = self.engine.cache
         n_groups = len(cache.groups)
+        # Greedy decoding without stop tokens runs one step ahead of the host: a step takes its
+        # tokens from the picks of the step before on the device (Engine.step_from_picks), and the
+        # picks are read a step late, while the next step runs.  Until they are read the requests'
+        # lists hold None in their place.  What ends a request is then known without the token.
+        ahead_ok = not stop
+        behind = None            # (picks on their way, the requests they belong to)
+
+        def settle(behind):
+            picks, ids = behind
+            for rid, tok in zip(ids, picks.tolist()):
+                r = reqs[rid]
+                at = len(r.tokens) - 1
+                while r.tokens[at] is not None:      # the one place that is still open
+                    at -= 1
+                r.tokens[at] = int(tok)
+                r.out[at - r.prompt_len] = int(tok)
+
         try:
             while any(not r.done for r in reqs.values()):
                 plan, preempted = sched.plan([cache.free_pages(g) for g in range(n_groups)])
+                feed = (behind is not None and not preempted and [p.id for p in plan] == behind[1]
+                        and all(p.count == 1 and p.wants_logits for p in plan))
+                if behind is not None and not feed:
+                    settle(behind)
+                    behind = None
                 for rid in preempted:
                     self.engine.release(rid)
                     stats.preemptions += 1
                 if not plan:
                     raise RuntimeError("the scheduler has requests but planned nothing: the cache pool is too small")
-                entries = [StepEntry(p.id, reqs[p.id].tokens[p.start:p.start + p.count],
-                                     [p.count - 1] if p.wants_logits else []) for p in plan]
                 t_step = time.time()
-                logits = self.engine.step(entries)
+                if feed:
+                    logits = self.engine.step_from_picks([p.id for p in plan])
+                    settle(behind)               # the step before: read while this one runs
+                    behind = None
+                else:
+                    entries = [StepEntry(p.id, reqs[p.id].tokens[p.start:p.start + p.count],
+                                         [p.count - 1] if p.wants_logits else []) for p in plan]
+                    logits = self.engine.step(entries)
                 stats.steps += 1
                 wanted = [p for p in plan if p.wants_logits]
+                greedy_step = bool(wanted) and all(reqs[p.id].sampler is None for p in wanted)
                 picks = []
+                late = None
                 if wanted:
-                    if self.engine.last_picks is not None and all(reqs[p.id].sampler is None for p in wanted):
+                    if greedy_step and ahead_ok and len(wanted) == len(plan) and self.engine.picks_async() is not None:
+                        late = self.engine.picks_async()        # read after the next step is queued
+                    elif greedy_step and self.engine.last_picks is not None:
                         picks = self.engine.last_picks.tolist()     # a decoding step picked greedily already
                     else:
                         picks = pick_rows(self.rt, logits, [reqs[p.id].sampler for p in wanted],
@@ -122,10 +153,10 @@ class LLM:
                     r = reqs[p.id]
                     appended = finished = False
                     if p.wants_logits:
-                        tok = int(picks[at])
+                        tok = None if late is not None else int(picks[at])
                         at += 1
                         stats.decided += 1
-                        if tok in stop:
+                        if tok is not None and tok in stop:
                             finished = True
                         else:
                             r.tokens.append(tok)
@@ -138,6 +169,8 @@ class LLM:
                     if finished:
                         r.done = True
                         self.engine.release(p.id)
+                if late is not None:
+                    behind = (late, [p.id for p in plan])
                 dt = time.time() - t_step
                 if all(p.count == 1 and p.start > 0 for p in plan):
                     stats.decode_seconds += dt
@@ -146,6 +179,9 @@ class LLM:
                 else:
                     stats.prompt_seconds += dt
                     stats.prompt_tokens += sum(p.count for p in plan if p.wants_logits and p.count > 1)
+            if behind is not None:
+                settle(behind)
+                behind = None
         finally:
             for rid in order:
                 self.engine.release(rid)

@@ -77,6 +77,22 @@ class StepContext:
         return torch.empty((self.n_tokens, 0, 2), dtype=torch.float32, device=self.rt.device)
 
 
+class PendingPicks:
+    """The greedy picks of a decoding step on their way to the host: the copy was queued behind
+    the step, `tolist` waits for it alone (later steps may already be running).  The staging
+    buffer is one of a ring of four: read it before three further decoding steps are queued."""
+
+    def __init__(self, buffer: torch.Tensor, event, n: int):
+        self._buffer, self._event, self._n = buffer, event, n
+        self._values: Optional[List[int]] = None
+
+    def tolist(self) -> List[int]:
+        if self._values is None:
+            self._event.synchronize()
+            self._values = self._buffer[:self._n].tolist()
+        return self._values
+
+
 class Engine:
     def __init__(self, model: DecoderModel, rt: Runtime, cfg: EngineConfig):
         self.model = model
@@ -104,7 +120,14 @@ class Engine:
                 seen.add(pair[0])
                 self._shape_mixers.append(b.mixer)
         self._meta = torch.zeros((3, cfg.max_seqs), dtype=torch.int32, device=rt.device)
-        self._meta_host = torch.zeros((3, cfg.max_seqs), dtype=torch.int32).pin_memory()
+        # staging in pinned memory, a ring: a step's inputs and picks travel while the host
+        # prepares the next step
+        self._meta_hosts = [torch.zeros((3, cfg.max_seqs), dtype=torch.int32).pin_memory() for _ in range(4)]
+        self._pick_hosts = [torch.zeros(cfg.max_seqs, dtype=torch.int32).pin_memory() for _ in range(4)]
+        self._ring_events = [None] * 4
+        self._ring_at = 0
+        self._last_decode: Optional[List[Hashable]] = None      # the requests of the last decoding step, in order
+        self._pending: Optional[PendingPicks] = None
         self._index = torch.arange(cfg.max_seqs, dtype=torch.int32, device=rt.device)
         self._logits = None
         self._picks = torch.zeros(cfg.max_seqs, dtype=torch.int32, device=rt.device)
@@ -134,6 +157,8 @@ class Engine:
         req = self.live.pop(rid, None)
         if req is not None:
             self.cache.close(req.slot)
+            if self._last_decode is not None and rid in self._last_decode:
+                self._last_decode = None
 
     def release_all(self) -> None:
         for rid in list(self.live):
@@ -181,6 +206,8 @@ class Engine:
 
         logits = None
         self.last_picks = None
+        self._last_decode = None
+        self._pending = None
         if entries:
             tokens, positions, rows, want_rows, spans = [], [], [], [], []
             for e in entries:
@@ -196,6 +223,7 @@ class Engine:
             self.cache.sync_tables()
             if T == len(entries) and len(want_rows) == T and T <= self.cfg.max_seqs:
                 logits = self._decode_step(tokens, positions, rows, spans)
+                self._last_decode = [e.id for e in entries]
             else:
                 meta = torch.tensor([tokens, positions, rows], dtype=torch.int32).to(self.rt.device)
                 ctx = StepContext(self.rt, self.cache, self.ws, meta, T, spans)
@@ -212,6 +240,38 @@ class Engine:
         for rid in end:
             self.release(rid)
         return logits
+
+    def step_from_picks(self, ids: Sequence[Hashable]) -> torch.Tensor:
+        """One more decoding step for exactly the requests of the last decoding step, in its
+        order: each takes as its token the greedy pick that step made for it.  The pick is taken
+        on the device, so the host need not have read it yet: it can queue this step and read
+        the previous step's picks (`picks_async`) while this one runs.  Returns the logits as
+        `step` does."""
+        ids = list(ids)
+        if self._last_decode is None or ids != self._last_decode:
+            raise StepError("step_from_picks continues the last decoding step: the same requests in the same order")
+        reqs = [self.live[rid] for rid in ids]
+        for rid, req in zip(ids, reqs):
+            if req.n_cached + 1 > self.max_seq_len:
+                raise StepError(f"request {rid!r} would reach {req.n_cached + 1} positions, at most {self.max_seq_len}")
+        for req in reqs:
+            self.cache.reserve(req.slot, req.n_cached + 1)      # OutOfPages: nothing has run
+        positions = [req.n_cached for req in reqs]
+        rows = [req.slot for req in reqs]
+        spans = [Span(req.slot, i, 1, req.n_cached) for i, req in enumerate(reqs)]
+        self.cache.sync_tables()
+        logits = self._decode_step(None, positions, rows, spans)
+        for req in reqs:
+            req.n_cached += 1
+            if self.has_window:
+                self.cache.trim(req.slot, req.n_cached)
+        self.steps += 1
+        return logits
+
+    def picks_async(self) -> Optional[PendingPicks]:
+        """The last decoding step's greedy picks as a copy that is under way (None after any
+        other step)."""
+        return self._pending
 
     # ------------------------------------------------------------------ decoding steps
     def _decode_forward(self, T: int, spans: List[Span], shapes: Dict):
@@ -231,13 +291,24 @@ class Engine:
         device buffers; with graphs on, the launches of this (number of tokens, shape) are
         captured once and replayed afterwards.  Returns a view of a static logits buffer, valid
         until the next decoding step; `last_picks` holds the greedy pick of each row."""
-        T = len(tokens)
+        T = len(positions)
         if self._logits is None:
             self._logits = torch.empty((self.cfg.max_seqs, self.model.vocab_size), dtype=torch.float32,
                                        device=self.rt.device)
-        host = self._meta_host
-        host[:, :T] = torch.tensor([tokens, positions, rows], dtype=torch.int32)
-        self._meta.copy_(host)          # one small copy, complete before the host buffer is written again
+        # inputs through a ring of pinned buffers, without waiting: a buffer is written again only
+        # after the copies that read or wrote it have run
+        at = self._ring_at = (self._ring_at + 1) % len(self._meta_hosts)
+        if self._ring_events[at] is not None:
+            self._ring_events[at].synchronize()
+        host = self._meta_hosts[at]
+        if tokens is None:
+            # the tokens are the previous step's picks, already on the device
+            host[1:, :T] = torch.tensor([positions, rows], dtype=torch.int32)
+            self._meta[1:].copy_(host[1:], non_blocking=True)
+            self._meta[0, :T].copy_(self._picks[:T])
+        else:
+            host[:, :T] = torch.tensor([tokens, positions, rows], dtype=torch.int32)
+            self._meta.copy_(host, non_blocking=True)
         shapes = {}
         for mixer in self._shape_mixers:
             name, value = mixer.decode_shape(positions)
@@ -261,4 +332,10 @@ class Engine:
             entry[0].replay()
             logits = entry[1]
         self.last_picks = self._picks[:T]
+        # the picks start their way to the host behind the step
+        self._pick_hosts[at][:T].copy_(self._picks[:T], non_blocking=True)
+        event = self._ring_events[at] or torch.cuda.Event()
+        event.record()
+        self._ring_events[at] = event
+        self._pending = PendingPicks(self._pick_hosts[at], event, T)
         return logits

@@ -66,7 +66,7 @@ def main() -> int:
     ctx_len, page = cfg["max_position_embeddings"], 16
     elem = 2 if args.dtype == "bfloat16" else 4
     most_batch = args.batch if args.no_points else max(args.batch, 64)
-    tokens_needed = most_batch * (args.prompt + args.steps + args.warmup + 16)
+    tokens_needed = most_batch * (args.prompt + args.steps + args.warmup + 17)
     llm = axon_amd.load(cfg, dtype=args.dtype, random_seed=0, init_std=0.02, page_size=page,
                         num_pages=-(-tokens_needed // page) + most_batch, max_seqs=most_batch,
                         max_batch_tokens=max(args.prompt, 2048), max_seq_len=ctx_len)
@@ -103,19 +103,29 @@ def main() -> int:
             eng.step([StepEntry(rid, pr[:-1], [])])
             last.append(pr[-1])
 
-        def one(tokens):
-            eng.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, tokens)])
-            return eng.last_picks.tolist()           # the greedy picks come back to the host, as in serving
+        # The first step takes its tokens from the host.  Every later step takes each request's
+        # token from the pick the step before made for it, on the device, and the greedy picks
+        # come back to the host one step behind, while the next step runs: as `generate` decodes.
+        eng.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, last)])
+        pending = eng.picks_async()
+
+        def one(pending):
+            eng.step_from_picks(ids)
+            behind = eng.picks_async()
+            pending.tolist()
+            return behind
 
         for _ in range(warmup):
-            last = one(last)
+            pending = one(pending)
+        pending.tolist()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            last = one(last)
+            pending = one(pending)
+        pending.tolist()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        mid_ctx = args.prompt + warmup + steps / 2
+        mid_ctx = args.prompt + 1 + warmup + steps / 2
         for rid in ids:
             eng.release(rid)
         kv_bytes = batch * mid_ctx * L * 2 * nkv * hd * elem

@@ -59,6 +59,53 @@ def test_sampled_generation_matches_the_plain_sampler(model_dirs):
                                       repeat_penalty=1.0, repeat_last_n=64, seed=9)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_one_step_ahead_of_the_host(dtype, model_dirs):
+    """A step fed from the previous step's picks on the device gives the logits and tokens of a
+    step fed the same tokens from the host, bit for bit; and generation that runs ahead (greedy,
+    no stop tokens) returns what generation that reads every token first returns."""
+    from axon_amd.engine import StepEntry
+    d = model_dirs("B", dtype)
+    prompts = prompts_for("B", [7, 30, 19], seed=11)
+    ahead = axon_amd.load(d, dtype=dtype, page_size=16, num_pages=32, max_seqs=4, max_batch_tokens=64).engine
+    plain = axon_amd.load(d, dtype=dtype, page_size=16, num_pages=32, max_seqs=4, max_batch_tokens=64).engine
+    ids = ["x", "y", "z"]
+    for eng in (ahead, plain):
+        for rid, p in zip(ids, prompts):
+            eng.step([StepEntry(rid, p[:-1], [])])
+    first = [StepEntry(rid, [p[-1]], [0]) for rid, p in zip(ids, prompts)]
+    ahead.step(first)
+    late = ahead.picks_async()
+    plain.step(first)
+    toks = plain.last_picks.tolist()
+    assert late.tolist() == toks
+    for i in range(20):
+        got = ahead.step_from_picks(ids).clone()
+        behind, late = late, ahead.picks_async()
+        assert behind.tolist() == toks
+        want = plain.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, toks)])
+        assert torch.equal(got, want), i
+        toks = plain.last_picks.tolist()
+    assert late.tolist() == toks
+    with pytest.raises(axon_amd.engine.StepError):
+        ahead.step_from_picks(["x", "y"])                   # not the last step's requests
+    ahead.release("z")
+    with pytest.raises(axon_amd.engine.StepError):
+        ahead.step_from_picks(ids)
+    ahead.release_all()
+    ahead.cache.check()
+
+    llm = axon_amd.load(d, dtype=dtype, page_size=16, num_pages=32, max_seqs=4, max_batch_tokens=24)
+    more = prompts_for("B", [5, 40, 12, 26, 9], seed=12)
+    run_ahead = llm.generate(more, max_new_tokens=21)
+    steps_ahead = llm.last_stats.steps
+    one_by_one = llm.generate(more, max_new_tokens=21, stop=[-1])      # a stop token: every token is read first
+    assert run_ahead == one_by_one and steps_ahead == llm.last_stats.steps
+    assert all(len(o) == 21 and None not in o for o in run_ahead)
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_pages() == 32 and not llm.engine.live
+
+
 def test_stop_tokens_end_a_request_and_are_not_returned(model_dirs):
     d = model_dirs("A")
     cfg, w = P.load_plain(d)
