@@ -54,15 +54,17 @@ int axk_attention(const void* q, int q_stride, const void* k_cache, const void* 
 // axk_attention_fast_ok: 1 if they take this head size, page size and group of heads.
 // axk_attention_prefill: tiles [n_tiles][2] = (first token, count <= 128): consecutive tokens of
 // one request; every token of the step in some tile gets its row of `out`.
-// axk_attention_decode: token_index [n_tokens] names single tokens; a context longer than 64
-// positions is cut into chunks of 64 whose partial results go through `partial`
-// (axk_attention_decode_workspace floats) and are folded in ascending order.
+// axk_attention_decode: token_index [n_tokens] names single tokens; a context longer than one
+// chunk (axk_attention_decode_chunk positions) is cut into chunks whose partial results go
+// through `partial` (axk_attention_decode_workspace floats) and are folded in ascending order;
+// max_chunks is the most chunks any of the tokens has.
 int axk_attention_fast_ok(int head_dim, int page_size, int n_heads, int n_kv_heads);
 int axk_attention_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                           const int32_t* block_table, int table_stride, const int32_t* positions,
                           const int32_t* seq_rows, void* out, const int32_t* tiles, int n_tiles,
                           int n_heads, int n_kv_heads, int head_dim, int page_size, int window,
                           float scale, void* stream);
+int axk_attention_decode_chunk(void);
 long axk_attention_decode_workspace(int n_tokens, int n_heads, int head_dim, int max_chunks);
 int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                          const int32_t* block_table, int table_stride, const int32_t* positions,

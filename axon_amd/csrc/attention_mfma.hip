@@ -18,6 +18,8 @@
 #include "api.h"
 #include "common.h"
 
+#define DC_CHUNK 256   // positions of one chunk of a decoding token's range
+
 #if AXON_BF16
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -320,16 +322,18 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
 }
 
 // ============================================================================ decoding tokens
-// grid (tokens, kv heads, chunks): one wave per (token, kv head, chunk of 64 positions = one
-// block of the fold).  The wave issues every load of its chunk at once (K rows and V^T rows go
-// straight from the pages into 16x16x32 MFMA operands, 32 KB in flight per wave), then
-// multiplies; the query heads of the group are the 16 columns (a group of up to 16 heads).
-// Output: if the token's whole range is one chunk, the normalised result; else the chunk's
-// (max, sum, unnormalised output) into `partial`, folded by attention_combine_kernel.
-#define DC_CHUNK 64
+// grid (tokens, kv heads, chunks): a block of four waves per (token, kv head, chunk of 256
+// positions); a wave takes 64 of them.  The wave issues every load of its positions at once (K
+// rows and V^T rows go straight from the pages into 16x16x32 MFMA operands, 32 KB in flight per
+// wave), then multiplies; the query heads of the group are the 16 columns (a group of up to 16
+// heads).  The four waves' results are folded in LDS, in wave order.  Output: if the token's
+// whole range is one chunk, the normalised result; else the chunk's (max, sum, unnormalised
+// output) into `partial`, folded by attention_combine_kernel.  How a token's range is cut
+// depends on its own position and the window alone, never on the rest of the batch.
+#define DC_WAVE 64
 
 template <int HD>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
                         const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
@@ -337,53 +341,54 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
                         int max_chunks, int n_heads, int n_kv_heads, int page_size, int window, float scale) {
   constexpr int KS = HD / 32;   // k steps of S^T (32 dims each)
   constexpr int DT = HD / 16;   // output tiles (16 dims each)
-  const int lane = threadIdx.x;
-  const int t = token_index[blockIdx.x];
-  const int kvh = blockIdx.y, chunk = blockIdx.z;
+  constexpr int ROW = HD + 4;   // floats of a head's row in LDS (padded: rows start in different banks)
+  __shared__ float fold_o[4][16][ROW];
+  __shared__ float fold_ml[4][16][2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int t = token_index[blockIdx.z];
+  const int kvh = blockIdx.y, chunk = blockIdx.x;
   const int group = n_heads / n_kv_heads;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
   const int first = (lo / DC_CHUNK) * DC_CHUNK;
   const int n_chunks = (pos - first) / DC_CHUNK + 1;
-  if (chunk >= n_chunks) return;
-  const int p0 = first + chunk * DC_CHUNK;
-  const int c1 = min(p0 + DC_CHUNK - 1, pos);        // last position of this chunk
-  const int32_t* table_row = block_table + (size_t)seq_rows[t] * table_stride;
+  if (chunk >= n_chunks) return;                     // the whole block: no wave of it waits below
+  const int p0 = first + chunk * DC_CHUNK + wave * DC_WAVE;
+  const int c1 = min(p0 + DC_WAVE - 1, pos);         // last position of this wave
   const int r16 = lane & 15, q4 = lane >> 4;
+  // a wave with no position at all (past the token, or wholly before the window): nothing to add
+  const bool wave_live = p0 <= pos && c1 >= lo;
+  if (wave_live) {
+  const int32_t* table_row = block_table + (size_t)seq_rows[t] * table_stride;
   const size_t kv_head_stride = (size_t)HD * page_size;
 
-  // ---- every load first.  K (A operand of S^T): 4 tiles of 16 positions; row = position
-  // p0 + 16 pt + r16, 8 consecutive dims from 32 ks + 8 q4.  Rows past the chunk's end: any valid
-  // row (masked below).
+  // ---- every load first.  K (A operand of S^T): 4 tiles of 16 positions.  Row r of tile pt is
+  // position p0 + 32 (pt / 2) + 8 (r / 4) + 4 (pt % 2) + r % 4, so that what S^T leaves in a
+  // lane's registers (rows 4 q4 .. 4 q4 + 3 of every tile) are, over a pair of tiles, 8
+  // consecutive positions: the V^T operand below is then one 16-byte read.  8 consecutive dims
+  // from 32 ks + 8 q4.  Rows past the chunk's end: any valid row (masked below).
   uint4 kf[4][KS];
 #pragma unroll
   for (int pt = 0; pt < 4; ++pt) {
-    const int p = min(p0 + pt * 16 + r16, c1);
+    const int p = min(p0 + 32 * (pt >> 1) + 8 * (r16 >> 2) + 4 * (pt & 1) + (r16 & 3), c1);
     const bf16_t* krow = k_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * kv_head_stride +
                          (size_t)(p % page_size) * HD + q4 * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) kf[pt][ks] = *reinterpret_cast<const uint4*>(krow + ks * 32);
   }
-  // V^T (A operand of O^T): k step u takes the lane's positions p0 + 32u + 4 q4 + {0..3} and the
-  // same + 16 (what S^T leaves in its registers): two 8-byte reads per output tile.
-  uint2 vf[2][DT][2];
-  int keep[2][2];
+  // V^T (A operand of O^T): k step u takes the lane's positions p0 + 32 u + 8 q4 + {0..7} of dim
+  // 16 dt + r16: 16 bytes of one page (a page holds a multiple of 8 positions).
+  uint4 vf[2][DT];
+  int keep[2];
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
-    const int pa = p0 + 32 * u + 4 * q4, pb = pa + 16;
-    keep[u][0] = max(0, min(c1 - pa + 1, 4));
-    keep[u][1] = max(0, min(c1 - pb + 1, 4));
-    const int pa_c = min(pa, c1), pb_c = min(pb, c1);
+    const int pa = p0 + 32 * u + 8 * q4;
+    keep[u] = max(0, min(c1 - pa + 1, 8));
+    const int pa_c = min(pa, c1);
     const bf16_t* va = v_cache + ((size_t)table_row[pa_c / page_size] * n_kv_heads + kvh) * kv_head_stride +
-                       ((pa_c % page_size) & ~3);
-    const bf16_t* vb = v_cache + ((size_t)table_row[pb_c / page_size] * n_kv_heads + kvh) * kv_head_stride +
-                       ((pb_c % page_size) & ~3);
+                       ((pa_c % page_size) & ~7);
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const size_t doff = (size_t)(dt * 16 + r16) * page_size;
-      vf[u][dt][0] = *reinterpret_cast<const uint2*>(va + doff);
-      vf[u][dt][1] = *reinterpret_cast<const uint2*>(vb + doff);
-    }
+    for (int dt = 0; dt < DT; ++dt) vf[u][dt] = *reinterpret_cast<const uint4*>(va + (size_t)(dt * 16 + r16) * page_size);
   }
   // Q^T (B operand): column = head of the group (zero beyond it), 8 consecutive dims
   bf16x8 qf[KS];
@@ -406,14 +411,14 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
     for (int ks = 0; ks < KS; ++ks)
       s_acc[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag_of(kf[pt][ks]), qf[ks], s_acc[pt], 0, 0, 0);
   }
-  // this lane: head r16; positions p0 + 16 pt + 4 q4 + e
+  // this lane: head r16; positions p0 + 32 (pt / 2) + 8 q4 + 4 (pt % 2) + e
   const float c = scale * LOG2E;
   float m = -INFINITY;
 #pragma unroll
   for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int p = p0 + pt * 16 + q4 * 4 + e;
+      const int p = p0 + 32 * (pt >> 1) + 8 * q4 + 4 * (pt & 1) + e;
       const float v = (p <= c1 && p >= lo) ? s_acc[pt][e] * c : -INFINITY;
       s_acc[pt][e] = v;
       m = fmaxf(m, v);
@@ -446,41 +451,69 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
     pf.w[3] = pack_bf16(s_acc[2 * u + 1][2], s_acc[2 * u + 1][3]);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      uint2 v0 = vf[u][dt][0], v1 = vf[u][dt][1];
-      if (keep[u][0] < 4) {
-        if (keep[u][0] < 1) v0.x = 0; else if (keep[u][0] < 2) v0.x &= 0xffffu;
-        if (keep[u][0] < 3) v0.y = 0; else v0.y &= 0xffffu;
-      }
-      if (keep[u][1] < 4) {
-        if (keep[u][1] < 1) v1.x = 0; else if (keep[u][1] < 2) v1.x &= 0xffffu;
-        if (keep[u][1] < 3) v1.y = 0; else v1.y &= 0xffffu;
+      uint4 v = vf[u][dt];
+      if (keep[u] < 8) {
+        uint32_t* w = reinterpret_cast<uint32_t*>(&v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (keep[u] <= 2 * i) w[i] = 0;
+          else if (keep[u] == 2 * i + 1) w[i] &= 0xffffu;
+        }
       }
       if (u == 0) o_acc[dt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag_of2(v0, v1), pf.f, o_acc[dt], 0, 0, 0);
+      o_acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag_of(v), pf.f, o_acc[dt], 0, 0, 0);
     }
   }
 
-  if (r16 >= group) return;
-  const int head = kvh * group + r16;
-  if (n_chunks == 1) {
-    const float inv = 1.0f / l;
-    bf16_t* orow = out + (size_t)t * n_heads * HD + (size_t)head * HD;
+  if (r16 < group) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      uint2 pk;
-      pk.x = pack_bf16(o_acc[dt][0] * inv, o_acc[dt][1] * inv);
-      pk.y = pack_bf16(o_acc[dt][2] * inv, o_acc[dt][3] * inv);
-      *reinterpret_cast<uint2*>(orow + dt * 16 + q4 * 4) = pk;
-    }
-  } else {
-    // partial [token slot][head][chunk][HD + 2]: output, then max (log2 domain) and sum
-    float* dst = partial + (((size_t)blockIdx.x * n_heads + head) * max_chunks + chunk) * (HD + 2);
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      *reinterpret_cast<f32x4*>(dst + dt * 16 + q4 * 4) = o_acc[dt];
+    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(&fold_o[wave][r16][dt * 16 + q4 * 4]) = o_acc[dt];
     if (q4 == 0) {
-      dst[HD] = m;
-      dst[HD + 1] = l;
+      fold_ml[wave][r16][0] = m;
+      fold_ml[wave][r16][1] = l;
+    }
+  }
+  } else if (lane < 16) {
+    fold_ml[wave][lane][0] = -INFINITY;
+    fold_ml[wave][lane][1] = 0.0f;
+  }
+  __syncthreads();
+
+  // ---- the four waves' results into one, in wave order: a thread takes 4 dims of a head
+  for (int task = threadIdx.x; task < group * (HD / 4); task += 256) {
+    const int hg = task / (HD / 4), d = (task % (HD / 4)) * 4;
+    float M = fold_ml[0][hg][0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) M = fmaxf(M, fold_ml[w][hg][0]);
+    const float mref = M == -INFINITY ? 0.0f : M;
+    float L = 0.0f;
+    f32x4 O = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = fold_ml[w][hg][0];
+      if (mw == -INFINITY) continue;                 // a wave without positions wrote no output
+      const float weight = __builtin_amdgcn_exp2f(mw - mref);
+      L = fmaf(fold_ml[w][hg][1], weight, L);
+      const f32x4 o = *reinterpret_cast<const f32x4*>(&fold_o[w][hg][d]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) O[e] = fmaf(o[e], weight, O[e]);
+    }
+    const int head = kvh * group + hg;
+    if (n_chunks == 1) {
+      const float inv = 1.0f / L;
+      uint2 pk;
+      pk.x = pack_bf16(O[0] * inv, O[1] * inv);
+      pk.y = pack_bf16(O[2] * inv, O[3] * inv);
+      *reinterpret_cast<uint2*>(out + (size_t)t * n_heads * HD + (size_t)head * HD + d) = pk;
+    } else {
+      // partial [token slot][head][chunk][HD + 2]: output, then max (log2 domain) and sum
+      float* dst = partial + (((size_t)blockIdx.z * n_heads + head) * max_chunks + chunk) * (HD + 2);
+      *reinterpret_cast<float2*>(dst + d) = make_float2(O[0], O[1]);
+      *reinterpret_cast<float2*>(dst + d + 2) = make_float2(O[2], O[3]);
+      if (d == 0) {
+        dst[HD] = M;
+        dst[HD + 1] = L;
+      }
     }
   }
 }
@@ -593,6 +626,9 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
 #endif
 }
 
+// Positions of one chunk of a decoding token's range.
+extern "C" int axk_attention_decode_chunk(void) { return DC_CHUNK; }
+
 // Floats of `partial` that n_tokens decoding tokens with up to max_chunks chunks need.
 extern "C" long axk_attention_decode_workspace(int n_tokens, int n_heads, int head_dim, int max_chunks) {
   return (long)n_tokens * n_heads * max_chunks * (head_dim + 2);
@@ -607,18 +643,18 @@ extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_c
   AXK_REQUIRE(axk_attention_fast_ok(head_dim, page_size, n_heads, n_kv_heads),
               "attention_decode: head_dim %d, page size %d, %d/%d heads are not taken by this kernel", head_dim,
               page_size, n_heads, n_kv_heads);
-  AXK_REQUIRE(max_chunks <= CMB_MAX_CHUNKS, "attention_decode: %d chunks of 64 positions (at most %d: %d positions)",
-              max_chunks, CMB_MAX_CHUNKS, CMB_MAX_CHUNKS * 64);
+  AXK_REQUIRE(max_chunks <= CMB_MAX_CHUNKS, "attention_decode: %d chunks of %d positions (at most %d: %d positions)",
+              max_chunks, DC_CHUNK, CMB_MAX_CHUNKS, CMB_MAX_CHUNKS * DC_CHUNK);
   AXK_REQUIRE(n_tokens >= 0 && max_chunks >= 1 && max_chunks <= 65535 && n_kv_heads <= 65535 && window >= 0 &&
                   q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0,
               "attention_decode: bad arguments (tokens %d, chunks %d, window %d, q stride %d)", n_tokens, max_chunks,
               window, q_stride);
   AXK_REQUIRE(max_chunks == 1 || partial != nullptr, "attention_decode: %d chunks need a workspace", max_chunks);
   if (n_tokens == 0) return 0;
-  dim3 grid(n_tokens, n_kv_heads, max_chunks), cgrid(n_tokens, n_heads);
+  dim3 grid(max_chunks, n_kv_heads, n_tokens), cgrid(n_tokens, n_heads);
 #define LAUNCH(HD)                                                                                                   \
   {                                                                                                                  \
-    attention_decode_kernel<HD><<<grid, 64, 0, (hipStream_t)stream>>>(                                               \
+    attention_decode_kernel<HD><<<grid, 256, 0, (hipStream_t)stream>>>(                                               \
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,       \
         positions, seq_rows, (bf16_t*)out, token_index, partial, max_chunks, n_heads, n_kv_heads, page_size, window, \
         scale);                                                                                                      \

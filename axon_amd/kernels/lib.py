@@ -278,6 +278,12 @@ class Kernels:
             float(scale), _stream()))
         return out
 
+    @property
+    def attention_decode_chunk(self) -> int:
+        """Positions of one chunk of the decoding kernel: a token's range (from the chunk that
+        holds the window's first position, or 0) is cut into chunks of this size."""
+        return int(self.lib.axk_attention_decode_chunk())
+
     def attention_decode_workspace(self, n_tokens: int, n_heads: int, head_dim: int, max_chunks: int) -> int:
         return int(self.lib.axk_attention_decode_workspace(n_tokens, n_heads, head_dim, max_chunks))
 

@@ -25,8 +25,6 @@ from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, UnscaledRows, buil
 
 
 PREFILL_TILE = 128     # tokens of one request per tile of the prompt kernel
-DECODE_CHUNK = 64      # positions per chunk of the decoding kernel
-DECODE_BLOCK = 64
 
 
 class AttentionPlan:
@@ -49,7 +47,7 @@ class AttentionPlan:
             for s in ctx.spans:
                 if s.q_len == 1:
                     singles.append(s.q_start)
-                    chunks = max(chunks, decode_chunks_of(s.start_pos, window))
+                    chunks = max(chunks, decode_chunks_of(s.start_pos, window, ctx.rt.k.attention_decode_chunk))
                 else:
                     for at in range(0, s.q_len, PREFILL_TILE):
                         tiles.append((s.q_start + at, min(PREFILL_TILE, s.q_len - at)))
@@ -66,10 +64,10 @@ class AttentionPlan:
             self.partial = torch.empty(n, dtype=torch.float32, device=dev)
 
 
-def decode_chunks_of(pos: int, window: int) -> int:
-    """Chunks of 64 positions the decoding kernel cuts a token's range into."""
+def decode_chunks_of(pos: int, window: int, chunk: int) -> int:
+    """Chunks (of `chunk` positions, the kernel's constant) the decoding kernel cuts a token's range into."""
     lo = max(0, pos + 1 - window) if window > 0 else 0
-    return (pos - lo // DECODE_BLOCK * DECODE_BLOCK) // DECODE_CHUNK + 1
+    return (pos - lo // chunk * chunk) // chunk + 1
 
 
 def attention_plan(ctx, window: int, n_heads: int, head_dim: int) -> AttentionPlan:
@@ -103,6 +101,7 @@ class GQAttention(Mixer):
         base = prefix + names.get("scope", "self_attn.")
         self.n = {k: base + names.get(k, k + "_proj") for k in ("q", "k", "v", "o")}
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+        self.decode_chunk = 1 << 30          # until `load` has asked the kernels: one chunk
 
     # ------------------------------------------------------------------ declarations
     def tensors(self) -> List[TensorDecl]:
@@ -123,12 +122,15 @@ class GQAttention(Mixer):
         return CacheSpec(entries=2, heads=self.nkv, head_dim=self.hd, window=self.window)
 
     def decode_shape(self, positions):
-        """The decoding kernel's grid depends on the longest context, in chunks of 64 positions,
-        rounded up to a power of two so that few shapes exist."""
-        most = max(decode_chunks_of(p, self.window) for p in positions)
-        return ("attention_chunks", self.window), 1 << (most - 1).bit_length()
+        """The decoding kernel's grid depends on the longest context, in chunks of the kernel's
+        size, rounded up in steps of an eighth or less so that few shapes exist and few blocks of
+        the grid find nothing to do (they cost their launch all the same)."""
+        most = max(decode_chunks_of(p, self.window, self.decode_chunk) for p in positions)
+        step = 1 << max(0, most.bit_length() - 4)
+        return ("attention_chunks", self.window), -(-most // step) * step
 
     def load(self, store, rt) -> None:
+        self.decode_chunk = rt.k.attention_decode_chunk
         self.w_qkv = rt.k.prepare_weight(store.fused_matrix([self.n[k] + ".weight" for k in ("q", "k", "v")]))
         biases = [store.vector(self.n[k] + ".bias", optional=True) for k in ("q", "k", "v")] if self.qkv_bias else []
         present = [b is not None for b in biases]

@@ -436,7 +436,7 @@ def test_prompt_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
 
 @pytest.mark.parametrize("nh,nkv,hd,page,T,window", [
     (4, 2, 64, 16, 300, 0), (7, 1, 128, 16, 1030, 0), (28, 4, 128, 16, 600, 0), (6, 2, 128, 8, 255, 0),
-    (2, 2, 64, 64, 257, 0), (16, 1, 64, 32, 513, 0), (4, 1, 64, 16, 900, 300), (5, 5, 128, 16, 64, 0)])
+    (2, 2, 64, 64, 257, 0), (16, 1, 64, 32, 513, 0), (4, 1, 64, 16, 900, 300), (5, 5, 128, 16, 64, 0), (3, 1, 128, 16, 700, 70)])
 def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
     k = kernels("bfloat16")
     q, kc, vc, table, ref = _mfma_case(nh, nkv, hd, page, T, window, seed=5)
@@ -446,7 +446,8 @@ def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
     # single tokens at chosen positions: first, block and chunk edges, last
     picks = sorted({0, 1, 15, 16, 63, 64, 65, 255, 256, 257, 511, 512, T // 2, T - 2, T - 1} & set(range(T)))
     idx = torch.tensor(picks, dtype=torch.int32).cuda()
-    chunks = max((p - ((max(0, p + 1 - window) if window else 0) // 64 * 64)) // 64 + 1 for p in picks)
+    ch = k.attention_decode_chunk
+    chunks = max((p - ((max(0, p + 1 - window) if window else 0) // ch * ch)) // ch + 1 for p in picks)
     partial = torch.empty(k.attention_decode_workspace(len(picks), nh, hd, chunks), dtype=torch.float32, device="cuda")
     out = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
     k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, out, idx, partial, chunks, nh, nkv, hd, page, window, scale)
