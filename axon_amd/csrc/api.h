@@ -106,12 +106,23 @@ typedef struct {
   int norm_gain_is_f32;
   void* norm_values;
   float* norm_squares;
+  float norm_eps;      // of the whole norm behind a split product (axk_gemm_then_norm)
 } GemmNormFold;
 int axk_gemm_norm_fold_ok(int m, int n, int k, int mode);
 int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
                        int out_stride, int m, int n, int k, int mode, const float* in_squares, float in_eps,
                        const void* norm_gain, int norm_gain_is_f32, void* norm_values, float* norm_squares,
                        void* stream);
+
+// The product that adds into float32 rows (mode 1, W packed) followed by the RMS norm of the new
+// rows, for shapes that run with K split between blocks (axk_gemm_then_norm_ok says 1): the
+// kernel that adds the blocks' sums also writes norm_values elem [M, N] =
+// out / sqrt(mean(out^2) + norm_eps) * norm_gain.  Bit-identical to axk_gemm followed by
+// axk_rmsnorm.  workspace: axk_gemm_workspace bytes, as for axk_gemm.
+int axk_gemm_then_norm_ok(int m, int n, int k);
+int axk_gemm_then_norm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, float* out,
+                       int out_stride, int m, int n, int k, const void* norm_gain, int norm_gain_is_f32,
+                       float norm_eps, void* norm_values, void* workspace, long workspace_bytes, void* stream);
 
 // The attention's [q; k; v] product (W packed, [(n_heads + 2 n_kv_heads) head_dim, K], or the q rows alone
 // if write_kv is 0) with what follows it as its epilogue: bias, the rotary encoding of q and k

@@ -99,6 +99,18 @@ __device__ inline float wave_sum_to_last(float v) {
   return v;
 }
 
+// The sum over a block of 256 threads: within each wave (butterfly), then the four waves' sums
+// in wave order.  `partial` is 4 floats of LDS; every thread returns the same value.
+__device__ inline float block_sum_256(float v, float* partial) {
+  v = wave_sum(v);
+  if ((threadIdx.x & (AXON_WAVE - 1)) == 0) partial[threadIdx.x / AXON_WAVE] = v;
+  __syncthreads();
+  float total = partial[0];
+#pragma unroll
+  for (int w = 1; w < 256 / AXON_WAVE; ++w) total += partial[w];
+  return total;
+}
+
 __device__ inline float wave_max(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, AXON_WAVE));

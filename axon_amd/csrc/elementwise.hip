@@ -59,16 +59,6 @@ extern "C" int axk_embed(const int32_t* tokens, const void* table, int packed, f
 #define NORM_THREADS 256
 #define NORM_CACHED 4  // float4 a thread keeps in registers: rows up to 4096 wide are read once
 
-__device__ inline float block_sum_256(float v, float* partial) {
-  v = wave_sum(v);
-  if ((threadIdx.x & (AXON_WAVE - 1)) == 0) partial[threadIdx.x / AXON_WAVE] = v;
-  __syncthreads();
-  float total = partial[0];
-#pragma unroll
-  for (int w = 1; w < NORM_THREADS / AXON_WAVE; ++w) total += partial[w];
-  return total;
-}
-
 __device__ inline void store4(elem_t* dst, float a, float b, float c, float d) {
 #if AXON_BF16
   uint2 pk;

@@ -150,6 +150,7 @@ int gemm_pack_ok(int rows, int k, int gated);
 int launch_pack_matrix(const bf16_t* src, bf16_t* dst, int rows, int k, hipStream_t stream);
 size_t gemm_workspace_bytes(int m, int n, int k, int mode);
 int gemm_norm_fold_ok(int m, int n, int k, int mode);
+int gemm_then_norm_ok(int m, int n, int k);
 int gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim);
 int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out,
                          int out_stride, int m, int n, int k, const float* in_squares, float in_eps,
@@ -235,8 +236,31 @@ extern "C" int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, co
   AXK_REQUIRE(norm_gain == nullptr || (mode == MODE_ADD_F32 && norm_values && norm_squares),
               "gemm: the following norm needs the add-into-residual epilogue and both of its outputs");
   AXK_REQUIRE(((uintptr_t)in_squares & 15) == 0, "gemm: the rows' sums of squares must be 16-byte aligned");
-  const GemmNormFold fold = {in_squares, in_eps, norm_gain, norm_gain_is_f32, norm_values, norm_squares};
+  const GemmNormFold fold = {in_squares, in_eps, norm_gain, norm_gain_is_f32, norm_values, norm_squares, 0.0f};
   return gemm_checked(x, x_stride, w, 1, bias, bias_is_f32, out, out_stride, m, n, k, mode, &fold, nullptr, 0, stream);
+}
+
+extern "C" int axk_gemm_then_norm_ok(int m, int n, int k) {
+#if AXON_BF16
+  return m > 0 && n > 0 && k > 0 && gemm_then_norm_ok(m, n, k);
+#else
+  return 0;   // the 32-bit build keeps the norm a pass of its own
+#endif
+}
+
+extern "C" int axk_gemm_then_norm(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32,
+                                  float* out, int out_stride, int m, int n, int k, const void* norm_gain,
+                                  int norm_gain_is_f32, float norm_eps, void* norm_values, void* workspace,
+                                  long workspace_bytes, void* stream) {
+  AXK_REQUIRE(axk_gemm_then_norm_ok(m, n, k), "gemm: M=%d N=%d K=%d does not run with K split: the norm stays apart", m,
+              n, k);
+  AXK_REQUIRE(norm_gain && norm_values, "gemm: the norm behind the product needs its gain and its output");
+  AXK_REQUIRE(out_stride % 4 == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)norm_values & 7) == 0,
+              "gemm: the rows to add into must be 16-byte aligned (stride %d) and the norm's output 8-byte aligned",
+              out_stride);
+  const GemmNormFold fold = {nullptr, 0.0f, norm_gain, norm_gain_is_f32, norm_values, nullptr, norm_eps};
+  return gemm_checked(x, x_stride, w, 1, bias, bias_is_f32, out, out_stride, m, n, k, MODE_ADD_F32, &fold, workspace,
+                      workspace_bytes, stream);
 }
 
 extern "C" int axk_gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim) {

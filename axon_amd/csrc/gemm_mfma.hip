@@ -300,16 +300,28 @@ gemm_split_reduce_kernel(const float* __restrict__ partial, int splits, int M, i
   const int m = idx / n4, n = (idx % n4) * 4;
   const size_t plane = (size_t)M * N, at_in = (size_t)m * N + n;
   const int parts = mode == MODE_SWIGLU ? 2 : 1;
-  float4 g = *reinterpret_cast<const float4*>(partial + at_in), u = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-  if (parts == 2) u = *reinterpret_cast<const float4*>(partial + plane + at_in);
-  for (int z = 1; z < splits; ++z) {
-    const float4 a = *reinterpret_cast<const float4*>(partial + (size_t)z * parts * plane + at_in);
-    g.x += a.x; g.y += a.y; g.z += a.z; g.w += a.w;
-    if (parts == 2) {
-      const float4 b = *reinterpret_cast<const float4*>(partial + ((size_t)z * parts + 1) * plane + at_in);
-      u.x += b.x; u.y += b.y; u.z += b.z; u.w += b.w;
+  // the blocks' sums in block order; four loads under way at a time
+  auto summed = [&](const float* src, size_t step) {
+    float4 g = *reinterpret_cast<const float4*>(src);
+    int z = 1;
+    for (; z + 3 < splits; z += 4) {
+      const float4 a0 = *reinterpret_cast<const float4*>(src + (size_t)z * step);
+      const float4 a1 = *reinterpret_cast<const float4*>(src + (size_t)(z + 1) * step);
+      const float4 a2 = *reinterpret_cast<const float4*>(src + (size_t)(z + 2) * step);
+      const float4 a3 = *reinterpret_cast<const float4*>(src + (size_t)(z + 3) * step);
+      g.x += a0.x; g.y += a0.y; g.z += a0.z; g.w += a0.w;
+      g.x += a1.x; g.y += a1.y; g.z += a1.z; g.w += a1.w;
+      g.x += a2.x; g.y += a2.y; g.z += a2.z; g.w += a2.w;
+      g.x += a3.x; g.y += a3.y; g.z += a3.z; g.w += a3.w;
     }
-  }
+    for (; z < splits; ++z) {
+      const float4 a = *reinterpret_cast<const float4*>(src + (size_t)z * step);
+      g.x += a.x; g.y += a.y; g.z += a.z; g.w += a.w;
+    }
+    return g;
+  };
+  const float4 g = summed(partial + at_in, (size_t)parts * plane);
+  const float4 u = parts == 2 ? summed(partial + plane + at_in, (size_t)parts * plane) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
   float v[4] = {g.x, g.y, g.z, g.w};
   const size_t at = (size_t)m * out_stride + n;
   if (mode == MODE_SWIGLU) {
@@ -327,10 +339,109 @@ gemm_split_reduce_kernel(const float* __restrict__ partial, int splits, int M, i
   }
 }
 
+// An RMS norm of the rows right after a split product that adds into them (the residual
+// stream): the split-K sums, the bias and the addition as in gemm_split_reduce_kernel, then the
+// norm of the new row, values = out * (1 / sqrt(mean(out^2) + eps)) * gain, in the same launch.
+// A block of 1024 threads per row, a thread per 4 columns (and 4 more in a row wider than 4096):
+// every load of the sums is independent of the others.  The new row goes through LDS to the
+// first 256 threads, which add up its squares in the order of the norm's own kernel (thread t:
+// the float4 t, t + 256, ...; then the lanes of a wave; then the four waves), so both ways give
+// the same bits.
+struct SplitNorm {
+  const void* gain;
+  int gain_is_f32;
+  float eps;
+  bf16_t* values;      // [M, N]
+};
+
+#define SRN_THREADS 1024
+#define SRN_MAX_N 8192
+
+__global__ void __launch_bounds__(SRN_THREADS)
+gemm_split_reduce_norm_kernel(const float* __restrict__ partial, int splits, int M, int N, const void* __restrict__ bias,
+                              int bias_is_f32, float* __restrict__ out, int out_stride, SplitNorm norm) {
+  __shared__ float4 row[SRN_MAX_N / 4];
+  __shared__ float sums[4];
+  const int m = blockIdx.x, n4 = N / 4, tid = threadIdx.x;
+  const size_t plane = (size_t)M * N;
+  auto added = [&](int i) {
+    const int n = i * 4;
+    const float* src = partial + (size_t)m * N + n;
+    float4 g = *reinterpret_cast<const float4*>(src);
+    int z = 1;
+    for (; z + 3 < splits; z += 4) {           // four loads under way at a time; added in block order
+      const float4 a0 = *reinterpret_cast<const float4*>(src + (size_t)z * plane);
+      const float4 a1 = *reinterpret_cast<const float4*>(src + (size_t)(z + 1) * plane);
+      const float4 a2 = *reinterpret_cast<const float4*>(src + (size_t)(z + 2) * plane);
+      const float4 a3 = *reinterpret_cast<const float4*>(src + (size_t)(z + 3) * plane);
+      g.x += a0.x; g.y += a0.y; g.z += a0.z; g.w += a0.w;
+      g.x += a1.x; g.y += a1.y; g.z += a1.z; g.w += a1.w;
+      g.x += a2.x; g.y += a2.y; g.z += a2.z; g.w += a2.w;
+      g.x += a3.x; g.y += a3.y; g.z += a3.z; g.w += a3.w;
+    }
+    for (; z < splits; ++z) {
+      const float4 a = *reinterpret_cast<const float4*>(src + (size_t)z * plane);
+      g.x += a.x; g.y += a.y; g.z += a.z; g.w += a.w;
+    }
+    if (bias) {
+      g.x += load_vec(bias, bias_is_f32, n);
+      g.y += load_vec(bias, bias_is_f32, n + 1);
+      g.z += load_vec(bias, bias_is_f32, n + 2);
+      g.w += load_vec(bias, bias_is_f32, n + 3);
+    }
+    float4* dst = reinterpret_cast<float4*>(out + (size_t)m * out_stride + n);
+    float4 r = *dst;
+    r.x += g.x; r.y += g.y; r.z += g.z; r.w += g.w;
+    *dst = r;
+    return r;
+  };
+  constexpr int MINE = SRN_MAX_N / 4 / SRN_THREADS;
+  float4 mine[MINE];
+#pragma unroll
+  for (int c = 0; c < MINE; ++c) {
+    const int i = tid + c * SRN_THREADS;
+    if (i < n4) {
+      mine[c] = added(i);
+      row[i] = mine[c];
+    }
+  }
+  __syncthreads();
+  if (tid < 256) {
+    float ss = 0.0f;
+    for (int i = tid; i < n4; i += 256) {
+      const float4 v = row[i];
+      ss = fmaf(v.x, v.x, ss);
+      ss = fmaf(v.y, v.y, ss);
+      ss = fmaf(v.z, v.z, ss);
+      ss = fmaf(v.w, v.w, ss);
+    }
+    ss = wave_sum(ss);
+    if ((tid & (AXON_WAVE - 1)) == 0) sums[tid / AXON_WAVE] = ss;
+  }
+  __syncthreads();
+  const float total = ((sums[0] + sums[1]) + sums[2]) + sums[3];
+  const float inv = 1.0f / sqrtf(total / (float)N + norm.eps);
+  bf16_t* dst = norm.values + (size_t)m * N;
+#pragma unroll
+  for (int c = 0; c < MINE; ++c) {
+    const int i = tid + c * SRN_THREADS;
+    if (i < n4) {
+      const int e = i * 4;
+      const float4 v = mine[c];
+      uint2 pk;
+      pk.x = pack2_bf16((v.x * inv) * load_vec(norm.gain, norm.gain_is_f32, e),
+                        (v.y * inv) * load_vec(norm.gain, norm.gain_is_f32, e + 1));
+      pk.y = pack2_bf16((v.z * inv) * load_vec(norm.gain, norm.gain_is_f32, e + 2),
+                        (v.w * inv) * load_vec(norm.gain, norm.gain_is_f32, e + 3));
+      *reinterpret_cast<uint2*>(dst + e) = pk;
+    }
+  }
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK = 64, int STAGES = 2>
 static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                        int out_stride, int m, int n, int k, int mode, hipStream_t stream, int splits = 1,
-                       float* partial = nullptr) {
+                       float* partial = nullptr, const SplitNorm* norm = nullptr) {
   static bool configured = false;
   constexpr int lds_bytes = STAGES * (BM + BN) * BK * 2;
   static_assert(lds_bytes <= 160 * 1024, "the stages do not fit the LDS of a CU");
@@ -348,7 +459,11 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
   kernel<<<dim3(m_blocks * n_blocks, splits), WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks, splits > 1 ? partial : nullptr);
   AXK_LAUNCH_CHECK("gemm_tile");
-  if (splits > 1) {
+  if (splits > 1 && norm != nullptr) {
+    gemm_split_reduce_norm_kernel<<<m, SRN_THREADS, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, (float*)out, out_stride,
+                                                         *norm);
+    AXK_LAUNCH_CHECK("gemm_split_reduce_norm");
+  } else if (splits > 1) {
     gemm_split_reduce_kernel<<<ceil_div(m * (n / 4), 256), 256, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, out,
                                                                             out_stride, mode);
     AXK_LAUNCH_CHECK("gemm_split_reduce");
@@ -764,6 +879,14 @@ int gemm_norm_fold_ok(int m, int n, int k, int mode) {
   return gemm_pack_ok(mode == MODE_SWIGLU ? 2 * n : n, k, mode == MODE_SWIGLU) && skinny_takes(m, n, k, mode);
 }
 
+// Whether the product that adds into the rows runs with K split between blocks, so that the
+// kernel that adds the blocks' sums can also norm the finished rows (gemm_split_reduce_norm_kernel:
+// rows of up to SRN_MAX_N columns).
+int gemm_then_norm_ok(int m, int n, int k) {
+  return gemm_pack_ok(n, k, 0) && !skinny_takes(m, n, k, MODE_ADD_F32) && splits_of(m, n, k, MODE_ADD_F32) > 1 &&
+         n <= SRN_MAX_N;
+}
+
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                      int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold_in,
                      void* workspace, size_t workspace_bytes) {
@@ -792,9 +915,17 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
     // split K; the ring is as deep as the registers allow
     return n >= 32 * 128 ? launch_skinny<2, 1, 4, 8>(ARGS, fold) : launch_skinny<1, 1, 4, 8>(ARGS, fold);
   }
+  // the tiled kernels: no norm on the way in; on the way out only a whole norm behind split sums
+  SplitNorm after = {nullptr, 0, 0.0f, nullptr};
+  const SplitNorm* norm = nullptr;
   if (fold_in) {
-    axk_set_error("gemm: M=%d N=%d goes to the tiled kernel, which folds no norm", m, n);
-    return -1;
+    const bool whole = fold_in->in_squares == nullptr && fold_in->norm_gain && fold_in->norm_values && !fold_in->norm_squares;
+    if (!whole || mode != MODE_ADD_F32 || !gemm_then_norm_ok(m, n, k)) {
+      axk_set_error("gemm: M=%d N=%d K=%d mode %d goes to the tiled kernel, which folds no such norm", m, n, k, mode);
+      return -1;
+    }
+    after = SplitNorm{fold_in->norm_gain, fold_in->norm_gain_is_f32, fold_in->norm_eps, (bf16_t*)fold_in->norm_values};
+    norm = &after;
   }
   const int splits = splits_of(m, n, k, mode);
   const size_t need = gemm_workspace_bytes(m, n, k, mode);
@@ -807,11 +938,11 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
   if (m <= 256) {
     if (m > 64) {
       if (mode == MODE_SWIGLU) return launch_tile<128, 128, 2, 2, true>(ARGS, splits, ws);
-      return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws);
+      return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws, norm);
     }
     if (mode == MODE_SWIGLU) return launch_tile<64, 256, 1, 4, true, 64, 2>(ARGS, splits, ws);
-    if (n >= 8192) return launch_tile<64, 256, 1, 4, false, 64, 2>(ARGS, splits, ws);
-    return launch_tile<64, 128, 1, 4, false, 64, 3>(ARGS, splits, ws);
+    if (n >= 8192) return launch_tile<64, 256, 1, 4, false, 64, 2>(ARGS, splits, ws, norm);
+    return launch_tile<64, 128, 1, 4, false, 64, 3>(ARGS, splits, ws, norm);
   }
   // 256 x 256 tiles (8 waves) where they fill the chip: one round of at least 140 blocks (on 256
   // CUs), or several rounds of which the last is not mostly idle; else 128 x 128 tiles, four times
@@ -824,8 +955,8 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
     if (use_big) return launch_tile<256, 256, 4, 2, true>(ARGS, splits, ws);
     return launch_tile<128, 128, 2, 2, true>(ARGS, splits, ws);
   }
-  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS, splits, ws);
-  return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws);
+  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS, splits, ws, norm);
+  return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws, norm);
 #undef ARGS
 }
 

@@ -54,6 +54,9 @@ _SIGNATURES = {
     "axk_gemm_norm_fold_ok": [c_int, c_int, c_int, c_int],
     "axk_gemm_norm_fold": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                            c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+    "axk_gemm_then_norm_ok": [c_int, c_int, c_int],
+    "axk_gemm_then_norm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int,
+                           c_float, c_void_p, c_void_p, ctypes.c_long, c_void_p],
     "axk_swiglu": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_argmax": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p],
     "axk_topk": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -328,6 +331,11 @@ class Kernels:
             return self.pack_matrix(w.contiguous())
         return w
 
+    def gemm_then_norm_ok(self, m: int, n: int, k: int) -> bool:
+        """Whether the product that adds into [m, n] float32 rows can also write the RMS norm of
+        the new rows (see `gemm`: a `following_norm` without squares)."""
+        return bool(self.lib.axk_gemm_then_norm_ok(m, n, k))
+
     def gemm_norm_fold_ok(self, m: int, n: int, k: int, mode: int) -> bool:
         """Whether the product of these sizes can take an RMS norm into itself (see `gemm`)."""
         return bool(self.lib.axk_gemm_norm_fold_ok(m, n, k, mode))
@@ -342,8 +350,10 @@ class Kernels:
         An RMS norm folded in (where `gemm_norm_fold_ok`): with `row_squares` float32 [M, K / 16],
         x holds rows times their gain that still lack the scale 1/sqrt(sum(row_squares) / K + eps),
         which the product applies to its result.  `following_norm` = (gain, values [M, N],
-        squares [M, ceil(N / 16)]) with MODE_ADD_F32: the epilogue also writes out * gain and the
-        sums of out^2 over parts of 16 columns, for the next product's `row_squares` side."""
+        squares [M, ceil(N / 16)], eps) with MODE_ADD_F32: the epilogue also writes out * gain and
+        the sums of out^2 over parts of 16 columns, for the next product's `row_squares` side.
+        With squares None (where `gemm_then_norm_ok`): values = the whole norm of the new rows,
+        out / sqrt(mean(out^2) + eps) * gain."""
         packed = isinstance(w, PackedMatrix)
         self._elem(x, "gemm x"); self._elem(w.data if packed else w, "gemm w")
         M, K = x.shape
@@ -376,8 +386,21 @@ class Kernels:
                               f"[{M}, {K // 16}]")
         gain = values = squares = None
         if following_norm is not None:
-            gain, values, squares = following_norm
+            gain, values, squares, norm_eps = following_norm
             self._elem(values, "gemm norm values")
+            if squares is None:
+                if row_squares is not None or mode != MODE_ADD_F32:
+                    raise KernelError("gemm: a whole norm follows only the product that adds into float32 rows")
+                if gain.numel() != N or values.shape != (M, N) or not values.is_contiguous():
+                    raise KernelError(f"gemm: the following norm's gain {tuple(gain.shape)} or values "
+                                      f"{tuple(values.shape)} do not fit [{M}, {N}]")
+                need = self.lib.axk_gemm_workspace(M, N, K, mode)
+                work = torch.empty(need // 4, dtype=torch.float32, device=x.device) if need > 0 else None
+                self._check(self.lib.axk_gemm_then_norm(
+                    _ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"), _ptr(out), out.stride(0),
+                    M, N, K, _ptr(gain), self._vec_flag(gain, "gemm norm gain"), float(norm_eps), _ptr(values), _ptr(work),
+                    need, _stream()))
+                return out
             if (gain.numel() != N or values.shape != (M, N) or not values.is_contiguous()
                     or squares.shape != (M, -(-N // 16)) or squares.dtype != torch.float32 or not squares.is_contiguous()
                     or not squares.is_cuda):

@@ -114,8 +114,12 @@ class DecoderModel:
         for i, (run, binding) in enumerate(zip(self.order, self.cache_plan.bindings)):
             block = self.blocks[run.layer]
             fold = None
-            if i + 1 < len(self.order) and block.folds_following_norm(ctx):
-                fold = self.blocks[self.order[i + 1].layer].first_norm_fold(ctx, x.shape[0])
+            if i + 1 < len(self.order):
+                after = self.blocks[self.order[i + 1].layer]
+                if block.finishes_following_norm(ctx):
+                    fold = after.first_norm_fold(ctx, x.shape[0], whole=True)
+                elif block.folds_following_norm(ctx):
+                    fold = after.first_norm_fold(ctx, x.shape[0])
             if unscaled is None and fold is None:
                 block.forward(ctx, binding, x)
             else:

@@ -156,6 +156,9 @@ class GQAttention(Mixer):
         return (isinstance(self.w_o, PackedMatrix)
                 and ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.hidden, self.q_dim, MODE_ADD_F32))
 
+    def finishes_following_norm(self, ctx) -> bool:
+        return isinstance(self.w_o, PackedMatrix) and ctx.rt.k.gemm_then_norm_ok(ctx.n_tokens, self.hidden, self.q_dim)
+
     def forward(self, ctx, binding: CacheBinding, h, residual, fold=None) -> None:
         k = ctx.rt.k
         T = h.shape[0]

@@ -105,26 +105,28 @@ class UnscaledRows:
 
 class NormFold:
     """A norm handed to the part that runs before it: that part's last product, which adds into
-    the residual stream, also writes `values` = residual * gain and `squares` (see UnscaledRows)
-    in its epilogue; `rows()` is then what the part after the norm reads."""
+    the residual stream, does the norm's work in its epilogue, and `rows()` is then what the
+    part after the norm reads.  In parts (`squares` given): the product writes `values` =
+    residual * gain and `squares` (see UnscaledRows), and the next product applies the rows'
+    scale.  Whole (`squares` None): the product writes the finished norm into `values`."""
 
     def __init__(self, gain, eps: float, values, squares):
         self.gain, self.eps, self.values, self.squares = gain, eps, values, squares
 
     def following_norm(self):
-        return (self.gain, self.values, self.squares)
+        return (self.gain, self.values, self.squares, self.eps)
 
-    def rows(self) -> UnscaledRows:
-        return UnscaledRows(self.values, self.squares, self.eps)
+    def rows(self):
+        return self.values if self.squares is None else UnscaledRows(self.values, self.squares, self.eps)
 
 
 class Norm(Part):
     def forward(self, ctx, x, out=None):
         raise NotImplementedError
 
-    def fold(self, ctx, n_rows: int) -> Optional[NormFold]:
+    def fold(self, ctx, n_rows: int, whole: bool = False) -> Optional[NormFold]:
         """This norm as work for the neighbouring products (with buffers for `n_rows` rows), or
-        None if it has to run on its own."""
+        None if it has to run on its own.  `whole`: for a product that finishes the norm itself."""
         return None
 
 
@@ -152,7 +154,12 @@ class Mixer(Part):
         return False
 
     def folds_following_norm(self, ctx) -> bool:
-        """Whether `forward` takes a NormFold as a further argument in this step and fills it."""
+        """Whether `forward` takes a NormFold (in parts) as a further argument in this step and fills it."""
+        return False
+
+    def finishes_following_norm(self, ctx) -> bool:
+        """Whether `forward` takes a whole NormFold in this step: its last product also writes the
+        finished norm of the rows it has added into."""
         return False
 
     def forward(self, ctx, binding: CacheBinding, h, residual) -> None:
@@ -164,6 +171,9 @@ class FeedForward(Part):
         return False
 
     def folds_following_norm(self, ctx) -> bool:
+        return False
+
+    def finishes_following_norm(self, ctx) -> bool:
         return False
 
     def forward(self, ctx, h, residual) -> None:
@@ -178,13 +188,17 @@ class Block(Part):
         self.mixer = mixer
         self.feed_forward = feed_forward
 
-    def first_norm_fold(self, ctx, n_rows: int) -> Optional[NormFold]:
-        """The block's first norm as work for the block before it (see NormFold), or None: then
-        `forward` is called without `unscaled`."""
+    def first_norm_fold(self, ctx, n_rows: int, whole: bool = False) -> Optional[NormFold]:
+        """The block's first norm as work for the block before it (see NormFold; `whole` if that
+        block finishes the norm itself), or None: then `forward` is called without `unscaled`."""
         return None
 
     def folds_following_norm(self, ctx) -> bool:
-        """Whether `forward` takes the next block's first norm as `fold_next` in this step."""
+        """Whether `forward` takes the next block's first norm (in parts) as `fold_next` in this step."""
+        return False
+
+    def finishes_following_norm(self, ctx) -> bool:
+        """Whether `forward` takes the next block's first norm whole as `fold_next` in this step."""
         return False
 
     def forward(self, ctx, binding: CacheBinding, x, unscaled: Optional[UnscaledRows] = None,

@@ -11,7 +11,8 @@ from typing import List
 from .base import Block, CacheBinding, TensorDecl, register_block
 
 # A norm between two products can be folded into them where both offer it (short steps in
-# bfloat16: the products then run in kernels that take it): the block asks its parts.
+# bfloat16: the products then run in kernels that take it), or done whole by the product before
+# it where that one offers it (steps whose products split K): the block asks its parts.
 
 
 class PreNormBlock(Block):
@@ -31,17 +32,24 @@ class PreNormBlock(Block):
         for part in (self.norm1, self.mixer, self.norm2, self.feed_forward):
             part.load(store, rt)
 
-    def first_norm_fold(self, ctx, n_rows: int):
+    def first_norm_fold(self, ctx, n_rows: int, whole: bool = False):
+        if whole:
+            return self.norm1.fold(ctx, n_rows, whole=True)
         return self.norm1.fold(ctx, n_rows) if self.mixer.takes_unscaled_rows(ctx) else None
 
     def folds_following_norm(self, ctx) -> bool:
         return self.feed_forward.folds_following_norm(ctx)
 
+    def finishes_following_norm(self, ctx) -> bool:
+        return self.feed_forward.finishes_following_norm(ctx)
+
     def forward(self, ctx, binding: CacheBinding, x, unscaled=None, fold_next=None) -> None:
         mark = ctx.ws.mark()
         h = unscaled if unscaled is not None else self.norm1.forward(ctx, x)
         fold = None
-        if self.mixer.folds_following_norm(ctx) and self.feed_forward.takes_unscaled_rows(ctx):
+        if self.mixer.finishes_following_norm(ctx):
+            fold = self.norm2.fold(ctx, x.shape[0], whole=True)
+        elif self.mixer.folds_following_norm(ctx) and self.feed_forward.takes_unscaled_rows(ctx):
             fold = self.norm2.fold(ctx, x.shape[0])
         if fold is not None:
             self.mixer.forward(ctx, binding, h, x, fold)

@@ -41,6 +41,9 @@ class SwiGLUMLP(FeedForward):
         return (isinstance(self.w_down, PackedMatrix)
                 and ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.hidden, self.ffn, MODE_ADD_F32))
 
+    def finishes_following_norm(self, ctx) -> bool:
+        return isinstance(self.w_down, PackedMatrix) and ctx.rt.k.gemm_then_norm_ok(ctx.n_tokens, self.hidden, self.ffn)
+
     def forward(self, ctx, h, residual, fold=None) -> None:
         k = ctx.rt.k
         T = h.shape[0]

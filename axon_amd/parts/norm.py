@@ -34,10 +34,13 @@ class RMSNorm(Norm):
             out = ctx.ws.take((n, self.size), ctx.rt.dtype)
         return ctx.rt.k.rmsnorm(x, self.gain, self.eps, out, rows)
 
-    def fold(self, ctx, n_rows: int) -> Optional[NormFold]:
-        """The product before the norm leaves x * gain and the sums of squares, the product
-        after it applies 1/sqrt(mean + eps): the same formula, the row's scale moved behind the
-        product (it is common to the row)."""
+    def fold(self, ctx, n_rows: int, whole: bool = False) -> Optional[NormFold]:
+        """In parts: the product before the norm leaves x * gain and the sums of squares, the
+        product after it applies 1/sqrt(mean + eps): the same formula, the row's scale moved
+        behind the product (it is common to the row).  Whole: the product before the norm
+        writes the finished rows."""
+        if whole:
+            return NormFold(self.gain, self.eps, ctx.ws.take((n_rows, self.size), ctx.rt.dtype), None)
         if self.size % 16:
             return None
         values = ctx.ws.take((n_rows, self.size), ctx.rt.dtype)

@@ -230,6 +230,38 @@ def test_gemm_rows_do_not_depend_on_the_batch(dtype):
             assert (whole[rows] - whole[2100][:rows]).abs().max() <= 1e-5 * whole[2100].abs().max()
 
 
+@pytest.mark.parametrize("M,H,F", [(17, 256, 1024), (64, 384, 2048), (100, 256, 1024), (256, 128, 512), (300, 256, 8192),
+                                   (40, 4352, 512)])
+def test_gemm_followed_by_the_whole_norm(M, H, F):
+    """residual += a . Wo^T + bias; h = rmsnorm(residual) * gain, the norm written by the kernel
+    that adds the split product's sums: the same bits as the product and the norm one after the
+    other, and right against the plain formulas.  Where K is not split the kernels refuse."""
+    k = kernels("bfloat16")
+    eps = 2e-5
+    assert k.gemm_then_norm_ok(M, H, F)
+    a, ar = as_dtype(rnd(M, F, seed=50), "bfloat16")
+    wo, wor = as_dtype(rnd(H, F, seed=51, scale=0.3), "bfloat16")
+    w = packed(k, wo)
+    res = rnd(M, H, seed=52, scale=2.0)
+    res[M // 2] *= 40.0
+    bias = rnd(H, seed=53)
+    for gain_dt, b in ((torch.float32, None), (torch.bfloat16, bias.cuda())):
+        gain = (1.0 + 0.3 * rnd(H, seed=54)).to(gain_dt).cuda()
+        x1 = res.clone().cuda()
+        k.gemm(a, w, x1, b, MODE_ADD_F32)
+        h1 = k.rmsnorm(x1, gain, eps, torch.empty(M, H, dtype=torch.bfloat16, device="cuda"))
+        x2 = res.clone().cuda()
+        h2 = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device="cuda")
+        k.gemm(a, w, x2, b, MODE_ADD_F32, following_norm=(gain, h2, None, eps))
+        assert torch.equal(x1, x2) and torch.equal(h1, h2)
+        x_ref = res.double() + ar @ wor.T + (0 if b is None else bias.double())
+        h_ref = P.rms_norm(x_ref, gain.cpu().double(), eps)
+        assert (h2.cpu().double() - h_ref).abs().max() <= tol("bfloat16", h_ref, bf16=1.5e-2)
+    assert not k.gemm_then_norm_ok(8, H, F) and not k.gemm_then_norm_ok(3000, H, F)
+    with pytest.raises(KernelError):
+        k.gemm(a[:8], w, res[:8].clone().cuda(), None, MODE_ADD_F32, following_norm=(gain, h2[:8], None, eps))
+
+
 @pytest.mark.parametrize("M,H,F", [(1, 64, 128), (8, 192, 320), (16, 448, 64), (5, 4608, 64), (13, 128, 192)])
 def test_gemm_with_a_norm_folded_in(M, H, F):
     """residual += a . Wo^T; h = rmsnorm(residual) * gain; out = h . W^T + bias, with the norm done
@@ -249,7 +281,7 @@ def test_gemm_with_a_norm_folded_in(M, H, F):
         x = res.clone().cuda()
         values = torch.empty(M, H, dtype=torch.bfloat16, device="cuda")
         squares = torch.full((M, H // 16), float("nan"), dtype=torch.float32, device="cuda")
-        k.gemm(a, packed(k, wo), x, None, MODE_ADD_F32, following_norm=(gain.cuda(), values, squares))
+        k.gemm(a, packed(k, wo), x, None, MODE_ADD_F32, following_norm=(gain.cuda(), values, squares, eps))
         assert (x.cpu().double() - x_ref).abs().max() <= 2e-5 * math.sqrt(F) * x_ref.abs().max()
         got_sq = squares.cpu().double().sum(1)
         assert ((got_sq - (x_ref ** 2).sum(1)).abs() <= 1e-5 * (x_ref ** 2).sum(1)).all()

@@ -195,6 +195,58 @@ def test_prenorm_block_with_the_norms_folded_into_the_products():
     assert not mixer.takes_unscaled_rows(big.ctx([0] * 17)) and block.first_norm_fold(big.ctx([0] * 17), 17) is None
 
 
+def test_prenorm_block_whose_products_finish_the_norms_behind_them():
+    """A step of some tens of rows in bfloat16 with products wide enough to split K: the output
+    projection writes the second norm's rows and the down projection the next block's first
+    norm, whole; only a norm nobody did for the block runs on its own.  Against the plain formulas."""
+    dtype = "bfloat16"
+    hidden, nh, nkv, hd, ffn, eps, T = 256, 8, 2, 64, 512, 1e-3, 40
+    mixer = build_part("mixer", PartSpec("gqa_attention", {
+        "hidden_size": hidden, "num_heads": nh, "num_kv_heads": nkv, "head_dim": hd, "qkv_bias": True,
+        "position": PartSpec("rope", {"head_dim": hd, "theta": 100.0})}), "model.layers.0.")
+    ffn_part = build_part("feed_forward", PartSpec("swiglu_mlp", {"hidden_size": hidden, "intermediate_size": ffn}),
+                          "model.layers.0.")
+    block = build_block("prenorm", PartSpec("rmsnorm", {"size": hidden, "eps": eps}), mixer, ffn_part, "model.layers.0.")
+    from test_plain import random_weights
+    cfg = P.PlainConfig(1, hidden, nh, nkv, hd, 100.0, eps, True)
+    w = {k: rounded(v.float(), dtype) for k, v in random_weights(cfg, ffn, 10, 0.1).items() if "layers.0" in k}
+    p = "model.layers.0."
+    w[p + "input_layernorm.weight"] = 1.0 + 0.5 * rnd(hidden, seed=3)
+    w[p + "post_attention_layernorm.weight"] = 1.0 + 0.5 * rnd(hidden, seed=4)
+    h = PartHarness(dtype, mixer.cache_spec())
+    load(block, w, h)
+    ctx = h.ctx([0] * T)
+    assert mixer.finishes_following_norm(ctx) and block.finishes_following_norm(ctx)
+    assert not mixer.takes_unscaled_rows(ctx) and not mixer.folds_following_norm(ctx)
+    x0 = rnd(T, hidden, seed=9, scale=3.0)
+    x0[2] *= 30.0
+    next_gain = (1.0 + 0.5 * rnd(hidden, seed=5)).cuda()
+    nxt = block.first_norm_fold(ctx, T, whole=True)
+    nxt.gain, nxt.eps = next_gain, 1e-5
+    calls = []
+    real = h.rt.k.rmsnorm
+    h.rt.k.rmsnorm = lambda *a, **kw: (calls.append(1), real(*a, **kw))[1]
+    try:
+        x = x0.clone().cuda()
+        block.forward(ctx, CacheBinding(0, 0, True), x, None, nxt)
+    finally:
+        h.rt.k.rmsnorm = real
+    assert len(calls) == 1                                                    # the first norm alone
+    wd = {k: v.double() for k, v in w.items()}
+    r = x0.double()
+    r = r + P.attention_block(cfg, wd, 0, P.rms_norm(r, wd[p + "input_layernorm.weight"], eps), torch.arange(T))
+    r = r + P.mlp_block(wd, 0, P.rms_norm(r, wd[p + "post_attention_layernorm.weight"], eps))
+    assert (x.cpu().double() - r).abs().max() <= tol(dtype, r, 1e-5, 3e-2)
+    rows = nxt.rows()
+    want = P.rms_norm(r, next_gain.cpu().double(), 1e-5)
+    assert isinstance(rows, torch.Tensor) and (rows.cpu().double() - want).abs().max() <= tol(dtype, want, 0, 3e-2)
+    # the same block and rows with every norm on its own: the same bits
+    x2 = x0.clone().cuda()
+    block.forward(ctx, CacheBinding(0, 0, True), x2)
+    assert torch.equal(x2, x)
+    assert torch.equal(real(x2, next_gain, 1e-5, torch.empty(T, hidden, dtype=torch.bfloat16, device="cuda")), rows)
+
+
 def test_tied_head_and_embedding_share_the_packed_matrix(tmp_path):
     """bfloat16, widths the matrix cores take: the head's matrix is repacked for its product and
     the embedding reads rows out of that same copy (one matrix in memory); the rows are exact."""
