@@ -178,7 +178,7 @@ extern "C" int axk_rope_table(const int32_t* positions, const double* freqs, flo
 }
 
 // ---------------------------------------------------------------------------- rotary + cache store
-// One block per (token, head slot): q heads are rotated in place, k heads rotated and stored
+// One wave per (token, head slot), four waves a block: q heads are rotated in place, k heads rotated and stored
 // in the request's page for that position, v heads stored as they are (transposed: a page of
 // values is [dim][slot], so that the positions of one dim are contiguous).  Pair i of a head
 // is (i, i + rotary_dim / 2): out_i = a cos - b sin, out_{i+half} = a sin + b cos, each
@@ -189,7 +189,9 @@ __global__ void rope_kv_write_kernel(elem_t* __restrict__ qkv, const float* __re
                                      elem_t* __restrict__ k_cache, elem_t* __restrict__ v_cache, int n_heads,
                                      int n_kv_heads, int head_dim, int rotary_dim, int page_size, int write_kv) {
   const int t = blockIdx.x;
-  const int slot = blockIdx.y;  // 0..nh: q heads; then k heads; then v heads
+  const int slot = blockIdx.y * 4 + threadIdx.x / AXON_WAVE;  // 0..nh: q heads; then k heads; then v heads
+  const int lane = threadIdx.x % AXON_WAVE;
+  if (slot >= n_heads + (write_kv ? 2 * n_kv_heads : 0)) return;
   const int half = rotary_dim / 2;
   const int row_elems = (n_heads + 2 * n_kv_heads) * head_dim;
   elem_t* src = qkv + (size_t)t * row_elems + (size_t)slot * head_dim;
@@ -206,12 +208,12 @@ __global__ void rope_kv_write_kernel(elem_t* __restrict__ qkv, const float* __re
     if (is_v) {
       // values are kept position-contiguous: [page][kv head][dim][slot in page]
       elem_t* vdst = v_cache + ((size_t)page * n_kv_heads + kvh) * head_dim * page_size + in_page;
-      for (int i = threadIdx.x; i < head_dim; i += blockDim.x) vdst[(size_t)i * page_size] = src[i];
+      for (int i = lane; i < head_dim; i += AXON_WAVE) vdst[(size_t)i * page_size] = src[i];
       return;
     }
     dst = k_cache + (((size_t)page * n_kv_heads + kvh) * page_size + in_page) * head_dim;
   }
-  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+  for (int i = lane; i < half; i += AXON_WAVE) {
     const float s = tab[2 * i], c = tab[2 * i + 1];
     const float a = to_float(src[i]), b = to_float(src[i + half]);
     const float lo = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s));
@@ -220,7 +222,7 @@ __global__ void rope_kv_write_kernel(elem_t* __restrict__ qkv, const float* __re
     dst[i + half] = from_float(hi);
   }
   if (dst != src)
-    for (int i = rotary_dim + threadIdx.x; i < head_dim; i += blockDim.x) dst[i] = src[i];
+    for (int i = rotary_dim + lane; i < head_dim; i += AXON_WAVE) dst[i] = src[i];
 }
 
 extern "C" int axk_rope_kv_write(void* qkv, const float* table, const int32_t* positions, const int32_t* seq_rows,
@@ -233,8 +235,8 @@ extern "C" int axk_rope_kv_write(void* qkv, const float* table, const int32_t* p
   AXK_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
               "rope_kv_write: rotary_dim %d must be even and at most head_dim %d", rotary_dim, head_dim);
   if (n_tokens == 0) return 0;
-  dim3 grid(n_tokens, n_heads + (write_kv ? 2 * n_kv_heads : 0));
-  rope_kv_write_kernel<<<grid, 64, 0, (hipStream_t)stream>>>((elem_t*)qkv, table, positions, seq_rows, block_table,
+  dim3 grid(n_tokens, ceil_div(n_heads + (write_kv ? 2 * n_kv_heads : 0), 4));
+  rope_kv_write_kernel<<<grid, 4 * AXON_WAVE, 0, (hipStream_t)stream>>>((elem_t*)qkv, table, positions, seq_rows, block_table,
                                                             table_stride, (elem_t*)k_cache, (elem_t*)v_cache,
                                                             n_heads, n_kv_heads, head_dim, rotary_dim, page_size,
                                                             write_kv);

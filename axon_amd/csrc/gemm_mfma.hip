@@ -861,7 +861,7 @@ static int small_splits(int n, int k, int mode) {
 static int long_k_splits(int n, int k, int mode) {
   if (n % 4 != 0) return 1;
   const int n_blocks = ceil_div(n, mode == MODE_SWIGLU ? 128 : 256), nk = k / 64;
-  return nk >= 128 && n_blocks <= 18 ? 2 : 1;
+  return (nk >= 128 && n_blocks <= 18) || (nk >= 48 && n_blocks <= 14) ? 2 : 1;
 }
 
 static int splits_of(int m, int n, int k, int mode) {
