@@ -1,0 +1,76 @@
+"""One layer of the sizes the engine is measured at (width 3584, 28 query heads on 4 kv heads of
+128, feed-forward 18944) with a small vocabulary, against the plain implementation: the tiny
+configurations of the other tests never meet the kernels that these widths select (products
+that split K between blocks, norms finished by the product before them, the prompt kernel with
+two heads a block and a group of 7, decoding over several chunks).  A mixed schedule takes
+every product through each of its classes of rows (up to 16, 64, 256, more)."""
+import pytest
+import torch
+
+import axon_amd
+from axon_amd.config import config_from_dict
+from axon_amd.engine import StepEntry
+from axon_amd.weights import write_random_model
+from helpers import tolerance
+from plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+FULL = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=1, hidden_size=3584, intermediate_size=18944,
+            num_attention_heads=28, num_key_value_heads=4, head_dim=128, vocab_size=1024, max_position_embeddings=4096,
+            rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
+
+
+@pytest.fixture(scope="module")
+def full_layer(tmp_path_factory):
+    d = str(tmp_path_factory.mktemp("full_layer"))
+    write_random_model(config_from_dict(FULL), d, seed=31, std=0.02, storage="bfloat16")
+    cfg, w = P.load_plain(d)
+    g = torch.Generator().manual_seed(2)
+    prompts = {rid: torch.randint(0, FULL["vocab_size"], (n,), generator=g).tolist()
+               for rid, n in (("a", 620), ("b", 150), ("c", 61))}
+    oracle = {rid: P.forward_logits(cfg, w, toks) for rid, toks in prompts.items()}
+    return d, prompts, oracle
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_a_layer_of_the_measured_sizes_through_every_class_of_rows(dtype, full_layer):
+    d, prompts, oracle = full_layer
+    llm = axon_amd.load(d, dtype=dtype, page_size=16, num_pages=64, max_seqs=4, max_batch_tokens=512)
+    eng = llm.engine
+    fed = {rid: 0 for rid in prompts}
+    worst = 0.0
+
+    def step(parts, end=()):
+        """parts: (request, tokens to feed, wanted places among them)"""
+        nonlocal worst
+        entries, where = [], []
+        for rid, n, want in parts:
+            at = fed[rid]
+            entries.append(StepEntry(rid, prompts[rid][at:at + n], want))
+            where += [(rid, at + w) for w in want]
+            fed[rid] = at + n
+        logits = eng.step(entries, end=end)
+        if where:
+            got = logits.cpu().double()
+            for row, (rid, pos) in zip(got, where):
+                ref = oracle[rid][pos]
+                err = float((row - ref).abs().max())
+                assert err <= tolerance(dtype, ref), (rid, pos, err)
+                worst = max(worst, err / tolerance(dtype, ref))
+
+    step([("a", 300, [0, 150, 299])])                              # a prompt portion of more than 256 rows
+    step([("a", 130, [129]), ("b", 70, [3, 69])])                  # 200 rows: two portions
+    step([("a", 150, [149]), ("b", 2, [1]), ("c", 40, [39])])      # 192 rows, a portion of two tokens
+    step([("a", 1, [0]), ("b", 30, [29]), ("c", 19, [18])])        # 50 rows: a decoded token beside portions
+    step([("a", 1, [0]), ("b", 40, [0, 39]), ("c", 1, [0])])       # 42 rows
+    for _ in range(8):                                             # single tokens: the short-step kernels, graphs
+        step([("a", 1, [0]), ("b", 1, [0])])
+    step([("c", 1, [0])], end=["c"])
+    step([("a", 22, list(range(22)))])                             # 22 rows of one request, all wanted
+    for _ in range(8):
+        step([("a", 1, [0])])                                      # over 600 positions: three chunks
+    assert fed == {"a": 620, "b": 150, "c": 61}
+    eng.release_all()
+    eng.cache.check()
+    assert eng.cache.free_pages() == 64
