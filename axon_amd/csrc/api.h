@@ -54,7 +54,8 @@ int axk_attention(const void* q, int q_stride, const void* k_cache, const void* 
 // axk_attention_fast_ok: 1 if they take this head size, page size and group of heads.
 // axk_attention_prefill: tiles [n_tiles][2] = (first token, count <= 128): consecutive tokens of
 // one request; every token of the step in some tile gets its row of `out`.
-// axk_attention_decode: token_index [n_tokens] names single tokens; a context longer than one
+// axk_attention_decode: token_index [n_tokens] names single tokens (null: the first n_tokens
+// tokens of the step); a context longer than one
 // chunk (axk_attention_decode_chunk positions) is cut into chunks whose partial results go
 // through `partial` (axk_attention_decode_workspace floats) and are folded in ascending order;
 // max_chunks is the most chunks any of the tokens has.

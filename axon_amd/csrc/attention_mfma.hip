@@ -342,12 +342,13 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
   constexpr int KS = HD / 32;   // k steps of S^T (32 dims each)
   constexpr int DT = HD / 16;   // output tiles (16 dims each)
   constexpr int ROW = HD + 4;   // floats of a head's row in LDS (padded: rows start in different banks)
-  __shared__ float fold_o[4][16][ROW];
-  __shared__ float fold_ml[4][16][2];
+  extern __shared__ float fold_lds[];                // [4 waves][group][ROW] outputs, then [4][group][2] max and sum
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int t = token_index[blockIdx.z];
+  const int t = token_index ? token_index[blockIdx.z] : blockIdx.z;
   const int kvh = blockIdx.y, chunk = blockIdx.x;
   const int group = n_heads / n_kv_heads;
+  float* fold_o = fold_lds;
+  float* fold_ml = fold_lds + 4 * group * ROW;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
   const int first = (lo / DC_CHUNK) * DC_CHUNK;
@@ -467,34 +468,35 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
 
   if (r16 < group) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(&fold_o[wave][r16][dt * 16 + q4 * 4]) = o_acc[dt];
+    for (int dt = 0; dt < DT; ++dt)
+      *reinterpret_cast<f32x4*>(&fold_o[(wave * group + r16) * ROW + dt * 16 + q4 * 4]) = o_acc[dt];
     if (q4 == 0) {
-      fold_ml[wave][r16][0] = m;
-      fold_ml[wave][r16][1] = l;
+      fold_ml[(wave * group + r16) * 2] = m;
+      fold_ml[(wave * group + r16) * 2 + 1] = l;
     }
   }
-  } else if (lane < 16) {
-    fold_ml[wave][lane][0] = -INFINITY;
-    fold_ml[wave][lane][1] = 0.0f;
+  } else if (lane < group) {
+    fold_ml[(wave * group + lane) * 2] = -INFINITY;
+    fold_ml[(wave * group + lane) * 2 + 1] = 0.0f;
   }
   __syncthreads();
 
   // ---- the four waves' results into one, in wave order: a thread takes 4 dims of a head
   for (int task = threadIdx.x; task < group * (HD / 4); task += 256) {
     const int hg = task / (HD / 4), d = (task % (HD / 4)) * 4;
-    float M = fold_ml[0][hg][0];
+    float M = fold_ml[hg * 2];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) M = fmaxf(M, fold_ml[w][hg][0]);
+    for (int w = 1; w < 4; ++w) M = fmaxf(M, fold_ml[(w * group + hg) * 2]);
     const float mref = M == -INFINITY ? 0.0f : M;
     float L = 0.0f;
     f32x4 O = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      const float mw = fold_ml[w][hg][0];
+      const float mw = fold_ml[(w * group + hg) * 2];
       if (mw == -INFINITY) continue;                 // a wave without positions wrote no output
       const float weight = __builtin_amdgcn_exp2f(mw - mref);
-      L = fmaf(fold_ml[w][hg][1], weight, L);
-      const f32x4 o = *reinterpret_cast<const f32x4*>(&fold_o[w][hg][d]);
+      L = fmaf(fold_ml[(w * group + hg) * 2 + 1], weight, L);
+      const f32x4 o = *reinterpret_cast<const f32x4*>(&fold_o[(w * group + hg) * ROW + d]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) O[e] = fmaf(o[e], weight, O[e]);
     }
@@ -531,7 +533,7 @@ attention_combine_kernel(const float* __restrict__ partial, const int32_t* __res
                          int window) {
   __shared__ float weight[CMB_MAX_CHUNKS];
   __shared__ float red[2][HD / 64];
-  const int t = token_index[blockIdx.x], head = blockIdx.y, d = threadIdx.x;
+  const int t = token_index ? token_index[blockIdx.x] : blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
   const int n_chunks = (pos - (lo / DC_CHUNK) * DC_CHUNK) / DC_CHUNK + 1;
@@ -645,16 +647,17 @@ extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_c
               page_size, n_heads, n_kv_heads);
   AXK_REQUIRE(max_chunks <= CMB_MAX_CHUNKS, "attention_decode: %d chunks of %d positions (at most %d: %d positions)",
               max_chunks, DC_CHUNK, CMB_MAX_CHUNKS, CMB_MAX_CHUNKS * DC_CHUNK);
-  AXK_REQUIRE(n_tokens >= 0 && max_chunks >= 1 && max_chunks <= 65535 && n_kv_heads <= 65535 && window >= 0 &&
+  AXK_REQUIRE(n_tokens >= 0 && n_tokens <= 65535 && max_chunks >= 1 && n_kv_heads <= 65535 && window >= 0 &&
                   q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0,
               "attention_decode: bad arguments (tokens %d, chunks %d, window %d, q stride %d)", n_tokens, max_chunks,
               window, q_stride);
   AXK_REQUIRE(max_chunks == 1 || partial != nullptr, "attention_decode: %d chunks need a workspace", max_chunks);
   if (n_tokens == 0) return 0;
+  const int group = n_heads / n_kv_heads;
   dim3 grid(max_chunks, n_kv_heads, n_tokens), cgrid(n_tokens, n_heads);
 #define LAUNCH(HD)                                                                                                   \
   {                                                                                                                  \
-    attention_decode_kernel<HD><<<grid, 256, 0, (hipStream_t)stream>>>(                                               \
+    attention_decode_kernel<HD><<<grid, 256, 4 * group * (HD + 4 + 2) * sizeof(float), (hipStream_t)stream>>>(      \
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,       \
         positions, seq_rows, (bf16_t*)out, token_index, partial, max_chunks, n_heads, n_kv_heads, page_size, window, \
         scale);                                                                                                      \

@@ -292,12 +292,18 @@ class Kernels:
 
     def attention_decode(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, token_index,
                          partial, max_chunks, n_heads, n_kv_heads, head_dim, page_size, window, scale) -> torch.Tensor:
-        """Attention of single decoding tokens named by token_index (int32)."""
+        """Attention of single decoding tokens named by token_index (int32), or of the first
+        `token_index` tokens of the step if that is a number."""
         self._elem(q, "attention q"); self._elem(out, "attention out")
         self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
         self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
-        self._i32(token_index, "token_index")
-        n = token_index.numel()
+        if isinstance(token_index, int):
+            n, token_index = token_index, None
+        else:
+            self._i32(token_index, "token_index")
+            n = token_index.numel()
+        if n > q.shape[0]:
+            raise KernelError(f"attention_decode: {n} tokens, q has {q.shape[0]} rows")
         if out.shape[1] != n_heads * head_dim or not out.is_contiguous():
             raise KernelError(f"attention_decode: out {tuple(out.shape)}")
         if max_chunks > 1:

@@ -37,9 +37,9 @@ class AttentionPlan:
         self.tiles = None
         self.partial = None
         if ctx.decode_only:
-            # every span is one token: the engine keeps the index list on the device and has
-            # counted the chunks (what a captured graph replays must not come from the host)
-            self.decode_tokens = ctx.decode_index
+            # every span is one token, in order: no index list; the engine has counted the chunks
+            # (what a captured graph replays must not come from the host)
+            self.decode_tokens = ctx.n_tokens
             self.max_chunks = ctx.decode_shapes[("attention_chunks", window)]
             n_single = ctx.n_tokens
         else:

@@ -80,7 +80,7 @@ def main() -> int:
     p = prompt()
     eng.step([StepEntry("warm", p, [len(p) - 1])], end=["warm"])
     torch.cuda.synchronize()
-    reps = args.steps if args.phase == "prefill" else 1
+    reps = args.steps if args.phase == "prefill" else 4      # back to back: the average of full prefill steps
     t0 = time.perf_counter()
     for _ in range(reps):
         eng.step([StepEntry("pf", p, [len(p) - 1])], end=["pf"])

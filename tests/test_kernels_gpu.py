@@ -493,6 +493,14 @@ def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
     one = torch.tensor([picks[-1]], dtype=torch.int32).cuda()
     k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, solo, one, partial, chunks, nh, nkv, hd, page, window, scale)
     assert torch.equal(solo[picks[-1]], out[picks[-1]])
+    # without an index list: the first tokens of the step
+    first = min(T, 70)
+    named, plain = torch.zeros_like(out), torch.zeros_like(out)
+    wide = torch.empty(k.attention_decode_workspace(first, nh, hd, chunks), dtype=torch.float32, device="cuda")
+    k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, named, torch.arange(first, dtype=torch.int32).cuda(), wide,
+                       chunks, nh, nkv, hd, page, window, scale)
+    k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, plain, first, wide, chunks, nh, nkv, hd, page, window, scale)
+    assert torch.equal(named, plain) and (plain[:first].cpu().double() - ref[:first]).abs().max() <= tol("bfloat16", ref, bf16=1.5e-2)
 
 
 def test_matrix_core_attention_finds_a_far_key_and_respects_the_windows_edge():
