@@ -468,7 +468,7 @@ def test_prompt_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
 
 @pytest.mark.parametrize("nh,nkv,hd,page,T,window", [
     (4, 2, 64, 16, 300, 0), (7, 1, 128, 16, 1030, 0), (28, 4, 128, 16, 600, 0), (6, 2, 128, 8, 255, 0),
-    (2, 2, 64, 64, 257, 0), (16, 1, 64, 32, 513, 0), (4, 1, 64, 16, 900, 300), (5, 5, 128, 16, 64, 0), (3, 1, 128, 16, 700, 70)])
+    (2, 2, 64, 64, 257, 0), (16, 1, 64, 32, 513, 0), (4, 1, 64, 16, 900, 300), (5, 5, 128, 16, 64, 0), (3, 1, 128, 16, 700, 70), (4, 1, 128, 16, 4100, 0), (2, 1, 64, 32, 3000, 1000)])
 def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
     k = kernels("bfloat16")
     q, kc, vc, table, ref = _mfma_case(nh, nkv, hd, page, T, window, seed=5)
