@@ -2,8 +2,8 @@
 // portions, one for decoding tokens.  Both keep the order of attention.hip: positions in
 // blocks of 64 aligned to absolute position, folded in ascending order with running
 // (max, sum, output); the decoding kernel gives every block of 64 positions to a wave of its
-// own (a size that depends on nothing) and a second kernel folds the blocks' partial results
-// in ascending order.  No atomics.  Scores, softmax and all sums are 32-bit; q, k, v and the
+// own, folds the four waves of a chunk of 256 positions in wave order (sizes that depend on
+// nothing) and a second kernel folds the chunks' partial results in ascending order.  No atomics.  Scores, softmax and all sums are 32-bit; q, k, v and the
 // softmax weights enter the MFMAs as bfloat16.
 //
 // Both compute the TRANSPOSED products, S^T = K Q^T and O^T = V^T P^T, so that what one MFMA
