@@ -52,8 +52,11 @@ int axk_attention(const void* q, int q_stride, const void* k_cache, const void* 
 
 // The matrix-core attention kernels (bfloat16 build; the float32 build refuses them).
 // axk_attention_fast_ok: 1 if they take this head size, page size and group of heads.
-// axk_attention_prefill: tiles [n_tiles][2] = (first token, count <= 128): consecutive tokens of
-// one request; every token of the step in some tile gets its row of `out`.
+// axk_attention_prefill: tiles [n_tiles][4] = (first token, count <= 128) twice: consecutive
+// tokens of one request, and a second such run (count 0: none) that the same block takes after
+// the first; every token of the step in some run gets its row of `out`.  A causal prompt's runs
+// see 1, 2, 3 ... blocks of positions: pairing one that sees many with one that sees few gives
+// every block about the same work.
 // axk_attention_decode: token_index [n_tokens] names single tokens (null: the first n_tokens
 // tokens of the step); a context longer than one
 // chunk (axk_attention_decode_chunk positions) is cut into chunks whose partial results go

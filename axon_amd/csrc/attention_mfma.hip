@@ -57,13 +57,12 @@ __device__ inline uint32_t pack_bf16(float a, float b) { return pack2_bf16(a, b)
 #define PF_BLOCK 64
 
 template <int HD, int HPB>
-__global__ void __launch_bounds__(256 * HPB, 2)
-attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
-                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
-                         const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
-                         bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int n_heads, int n_kv_heads,
-                         int page_size, int window, float scale) {
-  extern __shared__ __align__(16) unsigned char smem[];
+__device__ __forceinline__ void
+attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __restrict__ q, int q_stride,
+                       const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                       const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ positions,
+                       const int32_t* __restrict__ seq_rows, bf16_t* __restrict__ out, int n_heads, int n_kv_heads,
+                       int page_size, int window, float scale) {
   constexpr int K_BYTES = PF_BLOCK * HD * 2;      // K tile: 64 rows of HD
   constexpr int V_BYTES = HD * PF_BLOCK * 2;      // V^T tile: HD rows of 64 positions
   constexpr int STAGE = K_BYTES + V_BYTES;
@@ -79,7 +78,6 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
 
   const int tid = threadIdx.x, lane = tid & 63, block_wave = tid >> 6;
   const int wave = block_wave & 3;                 // which 32 query rows of the tile
-  const int t0 = tiles[2 * blockIdx.x], count = tiles[2 * blockIdx.x + 1];
   const int group = n_heads / n_kv_heads, sets = (group + HPB - 1) / HPB;   // sets of HPB query heads per kv head
   const int kvh = blockIdx.y / sets;
   const int in_group = (blockIdx.y % sets) * HPB + (block_wave >> 2);
@@ -319,6 +317,28 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
       pk.y = pack_bf16(o_acc[dt][g * 4 + 2] * inv, o_acc[dt][g * 4 + 3] * inv);
       *reinterpret_cast<uint2*>(orow + d) = pk;
     }
+}
+
+// A block takes one tile or two, one after the other: tiles [n][4] = (first token, count) twice,
+// the second count 0 if there is none.  The caller pairs a tile that sees many positions with
+// one that sees few, so that every block has about the same work (a causal prompt's tiles see
+// 1, 2, 3 ... blocks of positions).
+template <int HD, int HPB>
+__global__ void __launch_bounds__(256 * HPB, 2)
+attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
+                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
+                         const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
+                         bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int n_heads, int n_kv_heads,
+                         int page_size, int window, float scale) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int32_t* mine = tiles + 4 * blockIdx.x;
+  for (int part = 0; part < 2; ++part) {
+    const int t0 = mine[2 * part], count = mine[2 * part + 1];
+    if (count <= 0) break;                        // the same for the whole block
+    if (part) __syncthreads();                    // everyone has read the first tile's last stage
+    attention_prefill_tile<HD, HPB>(smem, t0, count, q, q_stride, k_cache, v_cache, block_table, table_stride, positions,
+                                    seq_rows, out, n_heads, n_kv_heads, page_size, window, scale);
+  }
 }
 
 // ============================================================================ decoding tokens
@@ -613,8 +633,10 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,      \
         positions, seq_rows, (bf16_t*)out, tiles, n_heads, n_kv_heads, page_size, window, scale);                   \
   }
-  // two query heads a block where a kv head has more than one
-  if (group >= 2) {
+  // two query heads of a kv head a block (they share each K and V block in LDS) where that still
+  // gives the chip's 256 CUs about a block each; else one head a block
+  const int blocks_of_pairs = n_tiles * n_kv_heads * ((group + 1) / 2);
+  if (group >= 2 && blocks_of_pairs >= 200) {
     if (head_dim == 64) LAUNCH(64, 2) else LAUNCH(128, 2)
   } else {
     if (head_dim == 64) LAUNCH(64, 1) else LAUNCH(128, 1)

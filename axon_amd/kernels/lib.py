@@ -268,12 +268,17 @@ class Kernels:
 
     def attention_prefill(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, tiles, n_heads,
                           n_kv_heads, head_dim, page_size, window, scale) -> torch.Tensor:
-        """Attention of prompt portions: tiles [n, 2] int32 = (first token, count <= 128)."""
+        """Attention of prompt portions: tiles [n, 4] int32 = (first token, count <= 128) twice, the
+        two runs of tokens one block takes one after the other (second count 0: none); [n, 2]
+        is taken as one run a block.  `pair_tiles` pairs runs so that blocks get equal work."""
         self._elem(q, "attention q"); self._elem(out, "attention out")
         self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
         self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
         self._i32(tiles, "tiles")
-        if out.shape[1] != n_heads * head_dim or not out.is_contiguous() or tiles.dim() != 2 or tiles.shape[1] != 2:
+        if tiles.dim() == 2 and tiles.shape[1] == 2:
+            tiles = torch.cat([tiles, torch.zeros_like(tiles)], dim=1).contiguous()
+        if (out.shape[1] != n_heads * head_dim or not out.is_contiguous() or tiles.dim() != 2 or tiles.shape[1] != 4
+                or not tiles.is_contiguous()):
             raise KernelError(f"attention_prefill: out {tuple(out.shape)}, tiles {tuple(tiles.shape)}")
         self._check(self.lib.axk_attention_prefill(
             _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[-1], _ptr(positions),

@@ -43,25 +43,41 @@ class AttentionPlan:
             self.max_chunks = ctx.decode_shapes[("attention_chunks", window)]
             n_single = ctx.n_tokens
         else:
-            tiles, singles, chunks = [], [], 1
+            tiles, seen, singles, chunks = [], [], [], 1
             for s in ctx.spans:
                 if s.q_len == 1:
                     singles.append(s.q_start)
                     chunks = max(chunks, decode_chunks_of(s.start_pos, window, ctx.rt.k.attention_decode_chunk))
                 else:
                     for at in range(0, s.q_len, PREFILL_TILE):
-                        tiles.append((s.q_start + at, min(PREFILL_TILE, s.q_len - at)))
+                        n = min(PREFILL_TILE, s.q_len - at)
+                        tiles.append((s.q_start + at, n))
+                        last = s.start_pos + at + n                 # positions the tile's last token sees
+                        seen.append(min(last, window + n) if window > 0 else last)
             # the kernels trust these indices: check them here, on the host
             if (any(a < 0 or n < 1 or a + n > ctx.n_tokens for a, n in tiles)
                     or any(not 0 <= t < ctx.n_tokens for t in singles)):
                 raise ValueError("attention plan: a span lies outside the tokens of the step")
-            self.tiles = torch.tensor(tiles, dtype=torch.int32).to(dev) if tiles else None
+            self.tiles = torch.tensor(pair_tiles(tiles, seen), dtype=torch.int32).to(dev) if tiles else None
             self.decode_tokens = torch.tensor(singles, dtype=torch.int32).to(dev) if singles else None
             self.max_chunks = chunks
             n_single = len(singles)
         if n_single and self.max_chunks > 1:
             n = ctx.rt.k.attention_decode_workspace(n_single, n_heads, head_dim, self.max_chunks)
             self.partial = torch.empty(n, dtype=torch.float32, device=dev)
+
+
+def pair_tiles(tiles, seen):
+    """Two tiles a block, one that sees many positions with one that sees few: the tiles of a
+    causal prompt see 1, 2, 3 ... blocks of positions, and blocks of equal work finish together.
+    tiles: (first token, count); seen: positions each looks at.  Rows of (first, count, first,
+    count), the second count 0 where a tile is left alone."""
+    order = sorted(range(len(tiles)), key=lambda i: -seen[i])
+    rows = []
+    for k in range((len(order) + 1) // 2):
+        a, b = order[k], order[len(order) - 1 - k]
+        rows.append(tiles[a] + (tiles[b] if b != a else (0, 0)))
+    return rows
 
 
 def decode_chunks_of(pos: int, window: int, chunk: int) -> int:

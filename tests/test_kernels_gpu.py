@@ -457,6 +457,18 @@ def test_prompt_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
         assert not torch.isnan(out).any()                      # unused cache rows hold NaN: they must not leak
         assert (out[start:].cpu().double() - ref[start:]).abs().max() <= tol("bfloat16", ref, bf16=1.5e-2)
         assert out[:start].abs().sum() == 0                    # rows outside the tiles are not touched
+    # two tiles a block, paired as the engine pairs them: the same bits as one tile a block
+    from axon_amd.parts.attention import pair_tiles
+    tiles = [(a, min(128, T - a)) for a in range(0, T, 128)]
+    single = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+    k.attention_prefill(q, nh * hd, kc, vc, table, pos, rows, single, torch.tensor(tiles, dtype=torch.int32).cuda(), nh, nkv,
+                        hd, page, window, scale)
+    pairs = pair_tiles(tiles, [a + n for a, n in tiles])
+    assert sorted(t for row in pairs for t in (row[:2], row[2:]) if t[1]) == tiles
+    paired = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+    k.attention_prefill(q, nh * hd, kc, vc, table, pos, rows, paired, torch.tensor(pairs, dtype=torch.int32).cuda(), nh, nkv,
+                        hd, page, window, scale)
+    assert torch.equal(single, paired)
     # odd tiles: 2 tokens, 33 tokens, one token short of a block edge
     tiles = [(5, 2), (60, min(33, T - 63)), (T - 3, 3)]          # every tile lies inside the T tokens
     out = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
