@@ -89,6 +89,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   constexpr int STAGE = (BM + BN) * ROW;               // bytes per stage
   static_assert(XQ >= 1 && WQ >= 1 && (STAGES - 2) * (XQ + WQ) < 64, "tile too small or too many loads in flight");
   static_assert(BN / 16 * KBT % NW == 0 && WN % 32 == 0, "the 1 KB chunks of W are shared out evenly");
+  static_assert(!GLU || TN % 2 == 0, "a wave's gate columns and up columns are whole MFMA tiles");
 #define SWZ(row) (BK == 64 ? (((row) >> 1) & 7) : (((row) >> 2) & 3))
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
