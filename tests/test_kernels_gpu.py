@@ -164,7 +164,8 @@ def packed(k, w, gated=False):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (3, 100, 70), (17, 259, 130), (70, 96, 33), (130, 48, 257),
                                    (5, 1000, 512), (64, 256, 256), (200, 384, 1024), (33, 152, 3584), (64, 1000, 2048),
-                                   (20, 8200, 512), (48, 130, 1024), (100, 132, 2048), (256, 260, 1024)])
+                                   (20, 8200, 512), (48, 130, 1024), (100, 132, 2048), (256, 260, 1024),
+                                   (2048, 4608, 192), (1100, 9300, 128), (700, 260, 8192)])
 def test_gemm_every_epilogue(dtype, M, N, K):
     k = kernels(dtype)
     x, xr = as_dtype(rnd(M, K, seed=10), dtype)
@@ -191,7 +192,7 @@ def test_gemm_every_epilogue(dtype, M, N, K):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,F,K", [(1, 96, 64), (9, 176, 64), (40, 320, 192), (64, 130, 128), (70, 300, 128),
                                    (300, 512, 256), (600, 1000, 128), (5, 100, 70), (33, 19, 33), (2100, 384, 64),
-                                   (40, 320, 1024), (17, 132, 2048), (64, 96, 4096), (130, 96, 2048)])
+                                   (40, 320, 1024), (17, 132, 2048), (64, 96, 4096), (130, 96, 2048), (2048, 2600, 64)])
 def test_gemm_with_the_gated_epilogue(dtype, M, F, K):
     """One product over [gate; up] whose epilogue is silu(gate) * up."""
     k = kernels(dtype)
