@@ -58,8 +58,10 @@ int axk_attention(const void* q, int q_stride, const void* k_cache, const void* 
 // see 1, 2, 3 ... blocks of positions: pairing one that sees many with one that sees few gives
 // every block about the same work.
 // axk_attention_decode: token_index [n_tokens] names single tokens (null: the first n_tokens
-// tokens of the step); a context longer than one
-// chunk (axk_attention_decode_chunk positions) is cut into chunks whose partial results go
+// tokens of the step); a token's range (from the chunk that holds the window's first position,
+// or 0) is cut into chunks of axk_attention_decode_chunk positions.  work [n_work] lists the
+// chunks to compute, item = slot in token_index * axk_attention_decode_item_factor + chunk, or
+// -1 for none: every chunk of every token once.  With more than one chunk the partial results go
 // through `partial` (axk_attention_decode_workspace floats) and are folded in ascending order;
 // max_chunks is the most chunks any of the tokens has.
 int axk_attention_fast_ok(int head_dim, int page_size, int n_heads, int n_kv_heads);
@@ -69,12 +71,13 @@ int axk_attention_prefill(const void* q, int q_stride, const void* k_cache, cons
                           int n_heads, int n_kv_heads, int head_dim, int page_size, int window,
                           float scale, void* stream);
 int axk_attention_decode_chunk(void);
+int axk_attention_decode_item_factor(void);
 long axk_attention_decode_workspace(int n_tokens, int n_heads, int head_dim, int max_chunks);
 int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                          const int32_t* block_table, int table_stride, const int32_t* positions,
                          const int32_t* seq_rows, void* out, const int32_t* token_index, int n_tokens,
-                         float* partial, int max_chunks, int n_heads, int n_kv_heads, int head_dim,
-                         int page_size, int window, float scale, void* stream);
+                         const int32_t* work, int n_work, float* partial, int max_chunks, int n_heads,
+                         int n_kv_heads, int head_dim, int page_size, int window, float scale, void* stream);
 
 // The matrix-core products (bfloat16 build) read W packed: blocks of 16 rows x 32 k of 1 KB in
 // the order in which a wave holds them as an MFMA operand, [row tile][k block], rows padded with

@@ -18,7 +18,8 @@
 #include "api.h"
 #include "common.h"
 
-#define DC_CHUNK 256   // positions of one chunk of a decoding token's range
+#define DC_CHUNK 256          // positions of one chunk of a decoding token's range
+#define CMB_MAX_CHUNKS 1024   // the most chunks of a token; the factor of the token's slot in a work item
 
 #if AXON_BF16
 
@@ -342,14 +343,18 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
 }
 
 // ============================================================================ decoding tokens
-// grid (tokens, kv heads, chunks): a block of four waves per (token, kv head, chunk of 256
-// positions); a wave takes 64 of them.  The wave issues every load of its positions at once (K
-// rows and V^T rows go straight from the pages into 16x16x32 MFMA operands, 32 KB in flight per
-// wave), then multiplies; the query heads of the group are the 16 columns (a group of up to 16
-// heads).  The four waves' results are folded in LDS, in wave order.  Output: if the token's
-// whole range is one chunk, the normalised result; else the chunk's (max, sum, unnormalised
-// output) into `partial`, folded by attention_combine_kernel.  How a token's range is cut
-// depends on its own position and the window alone, never on the rest of the batch.
+// grid (work items x kv heads): a block of four waves per (token, kv head, chunk of 256
+// positions); a wave takes 64 of them.  The work list names the chunks that exist, token by
+// token (item = token slot * CMB_MAX_CHUNKS + chunk, -1: nothing), so that a batch of short and
+// long contexts launches no block without work: a block that only finds out that it has none
+// still holds its place on a CU for a good part of a working block's time.  The wave issues
+// every load of its positions at once (K rows and V^T rows go straight from the pages into
+// 16x16x32 MFMA operands, 32 KB in flight per wave), then multiplies; the query heads of the
+// group are the 16 columns (a group of up to 16 heads).  The four waves' results are folded in
+// LDS, in wave order.  Output: if the token's whole range is one chunk, the normalised result;
+// else the chunk's (max, sum, unnormalised output) into `partial`, folded by
+// attention_combine_kernel.  How a token's range is cut depends on its own position and the
+// window alone, never on the rest of the batch.
 #define DC_WAVE 64
 
 template <int HD>
@@ -357,15 +362,20 @@ __global__ void __launch_bounds__(256)
 attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
                         const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
-                        bf16_t* __restrict__ out, const int32_t* __restrict__ token_index, float* __restrict__ partial,
-                        int max_chunks, int n_heads, int n_kv_heads, int page_size, int window, float scale) {
+                        bf16_t* __restrict__ out, const int32_t* __restrict__ token_index,
+                        int n_tokens, const int32_t* __restrict__ work, float* __restrict__ partial, int max_chunks,
+                        int n_heads, int n_kv_heads, int page_size, int window, float scale) {
   constexpr int KS = HD / 32;   // k steps of S^T (32 dims each)
   constexpr int DT = HD / 16;   // output tiles (16 dims each)
   constexpr int ROW = HD + 4;   // floats of a head's row in LDS (padded: rows start in different banks)
   extern __shared__ float fold_lds[];                // [4 waves][group][ROW] outputs, then [4][group][2] max and sum
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int t = token_index ? token_index[blockIdx.z] : blockIdx.z;
-  const int kvh = blockIdx.y, chunk = blockIdx.x;
+  const int item = work[blockIdx.x / n_kv_heads];    // the kv heads of a chunk side by side: they share its pages
+  if (item < 0) return;                              // padding of the list
+  const int slot = item / CMB_MAX_CHUNKS, chunk = item % CMB_MAX_CHUNKS;
+  if (slot >= n_tokens || chunk >= max_chunks) return;   // no item of this launch
+  const int t = token_index ? token_index[slot] : slot;
+  const int kvh = blockIdx.x % n_kv_heads;
   const int group = n_heads / n_kv_heads;
   float* fold_o = fold_lds;
   float* fold_ml = fold_lds + 4 * group * ROW;
@@ -529,7 +539,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
       *reinterpret_cast<uint2*>(out + (size_t)t * n_heads * HD + (size_t)head * HD + d) = pk;
     } else {
       // partial [token slot][head][chunk][HD + 2]: output, then max (log2 domain) and sum
-      float* dst = partial + (((size_t)blockIdx.z * n_heads + head) * max_chunks + chunk) * (HD + 2);
+      float* dst = partial + (((size_t)slot * n_heads + head) * max_chunks + chunk) * (HD + 2);
       *reinterpret_cast<float2*>(dst + d) = make_float2(O[0], O[1]);
       *reinterpret_cast<float2*>(dst + d + 2) = make_float2(O[2], O[3]);
       if (d == 0) {
@@ -544,7 +554,6 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
 // L = sum l_c 2^(m_c - M) and O = sum o_c 2^(m_c - M); out = O / L.  The sums run in a fixed
 // order (the chunks' weights by a butterfly over lanes, the outputs chunk by chunk ascending).
 // grid (tokens, heads), HD threads.
-#define CMB_MAX_CHUNKS 1024
 
 template <int HD>
 __global__ void __launch_bounds__(HD)
@@ -650,8 +659,10 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
 #endif
 }
 
-// Positions of one chunk of a decoding token's range.
+// Positions of one chunk of a decoding token's range, and the factor of the token's slot in an
+// item of the work list (item = slot * factor + chunk).
 extern "C" int axk_attention_decode_chunk(void) { return DC_CHUNK; }
+extern "C" int axk_attention_decode_item_factor(void) { return CMB_MAX_CHUNKS; }
 
 // Floats of `partial` that n_tokens decoding tokens with up to max_chunks chunks need.
 extern "C" long axk_attention_decode_workspace(int n_tokens, int n_heads, int head_dim, int max_chunks) {
@@ -661,8 +672,9 @@ extern "C" long axk_attention_decode_workspace(int n_tokens, int n_heads, int he
 extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                     const int32_t* block_table, int table_stride, const int32_t* positions,
                                     const int32_t* seq_rows, void* out, const int32_t* token_index, int n_tokens,
-                                    float* partial, int max_chunks, int n_heads, int n_kv_heads, int head_dim,
-                                    int page_size, int window, float scale, void* stream) {
+                                    const int32_t* work, int n_work, float* partial, int max_chunks, int n_heads,
+                                    int n_kv_heads, int head_dim, int page_size, int window, float scale,
+                                    void* stream) {
 #if AXON_BF16
   AXK_REQUIRE(axk_attention_fast_ok(head_dim, page_size, n_heads, n_kv_heads),
               "attention_decode: head_dim %d, page size %d, %d/%d heads are not taken by this kernel", head_dim,
@@ -674,15 +686,17 @@ extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_c
               "attention_decode: bad arguments (tokens %d, chunks %d, window %d, q stride %d)", n_tokens, max_chunks,
               window, q_stride);
   AXK_REQUIRE(max_chunks == 1 || partial != nullptr, "attention_decode: %d chunks need a workspace", max_chunks);
-  if (n_tokens == 0) return 0;
+  AXK_REQUIRE(n_work >= 0 && (n_work == 0 || work != nullptr) && (long)n_work * n_kv_heads < (1l << 31),
+              "attention_decode: a work list of %d items", n_work);
+  if (n_tokens == 0 || n_work == 0) return 0;
   const int group = n_heads / n_kv_heads;
-  dim3 grid(max_chunks, n_kv_heads, n_tokens), cgrid(n_tokens, n_heads);
+  dim3 grid((unsigned)n_work * n_kv_heads), cgrid(n_tokens, n_heads);
 #define LAUNCH(HD)                                                                                                   \
   {                                                                                                                  \
     attention_decode_kernel<HD><<<grid, 256, 4 * group * (HD + 4 + 2) * sizeof(float), (hipStream_t)stream>>>(      \
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,       \
-        positions, seq_rows, (bf16_t*)out, token_index, partial, max_chunks, n_heads, n_kv_heads, page_size, window, \
-        scale);                                                                                                      \
+        positions, seq_rows, (bf16_t*)out, token_index, n_tokens, work, partial, max_chunks, n_heads, n_kv_heads,    \
+        page_size, window, scale);                                                                                   \
     if (max_chunks > 1)                                                                                              \
       attention_combine_kernel<HD><<<cgrid, HD, 0, (hipStream_t)stream>>>(partial, positions, token_index,          \
                                                                          (bf16_t*)out, max_chunks, n_heads, window); \

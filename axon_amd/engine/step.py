@@ -72,6 +72,7 @@ class StepContext:
         self.decode_only = False
         self.decode_index: Optional[torch.Tensor] = None
         self.decode_shapes: Dict = {}
+        self.decode_inputs: Dict = {}       # what the mixers asked to have on the device (Mixer.decode_input)
 
     def no_rotation(self) -> torch.Tensor:
         return torch.empty((self.n_tokens, 0, 2), dtype=torch.float32, device=self.rt.device)
@@ -119,6 +120,18 @@ class Engine:
             if pair is not None and pair[0] not in seen:
                 seen.add(pair[0])
                 self._shape_mixers.append(b.mixer)
+        # what mixers want on the device in a decoding step (Mixer.decode_input): a buffer that stays
+        # where it is, and its staging ring
+        self._input_mixers, self._inputs, self._input_hosts = [], {}, {}
+        seen = set()
+        for b in model.blocks:
+            asked = b.mixer.decode_input([0])
+            if asked is not None and asked[0] not in seen:
+                seen.add(asked[0])
+                cap = max(1, b.mixer.decode_input_capacity(cfg.max_seqs, self.max_seq_len))
+                self._input_mixers.append(b.mixer)
+                self._inputs[asked[0]] = torch.full((cap,), -1, dtype=torch.int32, device=rt.device)
+                self._input_hosts[asked[0]] = [torch.full((cap,), -1, dtype=torch.int32).pin_memory() for _ in range(4)]
         self._meta = torch.zeros((3, cfg.max_seqs), dtype=torch.int32, device=rt.device)
         # staging in pinned memory, a ring: a step's inputs and picks travel while the host
         # prepares the next step
@@ -274,13 +287,14 @@ class Engine:
         return self._pending
 
     # ------------------------------------------------------------------ decoding steps
-    def _decode_forward(self, T: int, spans: List[Span], shapes: Dict):
+    def _decode_forward(self, T: int, spans: List[Span], shapes: Dict, inputs: Dict):
         """A step of T single tokens whose tokens, positions and slots are in `self._meta`: the
         launches that a graph captures.  Logits go to the static buffer, greedy picks beside them."""
         ctx = StepContext(self.rt, self.cache, self.ws, self._meta, T, spans)
         ctx.decode_only = True
         ctx.decode_index = self._index[:T]
         ctx.decode_shapes = shapes
+        ctx.decode_inputs = inputs
         x = self.model.forward(ctx)
         logits = self.model.logits(ctx, x, ctx.decode_index, out=self._logits[:T])
         self.rt.k.argmax(logits, self._picks[:T])
@@ -313,21 +327,32 @@ class Engine:
         for mixer in self._shape_mixers:
             name, value = mixer.decode_shape(positions)
             shapes[name] = value
+        inputs = {}
+        for mixer in self._input_mixers:
+            name, values = mixer.decode_input(positions)
+            n = len(values)
+            if n > self._inputs[name].numel():
+                raise StepError(f"{name}: {n} values for the device, room for {self._inputs[name].numel()}")
+            staged = self._input_hosts[name][at]
+            staged[:n] = torch.tensor(values, dtype=torch.int32)
+            self._inputs[name][:n].copy_(staged[:n], non_blocking=True)
+            inputs[name] = self._inputs[name][:n]
+            shapes[("values of", name)] = n          # a graph reads exactly this many
         if not self.graphs_ok:
-            logits = self._decode_forward(T, spans, shapes)
+            logits = self._decode_forward(T, spans, shapes, inputs)
         else:
             key = (T, tuple(sorted(shapes.items(), key=repr)))
             entry = self._graphs.get(key)
             if entry is None:
                 # once without capture: kernels set themselves up at their first launch, and a
                 # decoding step writes the same cache rows however often it runs
-                self._decode_forward(T, spans, shapes)
+                self._decode_forward(T, spans, shapes, inputs)
                 torch.cuda.synchronize()
                 graph = torch.cuda.CUDAGraph()
                 if self._graph_pool is None:
                     self._graph_pool = torch.cuda.graph_pool_handle()
                 with torch.cuda.graph(graph, pool=self._graph_pool):
-                    logits = self._decode_forward(T, spans, shapes)
+                    logits = self._decode_forward(T, spans, shapes, inputs)
                 entry = self._graphs[key] = (graph, logits)
             entry[0].replay()
             logits = entry[1]

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_char_p, c_double, c_float, c_int, c_void_p
-from typing import Dict, Optional
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -45,7 +45,8 @@ _SIGNATURES = {
     "axk_attention_prefill": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "axk_attention_decode": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                             c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                             c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                             c_float, c_void_p],
     "axk_attention_fast_ok": [c_int, c_int, c_int, c_int],
     "axk_gemm": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
                  ctypes.c_long, c_void_p],
@@ -295,10 +296,27 @@ class Kernels:
     def attention_decode_workspace(self, n_tokens: int, n_heads: int, head_dim: int, max_chunks: int) -> int:
         return int(self.lib.axk_attention_decode_workspace(n_tokens, n_heads, head_dim, max_chunks))
 
+    def attention_decode_work(self, positions: Sequence[int], window: int, pad_to: int = 0) -> List[int]:
+        """The work list of the decoding kernel for single tokens at `positions` (in the order
+        of their slots): one item per (token, chunk), slot * factor + chunk, a token's chunks
+        side by side; padded with -1 to `pad_to` items."""
+        chunk, factor = self.attention_decode_chunk, int(self.lib.axk_attention_decode_item_factor())
+        items = []
+        for slot, pos in enumerate(positions):
+            lo = max(0, pos + 1 - window) if window > 0 else 0
+            n = (pos - lo // chunk * chunk) // chunk + 1
+            if n > factor:
+                raise KernelError(f"attention_decode: a context of {pos + 1} positions is more than {factor} chunks")
+            items.extend(slot * factor + c for c in range(n))
+        return items + [-1] * max(0, pad_to - len(items))
+
     def attention_decode(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, token_index,
-                         partial, max_chunks, n_heads, n_kv_heads, head_dim, page_size, window, scale) -> torch.Tensor:
+                         partial, max_chunks, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                         work: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Attention of single decoding tokens named by token_index (int32), or of the first
-        `token_index` tokens of the step if that is a number."""
+        `token_index` tokens of the step if that is a number.  `work` (int32, on the device):
+        the chunks to compute, as `attention_decode_work` lists them; None: made here from the
+        positions, which waits for the device."""
         self._elem(q, "attention q"); self._elem(out, "attention out")
         self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
         self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
@@ -315,10 +333,17 @@ class Kernels:
             self._f32(partial, "attention partial")
             if partial.numel() < self.attention_decode_workspace(n, n_heads, head_dim, max_chunks):
                 raise KernelError(f"attention_decode: workspace of {partial.numel()} floats is too small")
+        if work is None:
+            at = positions[:n] if token_index is None else positions[token_index.long()]
+            work = torch.tensor(self.attention_decode_work(at.tolist(), window), dtype=torch.int32).to(q.device)
+        self._i32(work, "attention work list")
+        if work.dim() != 1 or not work.is_contiguous():
+            raise KernelError(f"attention_decode: work list {tuple(work.shape)}")
         self._check(self.lib.axk_attention_decode(
             _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[-1], _ptr(positions),
-            _ptr(seq_rows), _ptr(out), _ptr(token_index), n, _ptr(partial if max_chunks > 1 else None), max_chunks,
-            n_heads, n_kv_heads, head_dim, page_size, window, float(scale), _stream()))
+            _ptr(seq_rows), _ptr(out), _ptr(token_index), n, _ptr(work), work.numel(),
+            _ptr(partial if max_chunks > 1 else None), max_chunks, n_heads, n_kv_heads, head_dim, page_size, window,
+            float(scale), _stream()))
         return out
 
     def pack_ok(self, rows: int, cols: int, gated: bool = False) -> bool:

@@ -36,11 +36,14 @@ class AttentionPlan:
         dev = ctx.rt.device
         self.tiles = None
         self.partial = None
+        self.decode_work = None
         if ctx.decode_only:
             # every span is one token, in order: no index list; the engine has counted the chunks
-            # (what a captured graph replays must not come from the host)
+            # and brought the list of them to the device (what a captured graph replays must not
+            # come from the host)
             self.decode_tokens = ctx.n_tokens
             self.max_chunks = ctx.decode_shapes[("attention_chunks", window)]
+            self.decode_work = ctx.decode_inputs[("attention_work", window)]
             n_single = ctx.n_tokens
         else:
             tiles, seen, singles, chunks = [], [], [], 1
@@ -62,6 +65,10 @@ class AttentionPlan:
             self.decode_tokens = torch.tensor(singles, dtype=torch.int32).to(dev) if singles else None
             self.max_chunks = chunks
             n_single = len(singles)
+            if singles:
+                at = {s.q_start: s.start_pos for s in ctx.spans if s.q_len == 1}
+                work = ctx.rt.k.attention_decode_work([at[t] for t in singles], window)
+                self.decode_work = torch.tensor(work, dtype=torch.int32).to(dev)
         if n_single and self.max_chunks > 1:
             n = ctx.rt.k.attention_decode_workspace(n_single, n_heads, head_dim, self.max_chunks)
             self.partial = torch.empty(n, dtype=torch.float32, device=dev)
@@ -78,6 +85,12 @@ def pair_tiles(tiles, seen):
         a, b = order[k], order[len(order) - 1 - k]
         rows.append(tiles[a] + (tiles[b] if b != a else (0, 0)))
     return rows
+
+
+def round_up_by_eighths(n: int) -> int:
+    """n rounded up to a multiple of a power of two that is at most an eighth of it."""
+    step = 1 << max(0, n.bit_length() - 4)
+    return -(-n // step) * step
 
 
 def decode_chunks_of(pos: int, window: int, chunk: int) -> int:
@@ -118,6 +131,7 @@ class GQAttention(Mixer):
         self.n = {k: base + names.get(k, k + "_proj") for k in ("q", "k", "v", "o")}
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
         self.decode_chunk = 1 << 30          # until `load` has asked the kernels: one chunk
+        self._work_list = lambda positions, window: list(range(len(positions)))
 
     # ------------------------------------------------------------------ declarations
     def tensors(self) -> List[TensorDecl]:
@@ -138,15 +152,25 @@ class GQAttention(Mixer):
         return CacheSpec(entries=2, heads=self.nkv, head_dim=self.hd, window=self.window)
 
     def decode_shape(self, positions):
-        """The decoding kernel's grid depends on the longest context, in chunks of the kernel's
-        size, rounded up in steps of an eighth or less so that few shapes exist and few blocks of
-        the grid find nothing to do (they cost their launch all the same)."""
+        """The decoding kernel's workspace is laid out by the longest context of the step, in
+        chunks of the kernel's size, rounded up in steps of an eighth or less so that few shapes
+        exist."""
         most = max(decode_chunks_of(p, self.window, self.decode_chunk) for p in positions)
-        step = 1 << max(0, most.bit_length() - 4)
-        return ("attention_chunks", self.window), -(-most // step) * step
+        return ("attention_chunks", self.window), round_up_by_eighths(most)
+
+    def decode_input(self, positions):
+        """The list of the chunks the decoding kernel computes, a block each: blocks are launched
+        for the chunks that exist, not for the longest context times the tokens.  Padded in
+        steps of an eighth or less."""
+        work = self._work_list(positions, self.window)
+        return ("attention_work", self.window), work + [-1] * (round_up_by_eighths(len(work)) - len(work))
+
+    def decode_input_capacity(self, max_seqs: int, max_seq_len: int) -> int:
+        return round_up_by_eighths(max_seqs * decode_chunks_of(max(0, max_seq_len - 1), 0, self.decode_chunk))
 
     def load(self, store, rt) -> None:
         self.decode_chunk = rt.k.attention_decode_chunk
+        self._work_list = rt.k.attention_decode_work
         self.w_qkv = rt.k.prepare_weight(store.fused_matrix([self.n[k] + ".weight" for k in ("q", "k", "v")]))
         biases = [store.vector(self.n[k] + ".bias", optional=True) for k in ("q", "k", "v")] if self.qkv_bias else []
         present = [b is not None for b in biases]
@@ -212,7 +236,8 @@ class GQAttention(Mixer):
             if plan.tiles is not None:
                 k.attention_prefill(qkv, qkv.stride(0), *common, plan.tiles, *sizes)
             if plan.decode_tokens is not None:
-                k.attention_decode(qkv, qkv.stride(0), *common, plan.decode_tokens, plan.partial, plan.max_chunks, *sizes)
+                k.attention_decode(qkv, qkv.stride(0), *common, plan.decode_tokens, plan.partial, plan.max_chunks, *sizes,
+                                   work=plan.decode_work)
         else:
             k.attention(qkv, qkv.stride(0), k_cache, v_cache, group.block_table, ctx.positions, ctx.seq_rows, att,
                         self.nh, self.nkv, self.hd, group.page_size, self.window, self.scale)

@@ -20,7 +20,7 @@ configuration then names it in a `PartSpec`.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Callable, Dict, List, Optional, Tuple
+from typing import Sequence, Any, Callable, Dict, List, Optional, Tuple
 
 from ..config.base import ConfigError, PartSpec
 
@@ -148,6 +148,19 @@ class Mixer(Part):
         that a captured graph is replayed only for steps of the same shape.  The pair is handed
         back in `ctx.decode_shapes[name]`.  None: nothing else matters."""
         return None
+
+    def decode_input(self, positions) -> Optional[Tuple[Any, Sequence[int]]]:
+        """For a step of single tokens at `positions`: (name, int32 values) that this mixer's
+        kernels read from the device (say, a list of the work to launch), or None.  The engine
+        copies the values into a buffer that stays where it is (a captured graph reads it again
+        at every replay) and hands it back as `ctx.decode_inputs[name]`; how many values there
+        are is part of the step's shape, so pad them to few different lengths."""
+        return None
+
+    def decode_input_capacity(self, max_seqs: int, max_seq_len: int) -> int:
+        """The most values `decode_input` ever returns with this many live requests of up to
+        this many positions each."""
+        return 0
 
     def takes_unscaled_rows(self, ctx) -> bool:
         """Whether `h` may be UnscaledRows in this step (the first product applies the scale)."""

@@ -506,6 +506,16 @@ def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
     one = torch.tensor([picks[-1]], dtype=torch.int32).cuda()
     k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, solo, one, partial, chunks, nh, nkv, hd, page, window, scale)
     assert torch.equal(solo[picks[-1]], out[picks[-1]])
+    # the list of chunks given by the caller, padded and in another order: the same bits
+    import random
+    work = k.attention_decode_work(picks, window, pad_to=len(picks) * chunks + 7)
+    assert sum(1 for w in work if w >= 0) == sum((p - ((max(0, p + 1 - window) if window else 0) // ch * ch)) // ch + 1
+                                                 for p in picks)
+    random.Random(3).shuffle(work)
+    listed = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+    k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, listed, idx, partial, chunks, nh, nkv, hd, page, window, scale,
+                       work=torch.tensor(work, dtype=torch.int32).cuda())
+    assert torch.equal(listed, out)
     # without an index list: the first tokens of the step
     first = min(T, 70)
     named, plain = torch.zeros_like(out), torch.zeros_like(out)
