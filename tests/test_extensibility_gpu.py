@@ -43,7 +43,17 @@ class DecayMixer(Mixer):
     def load(self, store, rt):
         self.w_in, self.w_out = store.matrix(self.n_in).float(), store.matrix(self.n_out).float()
 
+    # values of its own on the device in steps of single tokens (here only to show the way: the
+    # positions, padded to a multiple of four)
+    def decode_input(self, positions):
+        return "toy_positions", list(positions) + [-1] * (-len(positions) % 4)
+
+    def decode_input_capacity(self, max_seqs, max_seq_len):
+        return max_seqs + 3
+
     def forward(self, ctx, binding, h, residual):
+        if ctx.decode_only:
+            self.seen_on_device = ctx.decode_inputs["toy_positions"].clone()
         arena = ctx.cache.state(binding.state_index)
         u = h.float() @ self.w_in.T
         for span in ctx.spans:                                   # each request's tokens, in order
@@ -270,6 +280,9 @@ def test_the_toy_model_steps_like_its_plain_twin(toy_dir, dtype):
     # and generation works through the same entry point
     out = llm.generate([seqs[0][:9], seqs[1][:5]], max_new_tokens=6)
     assert [len(o) for o in out] == [6, 6]
+    # what the toy mixer asked to have on the device in the last step of single tokens
+    decay = next(b.mixer for b in llm.model.blocks if isinstance(b.mixer, DecayMixer))
+    assert decay.seen_on_device.tolist() == [13, 9, -1, -1]
     if dtype == "float32":
         for p, o in zip((seqs[0][:9], seqs[1][:5]), out):
             hist = list(p)
