@@ -153,10 +153,10 @@ class GQAttention(Mixer):
 
     def decode_shape(self, positions):
         """The decoding kernel's workspace is laid out by the longest context of the step, in
-        chunks of the kernel's size, rounded up in steps of an eighth or less so that few shapes
-        exist."""
+        chunks of the kernel's size, rounded up to a power of two so that few shapes exist (the
+        blocks that are launched are those of `decode_input`, whatever this number)."""
         most = max(decode_chunks_of(p, self.window, self.decode_chunk) for p in positions)
-        return ("attention_chunks", self.window), round_up_by_eighths(most)
+        return ("attention_chunks", self.window), 1 << (most - 1).bit_length()
 
     def decode_input(self, positions):
         """The list of the chunks the decoding kernel computes, a block each: blocks are launched
