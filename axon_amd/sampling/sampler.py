@@ -135,16 +135,21 @@ def pick_rows(rt, logits: torch.Tensor, samplers: Sequence[Optional[Sampler]],
         n = len(device_rows)
         recents = [samplers[r].recent(histories[r]) for r in device_rows]
         width = max(1, max(len(x) for x in recents))
-        rec = torch.zeros((n, width), dtype=torch.int32)
+        ks = [min(samplers[r].params.top_k, vocab) for r in device_rows]
+        # one copy to the device: the recent tokens, how many, k, and the penalties' bits
+        flat = torch.zeros(n * width + 3 * n, dtype=torch.int32)
+        rec = flat[:n * width].view(n, width)
         for i, x in enumerate(recents):
             rec[i, :len(x)] = torch.tensor(x, dtype=torch.int32)
-        ks = [min(samplers[r].params.top_k, vocab) for r in device_rows]
-        n_rec = torch.tensor([len(x) for x in recents], dtype=torch.int32)
-        pen = torch.tensor([samplers[r].params.repeat_penalty for r in device_rows], dtype=torch.float32)
-        k_t = torch.tensor(ks, dtype=torch.int32)
+        flat[n * width:n * width + n] = torch.tensor([len(x) for x in recents], dtype=torch.int32)
+        flat[n * width + n:n * width + 2 * n] = torch.tensor(ks, dtype=torch.int32)
+        flat[n * width + 2 * n:].view(torch.float32)[:] = torch.tensor(
+            [samplers[r].params.repeat_penalty for r in device_rows], dtype=torch.float32)
+        on = flat.to(dev)
         sel = logits if n == rows else logits[torch.tensor(device_rows, device=dev)].contiguous()
         cands = torch.zeros((n, max(ks)), dtype=torch.int64, device=dev)
-        rt.k.topk(sel, rec.to(dev), n_rec.to(dev), pen.to(dev), k_t.to(dev), cands)
+        rt.k.topk(sel, on[:n * width].view(n, width), on[n * width:n * width + n], on[n * width + 2 * n:].view(torch.float32),
+                  on[n * width + n:n * width + 2 * n], cands)
         host = cands.cpu()
         for i, r in enumerate(device_rows):
             picks[r] = samplers[r].pick_keys(host[i, :ks[i]].contiguous())
