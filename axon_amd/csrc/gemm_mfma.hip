@@ -857,12 +857,26 @@ static int small_splits(int n, int k, int mode) {
   return s < 1 ? 1 : s;
 }
 
-// 257 to 2048 rows: a narrow output over a long K (the feed-forward's down projection) gives too
-// few tiles for 256 CUs; K is halved.  By (N, K) alone.
+// 257 to 2048 rows: a narrow output gives too few 256 x 256 tiles for 256 CUs, or a number of
+// them that leaves the last round mostly idle; K is then cut into 2 to 4 parts.  By (N, K)
+// alone (the tiles are counted for 2,048 rows).  The time of the product is the rounds of blocks
+// over the parts; adding the parts' sums costs about 500 / K of the product's ideal time a
+// part (twice that for [gate; up]).  A cut has to win 8 % and leave 24 K tiles a part.
 static int long_k_splits(int n, int k, int mode) {
   if (n % 4 != 0) return 1;
-  const int n_blocks = ceil_div(n, mode == MODE_SWIGLU ? 128 : 256), nk = k / 64;
-  return (nk >= 128 && n_blocks <= 18) || (nk >= 48 && n_blocks <= 14) ? 2 : 1;
+  const bool glu = mode == MODE_SWIGLU;
+  const int tiles = 8 * ceil_div(n, glu ? 128 : 256), nk = k / 64;
+  int best = 1;
+  double best_cost = (double)ceil_div(tiles, 256);
+  for (int s = 2; s <= 4; ++s) {
+    if (nk / s < 24) break;
+    const double cost = (double)ceil_div(tiles * s, 256) / s + 500.0 * s / k * (tiles / 256.0) * (glu ? 2 : 1);
+    if (cost < 0.92 * best_cost) {
+      best = s;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 static int splits_of(int m, int n, int k, int mode) {
