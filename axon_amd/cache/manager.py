@@ -19,7 +19,7 @@ from __future__ import annotations
 import ctypes
 from ctypes import POINTER, c_char_p, c_int, c_long, c_void_p
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import List, Sequence, Tuple
 
 import torch
 

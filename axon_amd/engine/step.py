@@ -15,12 +15,12 @@ The reference runs prompt portions and decode rows as two passes of one schedule
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, Hashable, Iterable, List, Optional, Sequence
 
 import torch
 
-from ..cache.manager import CacheManager, OutOfPages
+from ..cache.manager import CacheManager
 from ..config.engine import EngineConfig
 from ..models.decoder import DecoderModel
 from .runtime import Runtime, Workspace

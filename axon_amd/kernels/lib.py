@@ -8,7 +8,7 @@ other implementation behind these calls: without the library they fail.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_double, c_float, c_int, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_void_p
 from typing import Dict, List, Optional, Sequence
 
 import torch

@@ -19,8 +19,8 @@ configuration then names it in a `PartSpec`.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Sequence, Any, Callable, Dict, List, Optional, Tuple
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
 
 from ..config.base import ConfigError, PartSpec
 

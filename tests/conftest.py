@@ -27,7 +27,7 @@ def pytest_collection_modifyitems(config, items):
 def model_dirs(tmp_path_factory):
     """Model folders of the tiny configurations with random weights, made once per session in
     a temporary folder: {(name, storage): path}."""
-    from helpers import TINY, make_model_dir
+    from helpers import make_model_dir
     made = {}
 
     def get(name: str, storage: str = "float32") -> str:

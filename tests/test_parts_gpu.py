@@ -1,6 +1,5 @@
 """Each part of a layer alone, built from a PartSpec with sizes of its own, against the plain
 function of the same part."""
-import math
 
 import pytest
 import torch

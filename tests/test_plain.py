@@ -10,7 +10,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from helpers import TINY, tolerance
+from helpers import tolerance
 from plain import qwen2_plain as P
 
 torch.manual_seed(0)

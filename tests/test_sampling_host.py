@@ -1,5 +1,4 @@
 """The native host sampler against the plain one and the reference's own vectors."""
-import ctypes
 import math
 import random
 
