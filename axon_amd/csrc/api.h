@@ -132,16 +132,19 @@ int axk_gemm_then_norm(const void* x, int x_stride, const void* w, const void* b
                        float norm_eps, void* norm_values, void* workspace, long workspace_bytes, void* stream);
 
 // The attention's [q; k; v] product (W packed, [(n_heads + 2 n_kv_heads) head_dim, K], or the q rows alone
-// if write_kv is 0) with what follows it as its epilogue: bias, the rotary encoding of q and k
+// if write_kv is 0) with what follows it in the same launches: bias, the rotary encoding of q and k
 // heads over their whole width (table [M, head_dim / 2, 2]: sin, cos), q into qkv [M, >= n_heads
-// head_dim], k and v into the request's pages (as axk_rope_kv_write stores them).  in_squares as in
-// axk_gemm_norm_fold, or null.  Bit-identical to axk_gemm followed by axk_rope_kv_write.
-int axk_gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim);
+// head_dim], k and v into the request's pages (as axk_rope_kv_write stores them).  Up to 16 rows it
+// is the product's epilogue (in_squares as in axk_gemm_norm_fold, or null); with more rows, where
+// the product splits K (axk_gemm_qkv_rope_ok says so; n = the rows of W), the kernel that adds the
+// parts' sums rotates and stores; workspace: axk_gemm_workspace(m, n, k, 0) bytes.  Bit-identical
+// to axk_gemm followed by axk_rope_kv_write.
+int axk_gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotary_dim);
 int axk_gemm_qkv_rope(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* qkv,
                       int qkv_stride, int m, int k, const float* in_squares, float in_eps, const float* table,
                       const int32_t* positions, const int32_t* seq_rows, const int32_t* block_table, int table_stride,
                       void* k_cache, void* v_cache, int n_heads, int n_kv_heads, int head_dim, int page_size,
-                      int write_kv, void* stream);
+                      int write_kv, void* workspace, long workspace_bytes, void* stream);
 
 // out[t, f] = silu(gu[t, f]) * gu[t, F + f]: gate in the first F columns, up in the last.
 int axk_swiglu(const void* gate_up, void* out, int n_tokens, int n_ffn, void* stream);

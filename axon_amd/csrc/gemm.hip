@@ -151,12 +151,13 @@ int launch_pack_matrix(const bf16_t* src, bf16_t* dst, int rows, int k, hipStrea
 size_t gemm_workspace_bytes(int m, int n, int k, int mode);
 int gemm_norm_fold_ok(int m, int n, int k, int mode);
 int gemm_then_norm_ok(int m, int n, int k);
-int gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim);
+int gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotary_dim);
 int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out,
                          int out_stride, int m, int n, int k, const float* in_squares, float in_eps,
                          const float* table, const int32_t* positions, const int32_t* seq_rows,
                          const int32_t* block_table, int table_stride, bf16_t* k_cache, bf16_t* v_cache, int n_heads,
-                         int n_kv_heads, int head_dim, int page_size, hipStream_t stream);
+                         int n_kv_heads, int head_dim, int page_size, void* workspace, size_t workspace_bytes,
+                         hipStream_t stream);
 #endif
 
 static int gemm_checked(const void* x, int x_stride, const void* w, int w_packed, const void* bias, int bias_is_f32,
@@ -263,9 +264,9 @@ extern "C" int axk_gemm_then_norm(const void* x, int x_stride, const void* w, co
                       workspace_bytes, stream);
 }
 
-extern "C" int axk_gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim) {
+extern "C" int axk_gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotary_dim) {
 #if AXON_BF16
-  return gemm_qkv_rope_ok(m, k, head_dim, rotary_dim);
+  return n > 0 && k > 0 && head_dim > 0 && gemm_qkv_rope_ok(m, n, k, head_dim, rotary_dim);
 #else
   return 0;   // the 32-bit build keeps the product, the rotation and the store apart
 #endif
@@ -275,24 +276,26 @@ extern "C" int axk_gemm_qkv_rope(const void* x, int x_stride, const void* w, con
                                  void* qkv, int qkv_stride, int m, int k, const float* in_squares, float in_eps,
                                  const float* table, const int32_t* positions, const int32_t* seq_rows,
                                  const int32_t* block_table, int table_stride, void* k_cache, void* v_cache,
-                                 int n_heads, int n_kv_heads, int head_dim, int page_size, int write_kv, void* stream) {
+                                 int n_heads, int n_kv_heads, int head_dim, int page_size, int write_kv, void* workspace,
+                                 long workspace_bytes, void* stream) {
 #if AXON_BF16
-  AXK_REQUIRE(n_heads > 0 && n_kv_heads > 0 && page_size > 0 && axk_gemm_qkv_rope_ok(m, k, head_dim, head_dim),
-              "gemm_qkv_rope: M=%d K=%d head_dim=%d heads %d/%d page %d are not taken", m, k, head_dim, n_heads,
-              n_kv_heads, page_size);
+  AXK_REQUIRE(n_heads > 0 && n_kv_heads > 0 && page_size > 0 && head_dim > 0, "gemm_qkv_rope: heads %d/%d of %d, page %d",
+              n_heads, n_kv_heads, head_dim, page_size);
   const int n = (n_heads + (write_kv ? 2 * n_kv_heads : 0)) * head_dim;
+  AXK_REQUIRE(axk_gemm_qkv_rope_ok(m, n, k, head_dim, head_dim), "gemm_qkv_rope: M=%d N=%d K=%d head_dim=%d are not taken",
+              m, n, k, head_dim);
   AXK_REQUIRE(x_stride >= k && x_stride % 8 == 0 && qkv_stride >= n_heads * head_dim && qkv_stride % 4 == 0 &&
                   ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)qkv & 7) == 0 &&
                   ((uintptr_t)table & 15) == 0 && ((uintptr_t)in_squares & 15) == 0,
               "gemm_qkv_rope: strides x=%d qkv=%d or the alignment of an operand are not taken", x_stride, qkv_stride);
-  AXK_REQUIRE(in_squares == nullptr || axk_gemm_norm_fold_ok(m, n, k, MODE_STORE),
+  AXK_REQUIRE(in_squares == nullptr || (m <= 16 && axk_gemm_norm_fold_ok(m, n, k, MODE_STORE)),
               "gemm_qkv_rope: no norm is folded into a step of %d rows", m);
   AXK_REQUIRE(table && positions && (!write_kv || (seq_rows && block_table && k_cache && v_cache)),
               "gemm_qkv_rope: a table, the positions or the cache is missing");
   return launch_gemm_qkv_rope((const bf16_t*)x, x_stride, (const bf16_t*)w, bias, bias_is_f32, (bf16_t*)qkv, qkv_stride,
                               m, n, k, in_squares, in_eps, table, positions, seq_rows, block_table, table_stride,
-                              (bf16_t*)k_cache, (bf16_t*)v_cache, n_heads, n_kv_heads, head_dim, page_size,
-                              (hipStream_t)stream);
+                              (bf16_t*)k_cache, (bf16_t*)v_cache, n_heads, n_kv_heads, head_dim, page_size, workspace,
+                              workspace_bytes > 0 ? (size_t)workspace_bytes : 0, (hipStream_t)stream);
 #else
   axk_set_error("gemm_qkv_rope: only in the bfloat16 build");
   return -1;

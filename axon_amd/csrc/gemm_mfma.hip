@@ -439,10 +439,14 @@ gemm_split_reduce_norm_kernel(const float* __restrict__ partial, int splits, int
   }
 }
 
+struct RopeStore;
+static int launch_split_reduce_rope(const float* partial, int splits, int m, int n, const void* bias, int bias_is_f32,
+                                    void* out, int out_stride, const RopeStore& rope, hipStream_t stream);
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK = 64, int STAGES = 2>
 static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                        int out_stride, int m, int n, int k, int mode, hipStream_t stream, int splits = 1,
-                       float* partial = nullptr, const SplitNorm* norm = nullptr) {
+                       float* partial = nullptr, const SplitNorm* norm = nullptr, const RopeStore* rope = nullptr) {
   static bool configured = false;
   constexpr int lds_bytes = STAGES * (BM + BN) * BK * 2;
   static_assert(lds_bytes <= 160 * 1024, "the stages do not fit the LDS of a CU");
@@ -460,6 +464,7 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
   kernel<<<dim3(m_blocks * n_blocks, splits), WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks, splits > 1 ? partial : nullptr);
   AXK_LAUNCH_CHECK("gemm_tile");
+  if (splits > 1 && rope != nullptr) return launch_split_reduce_rope(partial, splits, m, n, bias, bias_is_f32, out, out_stride, *rope, stream);
   if (splits > 1 && norm != nullptr) {
     gemm_split_reduce_norm_kernel<<<m, SRN_THREADS, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, (float*)out, out_stride,
                                                          *norm);
@@ -518,6 +523,59 @@ struct RopeStore {
 };
 
 enum { EPI_PLAIN = 0, EPI_GLU = 1, EPI_ROPE = 2 };
+
+// The sums of a split [q; k; v] product with the bias, the rotary encoding and the store into the
+// pages: what gemm_split_reduce_kernel (storing bfloat16) and the rotary kernel do one after the
+// other, bit for bit.  One wave per (token, head slot), four waves a block; q heads go rotated to
+// `out`, k heads rotated into the request's page of keys, v heads as they are into its page of
+// values.  Every head is rotated over its whole width.
+__global__ void __launch_bounds__(256)
+gemm_split_reduce_rope_kernel(const float* __restrict__ partial, int splits, int M, int N, const void* __restrict__ bias,
+                              int bias_is_f32, bf16_t* __restrict__ out, int out_stride, RopeStore rope) {
+  const int m = blockIdx.x, slot = blockIdx.y * 4 + threadIdx.x / AXON_WAVE, lane = threadIdx.x % AXON_WAVE;
+  const int hd = rope.head_dim, half = hd / 2;
+  if (slot * hd >= N) return;
+  const size_t plane = (size_t)M * N;
+  // a column's sum, rounded as the product's own store rounds it
+  auto value = [&](int col) {
+    const float* src = partial + (size_t)m * N + col;
+    float g = src[0];
+    for (int z = 1; z < splits; ++z) g += src[(size_t)z * plane];
+    if (bias) g += load_vec(bias, bias_is_f32, col);
+    return bf16_to_float(float_to_bf16(g));
+  };
+  bf16_t* dst;
+  if (slot < rope.n_heads) {
+    dst = out + (size_t)m * out_stride + (size_t)slot * hd;
+  } else {
+    const int pos = rope.positions[m];
+    const int page = rope.block_table[(size_t)rope.seq_rows[m] * rope.table_stride + pos / rope.page_size];
+    const int in_page = pos % rope.page_size;
+    if (slot >= rope.n_heads + rope.n_kv_heads) {
+      const int kvh = slot - rope.n_heads - rope.n_kv_heads;
+      bf16_t* vdst = rope.v_cache + ((size_t)page * rope.n_kv_heads + kvh) * hd * rope.page_size + in_page;
+      for (int i = lane; i < hd; i += AXON_WAVE) vdst[(size_t)i * rope.page_size] = float_to_bf16(value(slot * hd + i));
+      return;
+    }
+    dst = rope.k_cache + (((size_t)page * rope.n_kv_heads + (slot - rope.n_heads)) * rope.page_size + in_page) * hd;
+  }
+  const float* tab = rope.table + (size_t)m * half * 2;
+  for (int i = lane; i < half; i += AXON_WAVE) {
+    const float sn = tab[2 * i], cs = tab[2 * i + 1];
+    const float a = value(slot * hd + i), b = value(slot * hd + i + half);
+    dst[i] = float_to_bf16(__fsub_rn(__fmul_rn(a, cs), __fmul_rn(b, sn)));
+    dst[i + half] = float_to_bf16(__fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, cs)));
+  }
+}
+
+static int launch_split_reduce_rope(const float* partial, int splits, int m, int n, const void* bias, int bias_is_f32,
+                                    void* out, int out_stride, const RopeStore& rope, hipStream_t stream) {
+  const dim3 grid(m, ceil_div(n / rope.head_dim, 4));
+  gemm_split_reduce_rope_kernel<<<grid, 256, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, (bf16_t*)out, out_stride,
+                                                          rope);
+  AXK_LAUNCH_CHECK("gemm_split_reduce_rope");
+  return 0;
+}
 
 template <int NT16, int MT16, int WAVES, int DEPTH, int EPI>
 __global__ void __launch_bounds__(WAVES * 64)
@@ -902,9 +960,10 @@ int gemm_then_norm_ok(int m, int n, int k) {
          n <= SRN_MAX_N;
 }
 
-int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold_in,
-                     void* workspace, size_t workspace_bytes) {
+static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                              int out_stride, int m, int n, int k, int mode, hipStream_t stream,
+                              const GemmNormFold* fold_in, void* workspace, size_t workspace_bytes,
+                              const RopeStore* rope_after) {
   if (!gemm_pack_ok(mode == MODE_SWIGLU ? 2 * n : n, k, mode == MODE_SWIGLU)) {
     axk_set_error("gemm: N=%d K=%d is no shape of a packed matrix", n, k);
     return -1;
@@ -943,6 +1002,10 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
     norm = &after;
   }
   const int splits = splits_of(m, n, k, mode);
+  if (rope_after && (splits < 2 || mode != MODE_STORE)) {
+    axk_set_error("gemm: M=%d N=%d K=%d does not run with K split: the rotary kernel stays apart", m, n, k);
+    return -1;
+  }
   const size_t need = gemm_workspace_bytes(m, n, k, mode);
   if (need > workspace_bytes || (need > 0 && (workspace == nullptr || ((uintptr_t)workspace & 15)))) {
     axk_set_error("gemm: M=%d N=%d K=%d needs a workspace of %zu bytes, 16-byte aligned (got %zu)", m, n, k, need,
@@ -953,11 +1016,11 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
   if (m <= 256) {
     if (m > 64) {
       if (mode == MODE_SWIGLU) return launch_tile<128, 128, 2, 2, true>(ARGS, splits, ws);
-      return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws, norm);
+      return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws, norm, rope_after);
     }
     if (mode == MODE_SWIGLU) return launch_tile<64, 256, 1, 4, true, 64, 2>(ARGS, splits, ws);
-    if (n >= 8192) return launch_tile<64, 256, 1, 4, false, 64, 2>(ARGS, splits, ws, norm);
-    return launch_tile<64, 128, 1, 4, false, 64, 3>(ARGS, splits, ws, norm);
+    if (n >= 8192) return launch_tile<64, 256, 1, 4, false, 64, 2>(ARGS, splits, ws, norm, rope_after);
+    return launch_tile<64, 128, 1, 4, false, 64, 3>(ARGS, splits, ws, norm, rope_after);
   }
   // 256 x 256 tiles (8 waves) where they fill the chip: one round of at least 140 blocks (on 256
   // CUs), or several rounds of which the last is not mostly idle; else 128 x 128 tiles, four times
@@ -975,26 +1038,40 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
   // product, three quarters of the products per block).  The k order of a sum is the same.
   if (use_big && splits == 1 && big <= 192 && n % 192 == 0 && (long)ceil_div(m, 256) * (n / 192) <= 256)
     return launch_tile<256, 192, 4, 2, false>(ARGS, splits, ws, norm);
-  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS, splits, ws, norm);
-  return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws, norm);
+  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS, splits, ws, norm, rope_after);
+  return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws, norm, rope_after);
 #undef ARGS
 }
 
-// The [q; k; v] product with rotary encoding and cache store (see RopeStore): up to 16 rows
-// (what gemm_skinny takes), every head rotated over its whole width, halves of a head a
-// multiple of 16 wide.
-int gemm_qkv_rope_ok(int m, int k, int head_dim, int rotary_dim) {
-  return m >= 1 && m <= 16 && k % 64 == 0 && rotary_dim == head_dim && head_dim % 32 == 0;
+int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold_in,
+                     void* workspace, size_t workspace_bytes) {
+  return gemm_mfma_dispatch(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, fold_in, workspace,
+                            workspace_bytes, nullptr);
+}
+
+// The [q; k; v] product with rotary encoding and cache store (see RopeStore): up to 16 rows in
+// the epilogue of gemm_skinny, more rows where the product splits K (then the kernel that adds
+// the parts' sums rotates and stores); every head rotated over its whole width, halves of a head
+// a multiple of 16 wide.
+int gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotary_dim) {
+  if (m < 1 || k % 64 != 0 || rotary_dim != head_dim || head_dim % 32 != 0 || n % head_dim != 0) return 0;
+  if (m <= 16) return 1;
+  return gemm_pack_ok(n, k, 0) && n % 4 == 0 && splits_of(m, n, k, MODE_STORE) > 1;
 }
 
 int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out,
                          int out_stride, int m, int n, int k, const float* in_squares, float in_eps,
                          const float* table, const int32_t* positions, const int32_t* seq_rows,
                          const int32_t* block_table, int table_stride, bf16_t* k_cache, bf16_t* v_cache, int n_heads,
-                         int n_kv_heads, int head_dim, int page_size, hipStream_t stream) {
+                         int n_kv_heads, int head_dim, int page_size, void* workspace, size_t workspace_bytes,
+                         hipStream_t stream) {
   const NormFold fold = {in_squares, in_eps, nullptr, 0, nullptr, nullptr};
   const RopeStore rope = {table, positions, seq_rows, block_table, table_stride, k_cache, v_cache,
                           n_heads, n_kv_heads, head_dim, page_size};
+  if (m > 16)
+    return gemm_mfma_dispatch(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream, nullptr,
+                              workspace, workspace_bytes, &rope);
 #define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream, fold, rope
   return launch_skinny<2, 1, 4, 8, EPI_ROPE>(ARGS);
 #undef ARGS

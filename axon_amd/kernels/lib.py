@@ -36,10 +36,10 @@ _SIGNATURES = {
     "axk_rope_table": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_rope_kv_write": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "axk_gemm_qkv_rope_ok": [c_int, c_int, c_int, c_int],
+    "axk_gemm_qkv_rope_ok": [c_int, c_int, c_int, c_int, c_int],
     "axk_gemm_qkv_rope": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_float,
                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_int, c_void_p],
+                          c_int, c_void_p, ctypes.c_long, c_void_p],
     "axk_attention": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
                       c_int, c_int, c_int, c_int, c_float, c_void_p],
     "axk_attention_prefill": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
@@ -214,13 +214,14 @@ class Kernels:
             _ptr(k_cache if write_kv else None), _ptr(v_cache if write_kv else None), T, n_heads, n_kv_heads, head_dim,
             rotary_dim, page_size, 1 if write_kv else 0, _stream()))
 
-    def gemm_qkv_rope_ok(self, m: int, k: int, head_dim: int, rotary_dim: int) -> bool:
-        """Whether `gemm_qkv_rope` takes a step of m tokens and these sizes."""
-        return bool(self.lib.axk_gemm_qkv_rope_ok(m, k, head_dim, rotary_dim))
+    def gemm_qkv_rope_ok(self, m: int, n: int, k: int, head_dim: int, rotary_dim: int) -> bool:
+        """Whether `gemm_qkv_rope` takes a step of m tokens and a matrix of n rows of these sizes."""
+        return bool(self.lib.axk_gemm_qkv_rope_ok(m, n, k, head_dim, rotary_dim))
 
     def gemm_qkv_rope(self, x, w, bias, qkv, table, positions, seq_rows, block_table, k_cache, v_cache, n_heads,
                       n_kv_heads, head_dim, page_size, write_kv=True, row_squares=None, eps=0.0) -> None:
-        """The [q; k; v] product, the rotary encoding and the store into the pages in one launch:
+        """The [q; k; v] product, the rotary encoding and the store into the pages in one launch
+        (up to 16 tokens) or with the kernel that adds a split product's parts doing the rest:
         the same bits as `gemm` into qkv followed by `rope_kv_write`.  q lands in qkv[:, :n_heads *
         head_dim]; the k and v columns of qkv are not written.  Without write_kv, w holds the q
         rows only.  row_squares, eps: as in `gemm`."""
@@ -243,11 +244,13 @@ class Kernels:
             raise KernelError(f"gemm_qkv_rope: row_squares {tuple(row_squares.shape)} is not float32 [{M}, {K // 16}]")
         if write_kv:
             self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
+        need = self.lib.axk_gemm_workspace(M, rows, K, MODE_STORE)
+        work = torch.empty(need // 4, dtype=torch.float32, device=x.device) if need > 0 else None
         self._check(self.lib.axk_gemm_qkv_rope(
             _ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "qkv bias"), _ptr(qkv), qkv.stride(0), M, K,
             _ptr(row_squares), float(eps), _ptr(table), _ptr(positions), _ptr(seq_rows), _ptr(block_table),
             block_table.shape[-1], _ptr(k_cache if write_kv else None), _ptr(v_cache if write_kv else None), n_heads,
-            n_kv_heads, head_dim, page_size, 1 if write_kv else 0, _stream()))
+            n_kv_heads, head_dim, page_size, 1 if write_kv else 0, _ptr(work), need, _stream()))
 
     def attention(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, n_heads, n_kv_heads,
                   head_dim, page_size, window, scale) -> torch.Tensor:

@@ -220,8 +220,9 @@ class GQAttention(Mixer):
         else:
             # reading another run's cache: only the queries are needed
             w, bias = self.w_qkv[:self.q_dim], None if self.b_qkv is None else self.b_qkv[:self.q_dim]
-        if isinstance(w, PackedMatrix) and k.gemm_qkv_rope_ok(T, self.hidden, self.hd, rotary):
-            # a short step: product, rotation and the store into the pages in one launch
+        if isinstance(w, PackedMatrix) and k.gemm_qkv_rope_ok(T, w.shape[0], self.hidden, self.hd, rotary):
+            # product, rotation and the store into the pages in one launch (a short step) or with the
+            # rotation and the store done by the kernel that adds a split product's parts
             k.gemm_qkv_rope(h, w, bias, qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache,
                             self.nh, self.nkv, self.hd, group.page_size, binding.writes, **scaled)
         else:

@@ -303,15 +303,17 @@ def test_gemm_with_a_norm_folded_in(M, H, F):
 
 @pytest.mark.parametrize("M,nh,nkv,hd,hidden,page", [(1, 4, 2, 32, 64, 8), (8, 6, 2, 64, 192, 16), (16, 7, 1, 128, 256, 8),
                                                       (13, 3, 3, 96, 128, 4), (5, 4, 1, 64, 320, 32),
-                                                      (16, 2, 2, 128, 64, 16)])
+                                                      (16, 2, 2, 128, 64, 16), (40, 6, 2, 64, 512, 16),
+                                                      (100, 7, 1, 128, 1024, 8), (300, 4, 2, 64, 3072, 16)])
 def test_qkv_product_with_rotation_and_cache_store_in_one(M, nh, nkv, hd, hidden, page):
     """The fused launch against the product followed by the rotary kernel: the same bits in q, in
     the pages of keys and in the pages of values; other pages untouched."""
     k = kernels("bfloat16")
-    assert k.gemm_qkv_rope_ok(M, hidden, hd, hd)
-    assert not k.gemm_qkv_rope_ok(M, hidden, hd, hd // 2) and not k.gemm_qkv_rope_ok(17, hidden, hd, hd)
-    assert not k.gemm_qkv_rope_ok(M, hidden, 48, 48) and not kernels("float32").gemm_qkv_rope_ok(M, hidden, hd, hd)
     width = (nh + 2 * nkv) * hd
+    assert k.gemm_qkv_rope_ok(M, width, hidden, hd, hd) and k.gemm_qkv_rope_ok(M, nh * hd, hidden, hd, hd)
+    assert not k.gemm_qkv_rope_ok(M, width, hidden, hd, hd // 2) and not k.gemm_qkv_rope_ok(17, width, 64, hd, hd)
+    assert not k.gemm_qkv_rope_ok(M, 48 * (nh + 2 * nkv), hidden, 48, 48)
+    assert not kernels("float32").gemm_qkv_rope_ok(M, width, hidden, hd, hd)
     x, _ = as_dtype(rnd(M, hidden, seed=50), "bfloat16")
     w, _ = as_dtype(rnd(width, hidden, seed=51, scale=0.2), "bfloat16")
     g = torch.Generator().manual_seed(52)
