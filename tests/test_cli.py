@@ -40,3 +40,12 @@ def test_info_and_random_weights(tmp_path):
     assert "cache group: 3 layers x 2 x 1 heads x 32" in r.stdout
     r = run("--help")
     assert r.returncode == 0 and "gen" in r.stdout and "logits" in r.stdout
+
+
+def test_the_benchmark_refuses_more_than_one_gpu():
+    """bench.py runs on one GPU: asked for more it says so in one line and exits with 2, before
+    anything touches a device."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2
+    assert len(r.stdout.strip().splitlines()) == 1 and "one GPU" in r.stdout
