@@ -33,10 +33,11 @@ def full_layer(tmp_path_factory):
     return d, prompts, oracle
 
 
-@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
-def test_a_layer_of_the_measured_sizes_through_every_class_of_rows(dtype, full_layer):
+@pytest.mark.parametrize("dtype,page", [("bfloat16", 16), ("bfloat16", 64), ("bfloat16", 8), ("float32", 16)])
+def test_a_layer_of_the_measured_sizes_through_every_class_of_rows(dtype, page, full_layer):
     d, prompts, oracle = full_layer
-    llm = axon_amd.load(d, dtype=dtype, page_size=16, num_pages=64, max_seqs=4, max_batch_tokens=512)
+    n_pages = 1024 // page + 4
+    llm = axon_amd.load(d, dtype=dtype, page_size=page, num_pages=n_pages, max_seqs=4, max_batch_tokens=512)
     eng = llm.engine
     fed = {rid: 0 for rid in prompts}
     worst = 0.0
@@ -73,4 +74,4 @@ def test_a_layer_of_the_measured_sizes_through_every_class_of_rows(dtype, full_l
     assert fed == {"a": 620, "b": 150, "c": 61}
     eng.release_all()
     eng.cache.check()
-    assert eng.cache.free_pages() == 64
+    assert eng.cache.free_pages() == n_pages
