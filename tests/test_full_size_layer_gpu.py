@@ -1,4 +1,4 @@
-"""One layer of the sizes the engine is measured at (width 3584, 28 query heads on 4 kv heads of
+"""One layer of the sizes the engine is measured at, and one of the next size up (width 3584, 28 query heads on 4 kv heads of
 128, feed-forward 18944) with a small vocabulary, against the plain implementation: the tiny
 configurations of the other tests never meet the kernels that these widths select (products
 that split K between blocks, norms finished by the product before them, the prompt kernel with
@@ -21,21 +21,43 @@ FULL = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=1, hidden_size
             rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
 
 
-@pytest.fixture(scope="module")
-def full_layer(tmp_path_factory):
-    d = str(tmp_path_factory.mktemp("full_layer"))
-    write_random_model(config_from_dict(FULL), d, seed=31, std=0.02, storage="bfloat16")
+# the layer of the next size up: another width, a group of 5 query heads, other feed-forward width
+WIDER = dict(FULL, hidden_size=5120, intermediate_size=13824, num_attention_heads=40, num_key_value_heads=8,
+             rms_norm_eps=1e-5)
+
+
+def _layer_case(tmp_path_factory, sizes, name):
+    d = str(tmp_path_factory.mktemp(name))
+    write_random_model(config_from_dict(sizes), d, seed=31, std=0.02, storage="bfloat16")
     cfg, w = P.load_plain(d)
     g = torch.Generator().manual_seed(2)
-    prompts = {rid: torch.randint(0, FULL["vocab_size"], (n,), generator=g).tolist()
+    prompts = {rid: torch.randint(0, sizes["vocab_size"], (n,), generator=g).tolist()
                for rid, n in (("a", 620), ("b", 150), ("c", 61))}
     oracle = {rid: P.forward_logits(cfg, w, toks) for rid, toks in prompts.items()}
     return d, prompts, oracle
 
 
+@pytest.fixture(scope="module")
+def full_layer(tmp_path_factory):
+    return _layer_case(tmp_path_factory, FULL, "full_layer")
+
+
+@pytest.fixture(scope="module")
+def wider_layer(tmp_path_factory):
+    return _layer_case(tmp_path_factory, WIDER, "wider_layer")
+
+
 @pytest.mark.parametrize("dtype,page", [("bfloat16", 16), ("bfloat16", 64), ("bfloat16", 8), ("float32", 16)])
 def test_a_layer_of_the_measured_sizes_through_every_class_of_rows(dtype, page, full_layer):
-    d, prompts, oracle = full_layer
+    _through_every_class_of_rows(dtype, page, full_layer)
+
+
+def test_a_layer_of_the_next_size_through_every_class_of_rows(wider_layer):
+    _through_every_class_of_rows("bfloat16", 16, wider_layer)
+
+
+def _through_every_class_of_rows(dtype, page, case):
+    d, prompts, oracle = case
     n_pages = 1024 // page + 4
     llm = axon_amd.load(d, dtype=dtype, page_size=page, num_pages=n_pages, max_seqs=4, max_batch_tokens=512)
     eng = llm.engine
