@@ -1,9 +1,10 @@
-"""One layer of the sizes the engine is measured at, and one of the next size up (width 3584, 28 query heads on 4 kv heads of
-128, feed-forward 18944) with a small vocabulary, against the plain implementation: the tiny
-configurations of the other tests never meet the kernels that these widths select (products
-that split K between blocks, norms finished by the product before them, the prompt kernel with
-two heads a block and a group of 7, decoding over several chunks).  A mixed schedule takes
-every product through each of its classes of rows (up to 16, 64, 256, more)."""
+"""One layer of the sizes the engine is measured at (width 3584, 28 query heads on 4 kv heads of
+128, feed-forward 18944) and one of the next size up (width 5120, 40 heads on 8, feed-forward
+13824), with a small vocabulary, against the plain implementation: the tiny configurations of
+the other tests never meet the kernels that these widths select (products that split K between
+blocks, norms finished by the product before them, the prompt kernel with a group of 7 or 5,
+decoding over several chunks).  A mixed schedule takes every product through each of its
+classes of rows (up to 16, 64, 256, more)."""
 import pytest
 import torch
 
