@@ -155,6 +155,17 @@ long axk_argmax_workspace(int n_rows, int n);
 int axk_argmax(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n, void* workspace,
                void* stream);
 
+// axk_argmax without a workspace.  This entry point has no counterpart in the reference: it is
+// for callers that cannot allocate or pass device memory beyond inputs and outputs (code under
+// HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The chunks' keys go
+// through an array of the library's own, 128 KB on every GPU it runs on, for up to
+// axk_argmax_static_max_rows() rows of up to axk_argmax_static_max_n() logits; more is refused.
+// It allocates nothing and frees nothing.  Calls on one GPU share the array: calls that overlap
+// there (different streams or threads) race; calls on one stream are ordered and safe.
+int axk_argmax_static_max_rows(void);
+int axk_argmax_static_max_n(void);
+int axk_argmax_static(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n, void* stream);
+
 // Repeat penalty on `recent` ids, then the k best as 64-bit keys (order key of the logit <<
 // 32 | id), unsorted, into cands[r, 0..k); the penalty is applied to `logits` in place.  recent is [n_rows, recent_stride] with
 // n_recent[r] valid ids each; penalty 1 or n_recent 0: off.  k <= 1024.

@@ -6,6 +6,8 @@
 // larger id wins.  The largest key is the greedy pick: of equal maxima the last index, NaN
 // never, all NaN gives n - 1 (src/generate.rs:222-264).  Keys are distinct, so selection is
 // exact and has no order-dependent step: integer histograms only.
+#include <mutex>
+
 #include "api.h"
 #include "common.h"
 
@@ -188,5 +190,68 @@ extern "C" int axk_topk(float* logits, int logits_stride, const int32_t* recent,
   topk_kernel<<<n_rows, PICK_THREADS, 0, (hipStream_t)stream>>>(logits, logits_stride, recent, recent_stride,
                                                                n_recent, penalty, k_of_row, cands, cands_stride, n);
   AXK_LAUNCH_CHECK("topk");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------- argmax without a workspace
+// axk_argmax_static: axk_argmax for callers that cannot allocate or bring device memory beyond
+// their inputs and outputs.  The chunks' best keys (what axk_argmax keeps in the caller's
+// workspace) live in an array of the library's own, ARGMAX_STATIC_ROWS x ARGMAX_STATIC_CHUNKS
+// keys = 128 KB that every GPU the library runs on holds until the process ends.  In host code
+// the array's name is only a stand-in: the address on the current GPU comes from
+// hipGetSymbolAddress, asked once per device, and that pointer is what the kernels are given.
+// Nothing has to start at zero: the first launch writes every key the second reads.  All calls
+// on one GPU share the array, so calls that overlap there (two streams, two threads) race.
+#define ARGMAX_STATIC_ROWS 256
+#define ARGMAX_STATIC_CHUNKS 64
+#define ARGMAX_STATIC_DEVICES 64
+
+static __device__ __align__(256) uint64_t argmax_scratch[ARGMAX_STATIC_ROWS * ARGMAX_STATIC_CHUNKS];
+static uint64_t* argmax_scratch_at[ARGMAX_STATIC_DEVICES];     // per device; written once, under the lock
+static std::mutex argmax_scratch_lock;
+
+static int argmax_scratch_of_device(uint64_t** at) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess || device < 0 || device >= ARGMAX_STATIC_DEVICES) {
+    axk_set_error("argmax_static: no current device (%s, device %d)", hipGetErrorString(e), device);
+    return -2;
+  }
+  std::lock_guard<std::mutex> hold(argmax_scratch_lock);
+  if (argmax_scratch_at[device] == nullptr) {
+    uint64_t* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(argmax_scratch));
+    if (e != hipSuccess || p == nullptr) {
+      axk_set_error("argmax_static: the address of the scratch array on device %d: %s", device, hipGetErrorString(e));
+      return -2;
+    }
+    argmax_scratch_at[device] = p;
+  }
+  *at = argmax_scratch_at[device];
+  return 0;
+}
+
+extern "C" int axk_argmax_static_max_rows(void) { return ARGMAX_STATIC_ROWS; }
+extern "C" int axk_argmax_static_max_n(void) { return ARGMAX_STATIC_CHUNKS * ARGMAX_CHUNK; }
+
+extern "C" int axk_argmax_static(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n,
+                                 void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && n > 0 && logits_stride >= n, "argmax_static: bad sizes rows=%d n=%d stride=%d", n_rows, n,
+              logits_stride);
+  AXK_REQUIRE(n_rows <= ARGMAX_STATIC_ROWS && n <= ARGMAX_STATIC_CHUNKS * ARGMAX_CHUNK,
+              "argmax_static: %d rows of %d logits; the library's own scratch takes up to %d rows of %d", n_rows, n,
+              ARGMAX_STATIC_ROWS, ARGMAX_STATIC_CHUNKS * ARGMAX_CHUNK);
+  AXK_REQUIRE(logits != nullptr && picks != nullptr, "argmax_static: logits or picks missing");
+  if (n_rows == 0) return 0;
+  uint64_t* scratch = nullptr;
+  const int rc = argmax_scratch_of_device(&scratch);
+  if (rc != 0) return rc;
+  const int n_chunks = ceil_div(n, ARGMAX_CHUNK);
+  const int vec = logits_stride % 4 == 0 && ((uintptr_t)logits & 15) == 0;
+  argmax_chunk_kernel<<<dim3(n_chunks, n_rows), ARGMAX_THREADS, 0, (hipStream_t)stream>>>(logits, logits_stride,
+                                                                                         scratch, n, vec);
+  AXK_LAUNCH_CHECK("argmax_chunk");
+  argmax_rows_kernel<<<n_rows, AXON_WAVE, 0, (hipStream_t)stream>>>(scratch, n_chunks, picks);
+  AXK_LAUNCH_CHECK("argmax_rows");
   return 0;
 }
