@@ -59,11 +59,14 @@ int axk_attention(const void* q, int q_stride, const void* k_cache, const void* 
 // every block about the same work.
 // axk_attention_decode: token_index [n_tokens] names single tokens (null: the first n_tokens
 // tokens of the step); a token's range (from the chunk that holds the window's first position,
-// or 0) is cut into chunks of axk_attention_decode_chunk positions.  work [n_work] lists the
-// chunks to compute, item = slot in token_index * axk_attention_decode_item_factor + chunk, or
-// -1 for none: every chunk of every token once.  With more than one chunk the partial results go
-// through `partial` (axk_attention_decode_workspace floats) and are folded in ascending order;
-// max_chunks is the most chunks any of the tokens has.
+// or 0) is cut into chunks of axk_attention_decode_chunk positions, four blocks of 64 each.
+// work [n_work] lists the chunks to compute, item = slot in token_index *
+// axk_attention_decode_item_factor + chunk, or -1 for none: every chunk of every token once.  The
+// blocks' results go through `partial` (axk_attention_decode_workspace floats) and a second launch
+// folds them in ascending order; max_chunks is the most chunks any of the tokens has.
+// Both kernels compute the same arithmetic (blocks of 64 positions aligned to absolute position,
+// each with its own maximum, folded ascending): a position's result is bit for bit the same from
+// either, alone or in any batch.
 int axk_attention_fast_ok(int head_dim, int page_size, int n_heads, int n_kv_heads);
 int axk_attention_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                           const int32_t* block_table, int table_stride, const int32_t* positions,
@@ -92,38 +95,27 @@ int axk_pack_matrix(const void* src, void* dst, int rows, int k, void* stream);
 // float32 [M, N] (the residual stream); 2: store float32 [M, N] (logits); 3: W holds 2 N rows,
 // gate rows then up rows, and out elem [M, N] = silu(X . gate^T) * (X . up^T) (no bias).
 // x_stride / out_stride: elements between rows.  workspace: axk_gemm_workspace(m, n, k, mode) bytes
-// (0 for most shapes: then it may be null), 16-byte aligned; products of 17 to 2048 rows may split K
-// between blocks and add the blocks' sums through it.
+// (0 for most shapes: then it may be null), 16-byte aligned; products of more than 64 rows with a
+// narrow output give each segment of K blocks of their own and add the segments' sums through it.
+//
+// With a packed W every output element is the sum, in ascending order, of axk_gemm_segments(n, k,
+// gated) chains of 32x32x16 MFMAs over contiguous segments of K: the bits of a row do not depend on
+// M, that is, on what else is in the batch.
 long axk_gemm_workspace(int m, int n, int k, int mode);
+int axk_gemm_segments(int n, int k, int gated);
 int axk_gemm(const void* x, int x_stride, const void* w, int w_packed, const void* bias, int bias_is_f32, void* out,
              int out_stride, int m, int n, int k, int mode, void* workspace, long workspace_bytes, void* stream);
 
-// The same product with an RMS norm folded into it on either side, so that the norm needs no
-// pass of its own (bfloat16 build, W packed, shapes for which axk_gemm_norm_fold_ok says 1):
-// * in_squares [M, K / 16] (or null): X holds x * gain without the row's scale and in_squares
-//   the sums of x^2 over the 16-column parts of each row; the product's result is multiplied
-//   by 1 / sqrt(sum(in_squares[m]) / K + in_eps) before the bias is added.
-// * norm_gain (or null; mode 1 only): beside out += result, norm_values elem [M, N] =
-//   out * norm_gain and norm_squares [M, ceil(N / 16)] = sums of out^2 over 16 columns each:
-//   what the in_squares side of the next product takes.
 typedef struct {
-  const float* in_squares;
-  float in_eps;
   const void* norm_gain;
   int norm_gain_is_f32;
   void* norm_values;
-  float* norm_squares;
-  float norm_eps;      // of the whole norm behind a split product (axk_gemm_then_norm)
-} GemmNormFold;
-int axk_gemm_norm_fold_ok(int m, int n, int k, int mode);
-int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* out,
-                       int out_stride, int m, int n, int k, int mode, const float* in_squares, float in_eps,
-                       const void* norm_gain, int norm_gain_is_f32, void* norm_values, float* norm_squares,
-                       void* stream);
+  float norm_eps;
+} GemmNormFold;     // the norm behind a product (axk_gemm_then_norm)
 
 // The product that adds into float32 rows (mode 1, W packed) followed by the RMS norm of the new
-// rows, for shapes that run with K split between blocks (axk_gemm_then_norm_ok says 1): the
-// kernel that adds the blocks' sums also writes norm_values elem [M, N] =
+// rows, for shapes that run with a block per segment of K (axk_gemm_then_norm_ok says 1): the
+// kernel that adds the segments' sums also writes norm_values elem [M, N] =
 // out / sqrt(mean(out^2) + norm_eps) * norm_gain.  Bit-identical to axk_gemm followed by
 // axk_rmsnorm.  workspace: axk_gemm_workspace bytes, as for axk_gemm.
 int axk_gemm_then_norm_ok(int m, int n, int k);
@@ -134,17 +126,17 @@ int axk_gemm_then_norm(const void* x, int x_stride, const void* w, const void* b
 // The attention's [q; k; v] product (W packed, [(n_heads + 2 n_kv_heads) head_dim, K], or the q rows alone
 // if write_kv is 0) with what follows it in the same launches: bias, the rotary encoding of q and k
 // heads over their whole width (table [M, head_dim / 2, 2]: sin, cos), q into qkv [M, >= n_heads
-// head_dim], k and v into the request's pages (as axk_rope_kv_write stores them).  Up to 16 rows it
-// is the product's epilogue (in_squares as in axk_gemm_norm_fold, or null); with more rows, where
-// the product splits K (axk_gemm_qkv_rope_ok says so; n = the rows of W), the kernel that adds the
-// parts' sums rotates and stores; workspace: axk_gemm_workspace(m, n, k, 0) bytes.  Bit-identical
-// to axk_gemm followed by axk_rope_kv_write.
+// head_dim], k and v into the request's pages (as axk_rope_kv_write stores them).  Up to 64 rows it
+// is the product's epilogue; with more rows, where the product runs with a block per segment of K
+// (axk_gemm_qkv_rope_ok says so; n = the rows of W), the kernel that adds the segments' sums rotates
+// and stores; workspace: axk_gemm_workspace(m, n, k, 0) bytes.  Bit-identical to axk_gemm followed
+// by axk_rope_kv_write.
 int axk_gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotary_dim);
 int axk_gemm_qkv_rope(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32, void* qkv,
-                      int qkv_stride, int m, int k, const float* in_squares, float in_eps, const float* table,
-                      const int32_t* positions, const int32_t* seq_rows, const int32_t* block_table, int table_stride,
-                      void* k_cache, void* v_cache, int n_heads, int n_kv_heads, int head_dim, int page_size,
-                      int write_kv, void* workspace, long workspace_bytes, void* stream);
+                      int qkv_stride, int m, int k, const float* table, const int32_t* positions,
+                      const int32_t* seq_rows, const int32_t* block_table, int table_stride, void* k_cache,
+                      void* v_cache, int n_heads, int n_kv_heads, int head_dim, int page_size, int write_kv,
+                      void* workspace, long workspace_bytes, void* stream);
 
 // out[t, f] = silu(gu[t, f]) * gu[t, F + f]: gate in the first F columns, up in the last.
 int axk_swiglu(const void* gate_up, void* out, int n_tokens, int n_ffn, void* stream);

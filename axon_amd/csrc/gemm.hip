@@ -144,20 +144,19 @@ static int launch_fma(const elem_t* x, int x_stride, const elem_t* w, const void
 
 #if AXON_BF16
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold,
+                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* then_norm,
                      void* workspace, size_t workspace_bytes);
 int gemm_pack_ok(int rows, int k, int gated);
 int launch_pack_matrix(const bf16_t* src, bf16_t* dst, int rows, int k, hipStream_t stream);
 size_t gemm_workspace_bytes(int m, int n, int k, int mode);
-int gemm_norm_fold_ok(int m, int n, int k, int mode);
+int gemm_segments(int tiles32, int k);
 int gemm_then_norm_ok(int m, int n, int k);
 int gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotary_dim);
 int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out,
-                         int out_stride, int m, int n, int k, const float* in_squares, float in_eps,
-                         const float* table, const int32_t* positions, const int32_t* seq_rows,
-                         const int32_t* block_table, int table_stride, bf16_t* k_cache, bf16_t* v_cache, int n_heads,
-                         int n_kv_heads, int head_dim, int page_size, void* workspace, size_t workspace_bytes,
-                         hipStream_t stream);
+                         int out_stride, int m, int n, int k, const float* table, const int32_t* positions,
+                         const int32_t* seq_rows, const int32_t* block_table, int table_stride, bf16_t* k_cache,
+                         bf16_t* v_cache, int n_heads, int n_kv_heads, int head_dim, int page_size, void* workspace,
+                         size_t workspace_bytes, hipStream_t stream);
 #endif
 
 static int gemm_checked(const void* x, int x_stride, const void* w, int w_packed, const void* bias, int bias_is_f32,
@@ -179,7 +178,7 @@ static int gemm_checked(const void* x, int x_stride, const void* w, int w_packed
     return -1;
 #endif
   }
-  AXK_REQUIRE(fold == nullptr, "gemm: a norm is folded only into products with a packed matrix");
+  AXK_REQUIRE(fold == nullptr, "gemm: a norm follows only products with a packed matrix");
   return launch_fma((const elem_t*)x, x_stride, (const elem_t*)w, bias, bias_is_f32, out, out_stride, m, n, k, mode,
                     (hipStream_t)stream);
 }
@@ -220,25 +219,15 @@ extern "C" int axk_pack_matrix(const void* src, void* dst, int rows, int k, void
 #endif
 }
 
-extern "C" int axk_gemm_norm_fold_ok(int m, int n, int k, int mode) {
+// Segments K is cut into for a packed [n, k] matrix (gated: n is the width of the output, the
+// matrix holds 2 n rows): the order of addition of every product with it.  1 where nothing is packed.
+extern "C" int axk_gemm_segments(int n, int k, int gated) {
 #if AXON_BF16
-  return m >= 0 && n > 0 && k > 0 && gemm_norm_fold_ok(m, n, k, mode);
+  if (n <= 0 || k <= 0 || !gemm_pack_ok(gated ? 2 * n : n, k, gated)) return 1;
+  return gemm_segments(gated ? n / 16 : (n + 31) / 32, k);
 #else
-  return 0;   // the 32-bit build keeps the norm a pass of its own
+  return 1;
 #endif
-}
-
-extern "C" int axk_gemm_norm_fold(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32,
-                                  void* out, int out_stride, int m, int n, int k, int mode, const float* in_squares,
-                                  float in_eps, const void* norm_gain, int norm_gain_is_f32, void* norm_values,
-                                  float* norm_squares, void* stream) {
-  AXK_REQUIRE(axk_gemm_norm_fold_ok(m, n, k, mode), "gemm: no kernel folds a norm into M=%d N=%d K=%d mode %d", m, n, k,
-              mode);
-  AXK_REQUIRE(norm_gain == nullptr || (mode == MODE_ADD_F32 && norm_values && norm_squares),
-              "gemm: the following norm needs the add-into-residual epilogue and both of its outputs");
-  AXK_REQUIRE(((uintptr_t)in_squares & 15) == 0, "gemm: the rows' sums of squares must be 16-byte aligned");
-  const GemmNormFold fold = {in_squares, in_eps, norm_gain, norm_gain_is_f32, norm_values, norm_squares, 0.0f};
-  return gemm_checked(x, x_stride, w, 1, bias, bias_is_f32, out, out_stride, m, n, k, mode, &fold, nullptr, 0, stream);
 }
 
 extern "C" int axk_gemm_then_norm_ok(int m, int n, int k) {
@@ -259,7 +248,7 @@ extern "C" int axk_gemm_then_norm(const void* x, int x_stride, const void* w, co
   AXK_REQUIRE(out_stride % 4 == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)norm_values & 7) == 0,
               "gemm: the rows to add into must be 16-byte aligned (stride %d) and the norm's output 8-byte aligned",
               out_stride);
-  const GemmNormFold fold = {nullptr, 0.0f, norm_gain, norm_gain_is_f32, norm_values, nullptr, norm_eps};
+  const GemmNormFold fold = {norm_gain, norm_gain_is_f32, norm_values, norm_eps};
   return gemm_checked(x, x_stride, w, 1, bias, bias_is_f32, out, out_stride, m, n, k, MODE_ADD_F32, &fold, workspace,
                       workspace_bytes, stream);
 }
@@ -273,8 +262,7 @@ extern "C" int axk_gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotar
 }
 
 extern "C" int axk_gemm_qkv_rope(const void* x, int x_stride, const void* w, const void* bias, int bias_is_f32,
-                                 void* qkv, int qkv_stride, int m, int k, const float* in_squares, float in_eps,
-                                 const float* table, const int32_t* positions, const int32_t* seq_rows,
+                                 void* qkv, int qkv_stride, int m, int k, const float* table, const int32_t* positions, const int32_t* seq_rows,
                                  const int32_t* block_table, int table_stride, void* k_cache, void* v_cache,
                                  int n_heads, int n_kv_heads, int head_dim, int page_size, int write_kv, void* workspace,
                                  long workspace_bytes, void* stream) {
@@ -286,14 +274,12 @@ extern "C" int axk_gemm_qkv_rope(const void* x, int x_stride, const void* w, con
               m, n, k, head_dim);
   AXK_REQUIRE(x_stride >= k && x_stride % 8 == 0 && qkv_stride >= n_heads * head_dim && qkv_stride % 4 == 0 &&
                   ((uintptr_t)x & 15) == 0 && ((uintptr_t)w & 15) == 0 && ((uintptr_t)qkv & 7) == 0 &&
-                  ((uintptr_t)table & 15) == 0 && ((uintptr_t)in_squares & 15) == 0,
+                  ((uintptr_t)table & 15) == 0,
               "gemm_qkv_rope: strides x=%d qkv=%d or the alignment of an operand are not taken", x_stride, qkv_stride);
-  AXK_REQUIRE(in_squares == nullptr || (m <= 16 && axk_gemm_norm_fold_ok(m, n, k, MODE_STORE)),
-              "gemm_qkv_rope: no norm is folded into a step of %d rows", m);
   AXK_REQUIRE(table && positions && (!write_kv || (seq_rows && block_table && k_cache && v_cache)),
               "gemm_qkv_rope: a table, the positions or the cache is missing");
   return launch_gemm_qkv_rope((const bf16_t*)x, x_stride, (const bf16_t*)w, bias, bias_is_f32, (bf16_t*)qkv, qkv_stride,
-                              m, n, k, in_squares, in_eps, table, positions, seq_rows, block_table, table_stride,
+                              m, n, k, table, positions, seq_rows, block_table, table_stride,
                               (bf16_t*)k_cache, (bf16_t*)v_cache, n_heads, n_kv_heads, head_dim, page_size, workspace,
                               workspace_bytes > 0 ? (size_t)workspace_bytes : 0, (hipStream_t)stream);
 #else

@@ -4,35 +4,37 @@
 // W is PACKED (axk_pack_matrix, once, when the weights are loaded): blocks of 16 rows x 32 k, each
 // 1 KB in the order in which a wave holds them as an MFMA operand (lane l: row l % 16, the 8
 // consecutive k from 8 (l / 16)); blocks ordered [row tile][k block]; rows padded to a multiple
-// of 16 with zeros.  A wave instruction then reads 1 KB of consecutive memory (measured: 10 to 35 %
-// more bandwidth than 16 rows x 64 bytes of a row-major matrix), lands in LDS without a
-// permutation, and the same bytes serve the 16x16x32 and the 32x32x16 MFMA.
+// of 16 with zeros.  A wave instruction then reads whole kilobytes of consecutive memory, the
+// blocks land in LDS without a permutation, and the same bytes serve every kernel here.
 //
-// Two kernels, chosen by the number of rows M alone, so that a given (N, K) always meets the same
-// kernel and the same grouping of k for a given class of M:
+// ONE ORDER OF ADDITION PER MATRIX.  Every output element of a product with a given W is
+//     ((c_0 + c_1) + c_2) + ... + c_(S-1),   then the bias and the epilogue,
+// where K is cut into S = gemm_segments(W's row tiles, K) contiguous segments (by the matrix
+// alone, never by the number of rows M of X), and c_s is one chain of 32x32x16 MFMAs over
+// the segment's k in ascending steps of 16, starting from zero.  Every kernel below computes
+// exactly this, whatever its tiles, its number of waves or the way it spreads the segments over
+// waves, blocks or registers: a row of X gives the same bits whether it comes alone, among 16
+// rows or among 4,096 (src/lm.rs:272-278 asks this of a step; the reference's integer products
+// get it from exact block sums, src/cuda/decode.cu:352-369).  The kernels are chosen by M, for
+// speed alone:
 //
-// * gemm_skinny (M <= 16, decoding): bound by reading W once.  A block owns one or two row tiles
-//   of W; its four waves split K between them and stream their share from memory straight into
-//   MFMA operands (16x16x32), keeping a ring of steps in flight so that the memory pipe never
-//   drains; each multiplies with up to 16 rows of X, and the waves' sums are added in wave
-//   order through LDS.  No atomics, so the result does not depend on timing.  Epilogues: bias /
-//   residual add / SwiGLU, an RMS norm folded in on either side, and the attention's qkv product
-//   with the rotary encoding and the store into the paged cache.
+// * gemm_stream (M <= 64): bound by reading W once.  A wave owns 32 rows of W and one segment of
+//   K and streams its share from memory straight into MFMA operands, keeping a ring of steps
+//   in flight; W is the A operand, up to 64 rows of X the B operand.  The waves of a block are
+//   the segments of one tile of rows (or several tiles where S is small); their sums are added
+//   in segment order through LDS.  Epilogues: bias / residual add / SwiGLU, and the attention's
+//   qkv product with the rotary encoding and the store into the paged cache.
 //
-// * gemm_tile (M > 16): a block of 4 or 8 waves owns a BM x BN tile of the output, walks K in
+// * gemm_tile (M > 64): a block of 4 or 8 waves owns a BM x BN tile of the output, walks K in
 //   steps of 64 through LDS stages filled by direct global -> LDS loads (the next step's loads
 //   in flight while this one multiplies), and each wave keeps a tile of 32x32x16 MFMA
-//   accumulators.  X rows land in LDS with their 16-byte slots permuted so that fragment reads
-//   of neighbouring rows fall into different banks; W blocks land as they are.  Blocks are
-//   numbered so that the blocks of one XCD (every eighth block) share weight tiles in that
-//   XCD's L2.  Tiles: 64 x 128 / 64 x 256 for 17 to 64 rows, 128 x 128 for 65 to 256, and 256 x 256
-//   or 128 x 128 beyond, by how they fill the chip.  Where the output gives too few tiles for
-//   256 CUs, K is split between blocks (by (N, K) alone within a class of M), the blocks' sums go
-//   through a workspace and gemm_split_reduce adds them in block order and applies the epilogue.
-//
-// Classes of M: <= 16, 17..64, 65..256, 257..2048, > 2048.  Within a class a row's bits do not
-// depend on the other rows of the batch; between classes they differ by the rounding of 32-bit
-// sums (and only by that).
+//   accumulators.  The segments are either kept apart in registers (a second set of
+//   accumulators takes each finished segment's sums; SEG) or, where the output gives too few
+//   tiles for 256 CUs, given to blocks of their own (gridDim.y = S), whose sums go through a
+//   workspace and are added in segment order by gemm_split_reduce, which also applies the
+//   epilogue.  X rows land in LDS with their 16-byte slots permuted so that fragment reads of
+//   neighbouring rows fall into different banks; W blocks land as they are.  Blocks are numbered
+//   so that the blocks of one XCD (every eighth block) share weight tiles in that XCD's L2.
 #include "api.h"
 #include "common.h"
 
@@ -71,13 +73,16 @@ __device__ inline bf16x8 as_frag(u32x4 v) { return __builtin_bit_cast(bf16x8, v)
 // A block then owns BN / 2 output columns; each wave's share of the LDS tile holds the gate
 // rows of its columns and, after them, the up rows of the same columns, so that a lane ends
 // with both values of an output element.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK, int STAGES>
+//
+// SEG: the block walks all of K and keeps the `segs` segments apart: at the end of a segment its
+// sums are added to a second set of accumulators and the first starts from zero again.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK, int STAGES, bool SEG>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const void* __restrict__ bias,
                  int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode, int m_blocks,
-                 int n_blocks, float* __restrict__ partial) {
+                 int n_blocks, float* __restrict__ partial, int segs) {
   extern __shared__ __align__(16) unsigned char smem[];
-  static_assert(BK == 32 || BK == 64, "K steps of 32 or 64");
+  static_assert(BK == 64, "segments of K are counted in steps of 64");
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // a wave's tile
   constexpr int TM = WM / 32, TN = WN / 32;            // in 32 x 32 MFMA tiles
@@ -157,12 +162,17 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   };
 
   f32x16 acc[TM][TN];
+  f32x16 total[SEG ? TM : 1][SEG ? TN : 1];     // SEG: the sums of the segments that are finished
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+      for (int e = 0; e < 16; ++e) {
+        acc[i][j][e] = 0.0f;
+        if (SEG) total[i][j][e] = 0.0f;
+      }
+  int seg_at = 0, seg_end = SEG ? (int)((long)nk / segs) : 0;   // SEG: the segment under way ends before K tile seg_end
 
   // fragment addresses: row = tile row + lane % 32, k chunk = 2 ks + lane / 32, slot = chunk ^ SWZ(row)
   const int frow = lane & 31, fhalf = lane >> 5, fsw = SWZ(frow);
@@ -228,8 +238,28 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
         multiply(cur, TN / 2, TN);
       }
     }
+    if (SEG && kt + 1 == seg_end) {
+      // a segment's chain is complete: its sums join the finished ones, in segment order
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            total[i][j][e] += acc[i][j][e];
+            acc[i][j][e] = 0.0f;
+          }
+      ++seg_at;
+      seg_end = (int)((long)(seg_at + 1) * nk / segs);
+    }
   }
 #undef SWZ
+  if (SEG) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = total[i][j];
+  }
 
   // epilogue: lane holds column n = lane % 32 of each tile and rows (e/4)*8 + (lane/32)*4 + e%4
   if (partial) {
@@ -443,14 +473,14 @@ struct RopeStore;
 static int launch_split_reduce_rope(const float* partial, int splits, int m, int n, const void* bias, int bias_is_f32,
                                     void* out, int out_stride, const RopeStore& rope, hipStream_t stream);
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK = 64, int STAGES = 2>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, bool SEG = false, int BK = 64, int STAGES = 2>
 static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                       int out_stride, int m, int n, int k, int mode, hipStream_t stream, int splits = 1,
+                       int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs = 1,
                        float* partial = nullptr, const SplitNorm* norm = nullptr, const RopeStore* rope = nullptr) {
   static bool configured = false;
   constexpr int lds_bytes = STAGES * (BM + BN) * BK * 2;
   static_assert(lds_bytes <= 160 * 1024, "the stages do not fit the LDS of a CU");
-  auto kernel = &gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, GLU, BK, STAGES>;
+  auto kernel = &gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, GLU, BK, STAGES, SEG>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        lds_bytes);
@@ -460,9 +490,12 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
     }
     configured = true;
   }
+  // SEG: every block walks all segments; else a block a segment (gridDim.y) and the sums through `partial`
+  const int splits = SEG ? 1 : segs;
   const int m_blocks = ceil_div(m, BM), n_blocks = ceil_div(n, GLU ? BN / 2 : BN);
   kernel<<<dim3(m_blocks * n_blocks, splits), WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
-      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks, splits > 1 ? partial : nullptr);
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks, splits > 1 ? partial : nullptr,
+      segs);
   AXK_LAUNCH_CHECK("gemm_tile");
   if (splits > 1 && rope != nullptr) return launch_split_reduce_rope(partial, splits, m, n, bias, bias_is_f32, out, out_stride, *rope, stream);
   if (splits > 1 && norm != nullptr) {
@@ -477,40 +510,29 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
   return 0;
 }
 
-// ---------------------------------------------------------------------------- gemm_skinny
-// A block of WAVES waves owns NT16 row tiles (of 16) of W; wave v takes the k steps (of 64) v,
-// v + WAVES, ...  C[n][m] tiles of 16 x 16: the MFMA's A operand is W (a packed block as it lies
-// in memory), its B operand X (lane: row m = lane % 16, 8 consecutive k from (lane / 16) * 8).
-// A lane ends with 4 consecutive n of one m: one vector store.
-// GLU (NT16 = 2): the block's two tiles are the gate rows n0 .. n0 + 15 and the up rows of the
-// same columns (W holds 2 N rows), and the output is silu(gate) * up.
+// ---------------------------------------------------------------------------- gemm_stream
+// Up to 64 rows of X: the product is bound by reading W once.  A wave owns one tile of 32 rows
+// of W (two packed row tiles, A0 and A1) and one of the S segments of K.  Per step of 16 k it
+// loads 1 KB of W (the A operand of a 32x32x16 MFMA: lane l holds row l % 32, the 8 consecutive
+// k from 8 (l / 32); two pieces of 512 consecutive bytes, one in each packed tile) and, per 32
+// rows of X, 1 KB of X (the B operand: lane l holds row l % 32 of X, the same 8 k), and
+// multiplies; a ring of DEPTH steps is in flight, refilled as soon as a step is multiplied, so
+// the memory pipe never drains.  The waves of a block are TILES tiles x SEGS segments; the
+// segments' sums meet in LDS and are added in segment order, the 16 registers of a lane shared
+// out between the tile's waves in units of 4 consecutive output columns.
 //
-// An RMS norm can be folded into the product on either side, which saves the norm's own pass
-// over the rows (a launch each, between products that take microseconds):
-// * in_squares: X holds x * gain, not yet scaled by its row's 1/rms, and in_squares [M, K / 16]
-//   the sums of x^2 over the 16-column parts of each row.  Every block adds a row's parts (in
-//   the same order, so all blocks agree) and multiplies the finished sums of products by
-//   1/sqrt(sum / K + eps): the scale is common to the row, so it commutes with the product.
-// * norm_gain (with the add-into-residual epilogue): beside out += result the block writes what
-//   the next product's in_squares side takes: norm_values = out * norm_gain in bfloat16 and
-//   norm_squares [M, ceil(N / 16)], the sums of out^2 over each tile's 16 columns.
-struct NormFold {
-  const float* in_squares;
-  float in_eps;
-  const void* norm_gain;
-  int norm_gain_is_f32;
-  bf16_t* norm_values;
-  float* norm_squares;
-};
-
-// The product of the attention's fused [q; k; v] matrix with the rotary position encoding and the
-// store into the paged cache as its epilogue (EPI_ROPE, NT16 = 2): W's rows are heads of
-// head_dim; a block owns dims d0 .. d0 + 15 of one head and their rotation partners d0 + half ..,
-// so that a lane ends with both values of a pair.  q heads go rotated to `out`, k heads rotated
-// into the request's page of keys, v heads as they are into its page of values (kept
-// position-contiguous, [dim][slot]).  The arithmetic is that of the rotary kernel after a
-// plain product: the sums are rounded to bfloat16 first, and each product and sum of the
-// rotation is rounded on its own.
+// The accumulator of a 32 x 32 tile: lane l, register e holds W row 8 (e / 4) + 4 (l / 32) + e % 4
+// and X row l % 32.  Rows 0..15 come from packed tile A0, rows 16..31 from A1, so register e + 8
+// is the same row of A1 as register e of A0: the paired epilogues put partners there.
+// * plain: A0, A1 = tiles 2t, 2t + 1: 32 consecutive columns of the output.
+// * GLU: A0 = gate rows 16t .., A1 = the up rows of the same columns (W holds 2 N rows); the
+//   output is silu(gate) * up.
+// * ROPE (the attention's fused [q; k; v] matrix; W's rows are heads of head_dim): A0 = dims
+//   16j .. of a head, A1 = their rotation partners 16j + half ..; q heads go rotated to `out`,
+//   k heads rotated into the request's page of keys, v heads as they are into its page of
+//   values (kept position-contiguous, [dim][slot]).  The arithmetic is that of the rotary kernel
+//   after a plain product: the sums are rounded to bfloat16 first, and each product and sum of
+//   the rotation is rounded on its own.
 struct RopeStore {
   const float* table;            // [M, half, 2]: sin, cos of each token's angles
   const int32_t* positions;      // [M]
@@ -521,6 +543,7 @@ struct RopeStore {
   bf16_t* v_cache;
   int n_heads, n_kv_heads, head_dim, page_size;
 };
+
 
 enum { EPI_PLAIN = 0, EPI_GLU = 1, EPI_ROPE = 2 };
 
@@ -577,114 +600,72 @@ static int launch_split_reduce_rope(const float* partial, int splits, int m, int
   return 0;
 }
 
-template <int NT16, int MT16, int WAVES, int DEPTH, int EPI>
-__global__ void __launch_bounds__(WAVES * 64)
-gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w,
+template <int MT32, int SEGS, int TILES, int DEPTH, int EPI>
+__global__ void __launch_bounds__(SEGS * TILES * 64)
+gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w,
                    const void* __restrict__ bias, int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N,
-                   int K, int mode, NormFold fold, RopeStore rope) {
+                   int K, int mode, int n_tiles, RopeStore rope) {
   constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE;
-  static_assert(EPI == EPI_PLAIN || NT16 == 2, "the paired epilogues own two tiles of W rows");
-  __shared__ float partial[WAVES][NT16 * MT16][64][4];
-  __shared__ float row_scale[MT16 * 16];
+  constexpr int WAVES = SEGS * TILES;
+  // [wave][32 rows of X][4 groups of 4 registers][lane]: a lane's 4 consecutive registers are one 16-byte slot
+  __shared__ float4 sums[SEGS > 1 ? WAVES * MT32 * 4 * 64 : 1];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * (GLU ? 16 : NT16 * 16);
-  const int r16 = lane & 15, kq = (lane >> 4) * 8;
+  const int tile = blockIdx.x * TILES + wave / SEGS, seg = wave % SEGS;
+  const bool live = tile < n_tiles;                  // the last block may have tiles to spare
+  const int t = live ? tile : n_tiles - 1;
+  const int l32 = lane & 31, half = lane >> 5;
 
-  // the packed blocks of this block's row tiles: [row tile][k block of 32][lane][8]
+  // the two packed row tiles of this tile of 32 rows
   const int KB = K / 32;
-  const bf16_t* wtile[NT16];
-#pragma unroll
-  for (int i = 0; i < NT16; ++i) {
-    int tile;
-    if (GLU) tile = i * (N / 16) + blockIdx.x;                 // gate rows, then the up rows of the same columns
-    else if (ROPE) {
-      const int half = rope.head_dim / 2, per_head = half / 16;
-      tile = ((blockIdx.x / per_head) * rope.head_dim + i * half) / 16 + blockIdx.x % per_head;
-    } else tile = min(n0 / 16 + i, (N + 15) / 16 - 1);         // past the matrix: its last tile (columns dropped below)
-    wtile[i] = w + (size_t)tile * KB * 512 + lane * 8;
+  int a0, a1;
+  if (GLU) {
+    a0 = t;
+    a1 = N / 16 + t;
+  } else if (ROPE) {
+    const int per_head = rope.head_dim / 32;
+    a0 = (t / per_head) * (rope.head_dim / 16) + t % per_head;
+    a1 = a0 + rope.head_dim / 32;
+  } else {
+    const int last = (N + 15) / 16 - 1;              // past the matrix: its last tile (columns dropped below)
+    a0 = min(2 * t, last);
+    a1 = min(2 * t + 1, last);
   }
-  const bf16_t* xrow[MT16];
+  // step q (16 k from 16 q) of a packed row tile: the 512 bytes from 512 q; this lane's 16 of them
+  const bf16_t* wp = w + (size_t)((lane & 16) ? a1 : a0) * KB * 512 + (half * 16 + (lane & 15)) * 8;
+  const bf16_t* xp[MT32];
 #pragma unroll
-  for (int j = 0; j < MT16; ++j) xrow[j] = x + (size_t)min(j * 16 + r16, M - 1) * x_stride + kq;
+  for (int j = 0; j < MT32; ++j) xp[j] = x + (size_t)min(j * 32 + l32, M - 1) * x_stride + half * 8;
 
-  f32x4 acc[NT16][MT16];
-#pragma unroll
-  for (int i = 0; i < NT16; ++i)
-#pragma unroll
-    for (int j = 0; j < MT16; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  // this wave's segment: the K tiles (of 64) nk seg / SEGS .. nk (seg + 1) / SEGS - 1, in steps of 16
+  const int nk = K / 64;
+  const int q0 = (int)((long)seg * nk / SEGS) * 4;
+  const int steps = live ? (int)((long)(seg + 1) * nk / SEGS) * 4 - q0 : 0;
 
-  // This wave's steps (64 k each): wave, wave + WAVES, ...  A ring of DEPTH steps is kept in
-  // flight: a step is multiplied as soon as ITS loads have landed (loads return in order), and
-  // its place in the ring is refilled at once, so the memory pipe never drains.
-  const int steps = K / 64;
-  const int mine = steps > wave ? (steps - wave + WAVES - 1) / WAVES : 0;
-  uint4 wf[DEPTH][NT16][2], xf[DEPTH][MT16][2];
+  f32x16 acc[MT32];
+#pragma unroll
+  for (int j = 0; j < MT32; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[j][e] = 0.0f;
+
+  uint4 wf[DEPTH], xf[DEPTH][MT32];
   auto load = [&](int slot, int local) {
-    const int k0 = (wave + local * WAVES) * 64;
+    const int q = q0 + local;
+    wf[slot] = *reinterpret_cast<const uint4*>(wp + (size_t)q * 256);
 #pragma unroll
-    for (int i = 0; i < NT16; ++i) {
-      wf[slot][i][0] = *reinterpret_cast<const uint4*>(wtile[i] + k0 * 16);          // k block k0 / 32: 512 elements each
-      wf[slot][i][1] = *reinterpret_cast<const uint4*>(wtile[i] + k0 * 16 + 512);
-    }
-#pragma unroll
-    for (int j = 0; j < MT16; ++j) {
-      xf[slot][j][0] = *reinterpret_cast<const uint4*>(xrow[j] + k0);
-      xf[slot][j][1] = *reinterpret_cast<const uint4*>(xrow[j] + k0 + 32);
-    }
+    for (int j = 0; j < MT32; ++j) xf[slot][j] = *reinterpret_cast<const uint4*>(xp[j] + q * 16);
   };
   auto multiply = [&](int slot) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int i = 0; i < NT16; ++i)
-#pragma unroll
-        for (int j = 0; j < MT16; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[slot][i][h]), as_frag(xf[slot][j][h]), acc[i][j],
-                                                              0, 0, 0);
+    for (int j = 0; j < MT32; ++j)
+      acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(wf[slot]), as_frag(xf[slot][j]), acc[j], 0, 0, 0);
   };
-
-  // The rows' scales.  Wave v takes rows v, v + WAVES, ...; a lane adds every 64th part, then the
-  // lanes' sums are added.  Up to 256 parts (K <= 4096): one 16-byte load a lane and row, issued before the ring's,
-  // so they return first (loads return in order) and are added up while the ring's first loads
-  // are under way, and nothing between here and the main loop waits for the ring.  A wider K
-  // is added up in a loop, before the ring starts.
-  constexpr bool FOLDS = MT16 == 1;     // steps of up to 16 rows (see gemm_norm_fold_ok)
-  constexpr int RW = FOLDS ? 16 / WAVES : 1;
-  float4 sq[RW];
-  const int parts = K / 16;             // a multiple of 4, as K is one of 64
-  const bool fold_in = FOLDS && fold.in_squares != nullptr;
-  const bool few_parts = parts <= 256;
-  if (fold_in) {
-    if (few_parts) {
+  if (steps > 0) {
+    // The ring holds steps base .. base + DEPTH - 1: a step is multiplied as soon as ITS loads
+    // have landed (loads return in order), and its place is refilled at once.
 #pragma unroll
-      for (int i = 0; i < RW; ++i) {
-        const int m = wave + i * WAVES;
-        sq[i] = m < M && lane * 4 < parts ? *reinterpret_cast<const float4*>(fold.in_squares + (size_t)m * parts + lane * 4)
-                                          : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      }
-    } else {
-      for (int m = wave; m < M; m += WAVES) {
-        float sum = 0.0f;
-        for (int part = lane; part < parts; part += 64) sum += fold.in_squares[(size_t)m * parts + part];
-        const float total = wave_sum_to_last(sum);
-        if (lane == 63) row_scale[m] = 1.0f / sqrtf(total / (float)K + fold.in_eps);
-      }
-    }
-  }
-  if (mine > 0) {
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) load(d, min(d, mine - 1));   // beyond this wave's steps: a valid step again
-  }
-  if (fold_in && few_parts) {
-#pragma unroll
-    for (int i = 0; i < RW; ++i) {
-      const float total = wave_sum_to_last((sq[i].x + sq[i].y) + (sq[i].z + sq[i].w));
-      if (lane == 63) row_scale[wave + i * WAVES] = 1.0f / sqrtf(total / (float)K + fold.in_eps);
-    }
-  }
-  if (mine > 0) {
-    int base = 0;  // the ring holds local steps base .. base + DEPTH - 1
-    for (; base + 2 * DEPTH <= mine; base += DEPTH) {
+    for (int d = 0; d < DEPTH; ++d) load(d, min(d, steps - 1));    // beyond the segment: a valid step again
+    int base = 0;
+    for (; base + 2 * DEPTH <= steps; base += DEPTH) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
         multiply(d);
@@ -694,46 +675,62 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
     // the tail: what the ring holds, refilled only where a step is left, then those
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      if (base + d < mine) multiply(d);
-      if (base + DEPTH + d < mine) load(d, base + DEPTH + d);
+      if (base + d < steps) multiply(d);
+      if (base + DEPTH + d < steps) load(d, base + DEPTH + d);
     }
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d)
-      if (base + DEPTH + d < mine) multiply(d);
+      if (base + DEPTH + d < steps) multiply(d);
   }
 
+  if (SEGS > 1) {
 #pragma unroll
-  for (int i = 0; i < NT16; ++i)
+    for (int j = 0; j < MT32; ++j)
 #pragma unroll
-    for (int j = 0; j < MT16; ++j)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) partial[wave][i * MT16 + j][lane][e] = acc[i][j][e];
-  __syncthreads();
+      for (int g = 0; g < 4; ++g)
+        sums[((wave * MT32 + j) * 4 + g) * 64 + lane] =
+            make_float4(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
+    __syncthreads();
+  }
+  if (!live) return;
 
-  if (ROPE) {
-    const int hd = rope.head_dim, half = hd / 2, per_head = half / 16;
-    const int slot = blockIdx.x / per_head;                  // q heads, then k heads, then v heads
-    const int d = (blockIdx.x % per_head) * 16 + (lane >> 4) * 4;
-    for (int j = wave; j < MT16; j += WAVES) {
-      const int m = j * 16 + r16;
-      if (m >= M) continue;
-      const float scale = fold.in_squares ? row_scale[m] : 1.0f;
+  // Units of work: 4 registers (4 consecutive W rows 8 g + 4 half ..) of one 32-row part of X;
+  // the paired epilogues take group g (rows of A0) together with group g + 2 (the same rows of A1).
+  // The tile's waves share the units out; each adds the segments' sums in segment order.
+  constexpr int GROUPS = EPI == EPI_PLAIN ? 4 : 2;
+  const int first_wave = (wave / SEGS) * SEGS;
+  auto summed = [&](int j, int g) {
+    if (SEGS == 1) return make_float4(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
+    float4 v = sums[(((first_wave + 0) * MT32 + j) * 4 + g) * 64 + lane];
+#pragma unroll
+    for (int s = 1; s < SEGS; ++s) {
+      const float4 p = sums[(((first_wave + s) * MT32 + j) * 4 + g) * 64 + lane];
+      v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
+    }
+    return v;
+  };
+#pragma unroll
+  for (int u0 = 0; u0 < MT32 * GROUPS; u0 += SEGS) {
+    const int u = u0 + seg;
+    if (u >= MT32 * GROUPS) break;
+    // SEGS == 1: u is a compile-time constant, so the registers are indexed statically
+    const int j = u / GROUPS, g = u % GROUPS;
+    const int m = j * 32 + l32;
+    const int r = 8 * g + 4 * half;               // first of the 4 rows, within the 32 of the tile (or the 16 of A0)
+    if (m >= M) continue;
+    if (ROPE) {
+      const int hd = rope.head_dim, hh = hd / 2, per_head = hd / 32;
+      const int slot = tile / per_head;             // q heads, then k heads, then v heads
+      const int d = (tile % per_head) * 16 + r;
+      const float4 lo4 = summed(j, g), hi4 = summed(j, g + 2);
+      const float lo_s[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, hi_s[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
       float a[4], b[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float lo = partial[0][j][lane][e], hi = partial[0][MT16 + j][lane][e];
-#pragma unroll
-        for (int q = 1; q < WAVES; ++q) {
-          lo += partial[q][j][lane][e];
-          hi += partial[q][MT16 + j][lane][e];
-        }
-        if (fold.in_squares) {
-          lo *= scale;
-          hi *= scale;
-        }
+        float lo = lo_s[e], hi = hi_s[e];
         if (bias) {
           lo += load_vec(bias, bias_is_f32, slot * hd + d + e);
-          hi += load_vec(bias, bias_is_f32, slot * hd + half + d + e);
+          hi += load_vec(bias, bias_is_f32, slot * hd + hh + d + e);
         }
         a[e] = bf16_to_float(float_to_bf16(lo));
         b[e] = bf16_to_float(float_to_bf16(hi));
@@ -751,14 +748,14 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             vdst[(size_t)(d + e) * rope.page_size] = float_to_bf16(a[e]);
-            vdst[(size_t)(half + d + e) * rope.page_size] = float_to_bf16(b[e]);
+            vdst[(size_t)(hh + d + e) * rope.page_size] = float_to_bf16(b[e]);
           }
           continue;
         }
         const int kvh = slot - rope.n_heads;
         dst = rope.k_cache + (((size_t)page * rope.n_kv_heads + kvh) * rope.page_size + in_page) * hd;
       }
-      const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * half + d) * 2);
+      const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * hh + d) * 2);
       const float4 t0 = tab[0], t1 = tab[1];
       const float sn[4] = {t0.x, t0.z, t1.x, t1.z}, cs[4] = {t0.y, t0.w, t1.y, t1.w};
       float lo[4], hi[4];
@@ -773,85 +770,100 @@ gemm_skinny_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
       *reinterpret_cast<uint2*>(dst + d) = pk;
       pk.x = pack2_bf16(hi[0], hi[1]);
       pk.y = pack2_bf16(hi[2], hi[3]);
-      *reinterpret_cast<uint2*>(dst + half + d) = pk;
+      *reinterpret_cast<uint2*>(dst + hh + d) = pk;
+      continue;
     }
-    return;
-  }
-  if (GLU) {
-    // a wave takes both tiles of a column block: gate (tile j) and up (tile MT16 + j)
-    for (int j = wave; j < MT16; j += WAVES) {
-      const int m = j * 16 + r16;
-      const int n = n0 + (lane >> 4) * 4;
-      if (m >= M) continue;
-      const float scale = fold.in_squares ? row_scale[m] : 1.0f;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (n + e >= N) continue;
-        float g = partial[0][j][lane][e], u = partial[0][MT16 + j][lane][e];
-#pragma unroll
-        for (int q = 1; q < WAVES; ++q) {
-          g += partial[q][j][lane][e];
-          u += partial[q][MT16 + j][lane][e];
-        }
-        if (fold.in_squares) {
-          g *= scale;
-          u *= scale;
-        }
-        reinterpret_cast<bf16_t*>(out)[(size_t)m * out_stride + n + e] = float_to_bf16(swiglu1(g, u));
+    if (GLU) {
+      const int n = tile * 16 + r;                  // N is a multiple of 16: the unit's 4 columns exist
+      const float4 g4 = summed(j, g), u4 = summed(j, g + 2);
+      uint2 pk;
+      pk.x = pack2_bf16(swiglu1(g4.x, u4.x), swiglu1(g4.y, u4.y));
+      pk.y = pack2_bf16(swiglu1(g4.z, u4.z), swiglu1(g4.w, u4.w));
+      bf16_t* dst = reinterpret_cast<bf16_t*>(out) + (size_t)m * out_stride + n;
+      if (out_stride % 4 == 0 && ((uintptr_t)out & 7) == 0) *reinterpret_cast<uint2*>(dst) = pk;
+      else {
+        dst[0].bits = (uint16_t)pk.x; dst[1].bits = (uint16_t)(pk.x >> 16);
+        dst[2].bits = (uint16_t)pk.y; dst[3].bits = (uint16_t)(pk.y >> 16);
       }
+      continue;
     }
-    return;
-  }
-  // tiles are shared out between the waves; each sums the partials in wave order
-  for (int t = wave; t < NT16 * MT16; t += WAVES) {
-    const int i = t / MT16, j = t % MT16;
-    float v[4];
+    const int n = tile * 32 + r;
+    if (n >= N) continue;
+    const float4 v4 = summed(j, g);
+    float v[4] = {v4.x, v4.y, v4.z, v4.w};
+    if (bias) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float sum = partial[0][t][lane][e];
-#pragma unroll
-      for (int q = 1; q < WAVES; ++q) sum += partial[q][t][lane][e];
-      v[e] = sum;
+      for (int e = 0; e < 4; ++e)
+        if (n + e < N) v[e] += load_vec(bias, bias_is_f32, n + e);
     }
-    const int m = j * 16 + r16;
-    const int n = n0 + i * 16 + (lane >> 4) * 4;
-    const bool row_ok = m < M;
-    const float scale = fold.in_squares && row_ok ? row_scale[m] : 1.0f;
-    float squares = 0.0f;
+    const size_t at = (size_t)m * out_stride + n;
+    const bool whole = n + 3 < N && out_stride % 4 == 0;
+    if (mode == MODE_STORE) {
+      bf16_t* dst = reinterpret_cast<bf16_t*>(out) + at;
+      if (whole && ((uintptr_t)out & 7) == 0) {
+        uint2 pk;
+        pk.x = pack2_bf16(v[0], v[1]);
+        pk.y = pack2_bf16(v[2], v[3]);
+        *reinterpret_cast<uint2*>(dst) = pk;
+      } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (!row_ok || n + e >= N) continue;
-      float r = v[e];
-      if (fold.in_squares) r *= scale;
-      if (bias) r += load_vec(bias, bias_is_f32, n + e);
-      const size_t at = (size_t)m * out_stride + n + e;
-      if (mode == MODE_STORE) reinterpret_cast<bf16_t*>(out)[at] = float_to_bf16(r);
-      else if (mode == MODE_ADD_F32) {
-        const float sum = reinterpret_cast<float*>(out)[at] + r;
-        reinterpret_cast<float*>(out)[at] = sum;
-        if (fold.norm_gain) {
-          fold.norm_values[(size_t)m * N + n + e] = float_to_bf16(sum * load_vec(fold.norm_gain, fold.norm_gain_is_f32, n + e));
-          squares = fmaf(sum, sum, squares);
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) dst[e] = float_to_bf16(v[e]);
+      }
+    } else {
+      float* dst = reinterpret_cast<float*>(out) + at;
+      if (whole && ((uintptr_t)out & 15) == 0) {
+        float4 o = make_float4(v[0], v[1], v[2], v[3]);
+        if (mode == MODE_ADD_F32) {
+          const float4 old = *reinterpret_cast<const float4*>(dst);
+          o.x = old.x + v[0]; o.y = old.y + v[1]; o.z = old.z + v[2]; o.w = old.w + v[3];
         }
-      } else reinterpret_cast<float*>(out)[at] = r;
-    }
-    if (fold.norm_gain) {
-      // the four lanes that hold a row's 16 columns of this tile: lane, lane ^ 16, lane ^ 32, lane ^ 48
-      squares += __shfl_xor(squares, 16, AXON_WAVE);
-      squares += __shfl_xor(squares, 32, AXON_WAVE);
-      if (row_ok && lane < 16 && n0 + i * 16 < N) fold.norm_squares[(size_t)m * ((N + 15) >> 4) + (n0 >> 4) + i] = squares;
+        *reinterpret_cast<float4*>(dst) = o;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) dst[e] = mode == MODE_ADD_F32 ? dst[e] + v[e] : v[e];
+      }
     }
   }
 }
 
-template <int NT16, int MT16, int WAVES, int DEPTH, int EPI = EPI_PLAIN>
-static int launch_skinny(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                         int out_stride, int m, int n, int k, int mode, hipStream_t stream, const NormFold& fold,
-                         const RopeStore& rope = RopeStore()) {
-  gemm_skinny_kernel<NT16, MT16, WAVES, DEPTH, EPI><<<ceil_div(n, EPI == EPI_GLU ? 16 : NT16 * 16), WAVES * 64, 0, stream>>>(
-      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, fold, rope);
-  AXK_LAUNCH_CHECK("gemm_skinny");
+template <int MT32, int SEGS, int EPI>
+static int launch_stream(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                         int out_stride, int m, int n, int k, int mode, hipStream_t stream, int n_tiles,
+                         const RopeStore& rope) {
+  // eight waves a block where the segments allow it; the ring as deep as the registers allow
+  constexpr int TILES = SEGS >= 8 ? 1 : SEGS == 4 ? 2 : 4;
+  constexpr int DEPTH = MT32 == 1 ? 16 : 10;
+  gemm_stream_kernel<MT32, SEGS, TILES, DEPTH, EPI><<<ceil_div(n_tiles, TILES), SEGS * TILES * 64, 0, stream>>>(
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, n_tiles, rope);
+  AXK_LAUNCH_CHECK("gemm_stream");
   return 0;
+}
+
+template <int EPI>
+static int launch_stream_any(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                             int out_stride, int m, int n, int k, int mode, hipStream_t stream, int n_tiles, int segs,
+                             const RopeStore& rope) {
+#define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, n_tiles, rope
+  if (m <= 32) {
+    switch (segs) {
+      case 1: return launch_stream<1, 1, EPI>(ARGS);
+      case 2: return launch_stream<1, 2, EPI>(ARGS);
+      case 4: return launch_stream<1, 4, EPI>(ARGS);
+      case 8: return launch_stream<1, 8, EPI>(ARGS);
+    }
+  } else {
+    switch (segs) {
+      case 1: return launch_stream<2, 1, EPI>(ARGS);
+      case 2: return launch_stream<2, 2, EPI>(ARGS);
+      case 4: return launch_stream<2, 4, EPI>(ARGS);
+      case 8: return launch_stream<2, 8, EPI>(ARGS);
+    }
+  }
+#undef ARGS
+  axk_set_error("gemm_stream: %d segments", segs);
+  return -1;
 }
 
 // Shapes the MFMA kernels take: K a multiple of 64 and 16-byte aligned rows.  Decided by (N, K)
@@ -887,82 +899,49 @@ int launch_pack_matrix(const bf16_t* src, bf16_t* dst, int rows, int k, hipStrea
   return 0;
 }
 
-static bool skinny_takes(int m, int n, int k, int mode) { return m <= 16; }
 
-// 17 to 64 rows: one tile of rows (gemm_tile with a 64-row block), K split between blocks so
-// that the chip is full although the output is small; the blocks' sums go through a workspace
-// and are added in block order.  The number of splits depends on (N, K) alone: a row's bits do
-// not depend on how many rows ride along.
-static int mid_splits(int n, int k, int mode) {
-  if (n % 4 != 0) return 1;
-  const int per_block = mode == MODE_SWIGLU ? 128 : (n >= 8192 ? 256 : 128);
-  const int n_blocks = ceil_div(n, per_block), nk = k / 64;
-  // a block a CU for the narrow tile, two for the wide one (measured); at least four K tiles a block
-  int s = (per_block == 128 && mode != MODE_SWIGLU ? 256 : 512) / n_blocks;
-  if (s > nk / 4) s = nk / 4;
-  if (s > 32) s = 32;
-  return s < 1 ? 1 : s;
+// ---------------------------------------------------------------------------- the order and the dispatch
+// The number of segments K is cut into for a matrix of `tiles32` tiles of 32 rows (as gemm_stream
+// counts them: ceil(N / 32); N / 16 for a [gate; up] matrix of 2 N rows) and K columns: a power
+// of two up to 8, so that a step of few rows still gives some 768 waves a chain of their own,
+// with at least 4 K tiles (256 k) a segment.  It is a property of the matrix: it fixes the order
+// of addition of every product with it.
+int gemm_segments(int tiles32, int k) {
+  const int nk = k / 64;
+  int s = 1;
+  while (s < 8 && tiles32 * s < 768 && nk / (2 * s) >= 4) s *= 2;
+  return s;
 }
 
-// 65 to 256 rows: one or two rows of 128 x 128 tiles, which leave most CUs idle when N is small;
-// K is split so that about a block a CU runs.  Again by (N, K) alone.
-static int small_splits(int n, int k, int mode) {
-  if (n % 4 != 0) return 1;
-  const int n_blocks = ceil_div(n, mode == MODE_SWIGLU ? 64 : 128), nk = k / 64;
-  int s = 256 / (2 * n_blocks);
-  if (s > nk / 4) s = nk / 4;
-  if (s > 16) s = 16;
-  return s < 1 ? 1 : s;
-}
+static int tiles32_of(int n, int mode) { return mode == MODE_SWIGLU ? n / 16 : (n + 31) / 32; }
 
-// 257 to 2048 rows: a narrow output gives too few 256 x 256 tiles for 256 CUs, or a number of
-// them that leaves the last round mostly idle; K is then cut into 2 to 4 parts.  By (N, K)
-// alone (the tiles are counted for 2,048 rows).  The time of the product is the rounds of blocks
-// over the parts; adding the parts' sums costs about 500 / K of the product's ideal time a
-// part (twice that for [gate; up]).  A cut has to win 8 % and leave 24 K tiles a part.
-static int long_k_splits(int n, int k, int mode) {
-  if (n % 4 != 0) return 1;
-  const bool glu = mode == MODE_SWIGLU;
-  const int tiles = 8 * ceil_div(n, glu ? 128 : 256), nk = k / 64;
-  int best = 1;
-  double best_cost = (double)ceil_div(tiles, 256);
-  for (int s = 2; s <= 4; ++s) {
-    if (nk / s < 24) break;
-    const double cost = (double)ceil_div(tiles * s, 256) / s + 500.0 * s / k * (tiles / 256.0) * (glu ? 2 : 1);
-    if (cost < 0.92 * best_cost) {
-      best = s;
-      best_cost = cost;
-    }
-  }
-  return best;
-}
-
-static int splits_of(int m, int n, int k, int mode) {
-  if (m <= 16 || m > 2048) return 1;
-  return m <= 64 ? mid_splits(n, k, mode) : m <= 256 ? small_splits(n, k, mode) : long_k_splits(n, k, mode);
+// M > 64 with S > 1 segments: kept apart in registers by blocks that walk all of K where the output
+// alone gives enough tiles of 128 x 128 (or 128 x 256) to occupy the chip, else a block a segment
+// and the sums through a workspace.  Decided by the sizes alone.
+static bool segments_across_blocks(int m, int n, int k, int mode, int segs) {
+  if (segs <= 1 || n % 4 != 0) return false;
+  const long blocks = (long)ceil_div(m, 128) * ceil_div(n, mode == MODE_SWIGLU ? 64 : 128);
+  return blocks < 100;
 }
 
 size_t gemm_workspace_bytes(int m, int n, int k, int mode) {
-  if (k % 64 != 0) return 0;
-  const int s = splits_of(m, n, k, mode);
-  return s > 1 ? (size_t)s * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float) : 0;
+  if (k % 64 != 0 || m <= 64) return 0;
+  const int s = gemm_segments(tiles32_of(n, mode), k);
+  if (!segments_across_blocks(m, n, k, mode, s)) return 0;
+  return (size_t)s * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float);
 }
 
-int gemm_norm_fold_ok(int m, int n, int k, int mode) {
-  return gemm_pack_ok(mode == MODE_SWIGLU ? 2 * n : n, k, mode == MODE_SWIGLU) && skinny_takes(m, n, k, mode);
-}
-
-// Whether the product that adds into the rows runs with K split between blocks, so that the
-// kernel that adds the blocks' sums can also norm the finished rows (gemm_split_reduce_norm_kernel:
-// rows of up to SRN_MAX_N columns).
+// Whether the product that adds into the rows runs with a block a segment, so that the kernel that
+// adds the segments' sums can also norm the finished rows (gemm_split_reduce_norm_kernel: rows of
+// up to SRN_MAX_N columns).
 int gemm_then_norm_ok(int m, int n, int k) {
-  return gemm_pack_ok(n, k, 0) && !skinny_takes(m, n, k, MODE_ADD_F32) && splits_of(m, n, k, MODE_ADD_F32) > 1 &&
-         n <= SRN_MAX_N;
+  return gemm_pack_ok(n, k, 0) && m > 64 && n <= SRN_MAX_N &&
+         segments_across_blocks(m, n, k, MODE_ADD_F32, gemm_segments(tiles32_of(n, MODE_ADD_F32), k));
 }
 
 static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                               int out_stride, int m, int n, int k, int mode, hipStream_t stream,
-                              const GemmNormFold* fold_in, void* workspace, size_t workspace_bytes,
+                              const SplitNorm* norm, void* workspace, size_t workspace_bytes,
                               const RopeStore* rope_after) {
   if (!gemm_pack_ok(mode == MODE_SWIGLU ? 2 * n : n, k, mode == MODE_SWIGLU)) {
     axk_set_error("gemm: N=%d K=%d is no shape of a packed matrix", n, k);
@@ -973,37 +952,21 @@ static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, co
                   "(stride %d, M=%d)", x_stride, m);
     return -1;
   }
-  NormFold fold = {nullptr, 0.0f, nullptr, 0, nullptr, nullptr};
-  if (fold_in) {
-    fold.in_squares = fold_in->in_squares;
-    fold.in_eps = fold_in->in_eps;
-    fold.norm_gain = fold_in->norm_gain;
-    fold.norm_gain_is_f32 = fold_in->norm_gain_is_f32;
-    fold.norm_values = (bf16_t*)fold_in->norm_values;
-    fold.norm_squares = fold_in->norm_squares;
-  }
+  const int tiles32 = tiles32_of(n, mode);
+  const int segs = gemm_segments(tiles32, k);
 #define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream
-  if (skinny_takes(m, n, k, mode)) {
-    if (mode == MODE_SWIGLU) return launch_skinny<2, 1, 4, 8, EPI_GLU>(ARGS, fold);
-    // 32 rows of W per block where that still leaves 128 blocks or more, else 16; four waves
-    // split K; the ring is as deep as the registers allow
-    return n >= 32 * 128 ? launch_skinny<2, 1, 4, 8>(ARGS, fold) : launch_skinny<1, 1, 4, 8>(ARGS, fold);
-  }
-  // the tiled kernels: no norm on the way in; on the way out only a whole norm behind split sums
-  SplitNorm after = {nullptr, 0, 0.0f, nullptr};
-  const SplitNorm* norm = nullptr;
-  if (fold_in) {
-    const bool whole = fold_in->in_squares == nullptr && fold_in->norm_gain && fold_in->norm_values && !fold_in->norm_squares;
-    if (!whole || mode != MODE_ADD_F32 || !gemm_then_norm_ok(m, n, k)) {
-      axk_set_error("gemm: M=%d N=%d K=%d mode %d goes to the tiled kernel, which folds no such norm", m, n, k, mode);
+  if (m <= 64) {
+    if (norm || rope_after) {
+      axk_set_error("gemm: M=%d goes to the streaming kernel, which has these epilogues of its own", m);
       return -1;
     }
-    after = SplitNorm{fold_in->norm_gain, fold_in->norm_gain_is_f32, fold_in->norm_eps, (bf16_t*)fold_in->norm_values};
-    norm = &after;
+    if (mode == MODE_SWIGLU) return launch_stream_any<EPI_GLU>(ARGS, tiles32, segs, RopeStore());
+    return launch_stream_any<EPI_PLAIN>(ARGS, tiles32, segs, RopeStore());
   }
-  const int splits = splits_of(m, n, k, mode);
-  if (rope_after && (splits < 2 || mode != MODE_STORE)) {
-    axk_set_error("gemm: M=%d N=%d K=%d does not run with K split: the rotary kernel stays apart", m, n, k);
+  const bool across = segments_across_blocks(m, n, k, mode, segs);
+  if ((norm || rope_after) && (!across || mode != (norm ? MODE_ADD_F32 : MODE_STORE))) {
+    axk_set_error("gemm: M=%d N=%d K=%d mode %d does not run with a block a segment: no kernel adds sums after it", m, n,
+                  k, mode);
     return -1;
   }
   const size_t need = gemm_workspace_bytes(m, n, k, mode);
@@ -1013,68 +976,77 @@ static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, co
     return -1;
   }
   float* ws = (float*)workspace;
-  if (m <= 256) {
-    if (m > 64) {
-      if (mode == MODE_SWIGLU) return launch_tile<128, 128, 2, 2, true>(ARGS, splits, ws);
-      return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws, norm, rope_after);
+  const bool glu = mode == MODE_SWIGLU;
+  if (segs > 1 && !across) {
+    // the segments in registers: 128 x 256 tiles (8 waves) where they occupy the chip, else 128 x 128
+    const long wide = (long)ceil_div(m, 128) * ceil_div(n, glu ? 128 : 256);
+    if (wide >= 200) {
+      if (glu) return launch_tile<128, 256, 2, 4, true, true>(ARGS, segs);
+      return launch_tile<128, 256, 2, 4, false, true>(ARGS, segs);
     }
-    if (mode == MODE_SWIGLU) return launch_tile<64, 256, 1, 4, true, 64, 2>(ARGS, splits, ws);
-    if (n >= 8192) return launch_tile<64, 256, 1, 4, false, 64, 2>(ARGS, splits, ws, norm, rope_after);
-    return launch_tile<64, 128, 1, 4, false, 64, 3>(ARGS, splits, ws, norm, rope_after);
+    if (glu) return launch_tile<128, 128, 2, 2, true, true>(ARGS, segs);
+    return launch_tile<128, 128, 2, 2, false, true>(ARGS, segs);
+  }
+  if (m <= 256) {
+    if (glu) return launch_tile<128, 128, 2, 2, true>(ARGS, segs, ws);
+    return launch_tile<128, 128, 2, 2, false>(ARGS, segs, ws, norm, rope_after);
   }
   // 256 x 256 tiles (8 waves) where they fill the chip: one round of at least 140 blocks (on 256
   // CUs), or several rounds of which the last is not mostly idle; else 128 x 128 tiles, four times
   // as many blocks at twice the traffic from L2 per product.  Thresholds are measured ones.
-  const int n_per_block = mode == MODE_SWIGLU ? 128 : 256;
+  const int splits = across ? segs : 1;
+  const int n_per_block = glu ? 128 : 256;
   const long big = (long)ceil_div(m, 256) * ceil_div(n, n_per_block) * splits;
   const long rounds = (big + 255) / 256;
   const bool use_big = big <= 256 ? big >= 140 : big * 10 >= rounds * 256 * 7;
-  if (mode == MODE_SWIGLU) {
-    if (use_big) return launch_tile<256, 256, 4, 2, true>(ARGS, splits, ws);
-    return launch_tile<128, 128, 2, 2, true>(ARGS, splits, ws);
+  if (glu) {
+    if (use_big) return launch_tile<256, 256, 4, 2, true>(ARGS, segs, ws);
+    return launch_tile<128, 128, 2, 2, true>(ARGS, segs, ws);
   }
   // one round of 256 x 256 tiles that leaves a quarter of the CUs idle, and N in whole tiles of
   // 192 columns that still fit one round: the narrower tile (measured 1.1 times the cost per
-  // product, three quarters of the products per block).  The k order of a sum is the same.
+  // product, three quarters of the products per block).
   if (use_big && splits == 1 && big <= 192 && n % 192 == 0 && (long)ceil_div(m, 256) * (n / 192) <= 256)
-    return launch_tile<256, 192, 4, 2, false>(ARGS, splits, ws, norm);
-  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS, splits, ws, norm, rope_after);
-  return launch_tile<128, 128, 2, 2, false>(ARGS, splits, ws, norm, rope_after);
+    return launch_tile<256, 192, 4, 2, false>(ARGS, segs, ws, norm);
+  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS, segs, ws, norm, rope_after);
+  return launch_tile<128, 128, 2, 2, false>(ARGS, segs, ws, norm, rope_after);
 #undef ARGS
 }
 
 int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* fold_in,
+                     int out_stride, int m, int n, int k, int mode, hipStream_t stream, const GemmNormFold* then_norm,
                      void* workspace, size_t workspace_bytes) {
-  return gemm_mfma_dispatch(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, fold_in, workspace,
-                            workspace_bytes, nullptr);
+  SplitNorm after = {nullptr, 0, 0.0f, nullptr};
+  if (then_norm)
+    after = SplitNorm{then_norm->norm_gain, then_norm->norm_gain_is_f32, then_norm->norm_eps, (bf16_t*)then_norm->norm_values};
+  return gemm_mfma_dispatch(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream,
+                            then_norm ? &after : nullptr, workspace, workspace_bytes, nullptr);
 }
 
-// The [q; k; v] product with rotary encoding and cache store (see RopeStore): up to 16 rows in
-// the epilogue of gemm_skinny, more rows where the product splits K (then the kernel that adds
-// the parts' sums rotates and stores); every head rotated over its whole width, halves of a head
-// a multiple of 16 wide.
+// The [q; k; v] product with rotary encoding and cache store (see RopeStore): up to 64 rows in
+// the epilogue of gemm_stream, more rows where the product runs with a block a segment (then the
+// kernel that adds the segments' sums rotates and stores); every head rotated over its whole
+// width, halves of a head a multiple of 16 wide.
 int gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotary_dim) {
   if (m < 1 || k % 64 != 0 || rotary_dim != head_dim || head_dim % 32 != 0 || n % head_dim != 0) return 0;
-  if (m <= 16) return 1;
-  return gemm_pack_ok(n, k, 0) && n % 4 == 0 && splits_of(m, n, k, MODE_STORE) > 1;
+  if (!gemm_pack_ok(n, k, 0)) return 0;
+  if (m <= 64) return 1;
+  return segments_across_blocks(m, n, k, MODE_STORE, gemm_segments(tiles32_of(n, MODE_STORE), k));
 }
 
 int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out,
-                         int out_stride, int m, int n, int k, const float* in_squares, float in_eps,
-                         const float* table, const int32_t* positions, const int32_t* seq_rows,
-                         const int32_t* block_table, int table_stride, bf16_t* k_cache, bf16_t* v_cache, int n_heads,
-                         int n_kv_heads, int head_dim, int page_size, void* workspace, size_t workspace_bytes,
-                         hipStream_t stream) {
-  const NormFold fold = {in_squares, in_eps, nullptr, 0, nullptr, nullptr};
+                         int out_stride, int m, int n, int k, const float* table, const int32_t* positions,
+                         const int32_t* seq_rows, const int32_t* block_table, int table_stride, bf16_t* k_cache,
+                         bf16_t* v_cache, int n_heads, int n_kv_heads, int head_dim, int page_size, void* workspace,
+                         size_t workspace_bytes, hipStream_t stream) {
   const RopeStore rope = {table, positions, seq_rows, block_table, table_stride, k_cache, v_cache,
                           n_heads, n_kv_heads, head_dim, page_size};
-  if (m > 16)
+  if (m > 64)
     return gemm_mfma_dispatch(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream, nullptr,
                               workspace, workspace_bytes, &rope);
-#define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream, fold, rope
-  return launch_skinny<2, 1, 4, 8, EPI_ROPE>(ARGS);
-#undef ARGS
+  const int tiles32 = n / 32;
+  return launch_stream_any<EPI_ROPE>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream,
+                                     tiles32, gemm_segments(tiles32, k), rope);
 }
 
 #endif  // AXON_BF16

@@ -31,11 +31,3 @@ class Workspace:
 
     def take(self, shape, dtype) -> torch.Tensor:
         return torch.empty(shape, dtype=dtype, device=self.device)
-
-    take_persistent = take
-
-    def mark(self):
-        return None
-
-    def release(self, mark) -> None:
-        pass

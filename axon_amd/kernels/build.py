@@ -31,9 +31,12 @@ KERNEL_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "attention.hip
                   "sampling.hip"]
 HOST_SOURCES = ["host/cache.cpp", "host/scheduler.cpp", "host/sampler.cpp"]
 
-# Packed 32-bit float instructions are switched off for all device code.
-HIP_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
-             "-packed-fp32-ops", "-Wno-unused-result", "-Wno-unused-command-line-argument"]
+# Packed 32-bit float instructions are switched off for all device code.  No contraction of a
+# product and a sum into a multiply-add unless the source writes one (fmaf): two kernels that
+# hold the same expression must round it the same way, whatever surrounds it (hipcc would
+# otherwise fuse where a product happens to be in a register and not where it was loaded).
+HIP_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "-fPIC", "-ffp-contract=off", "-Xclang", "-target-feature",
+             "-Xclang", "-packed-fp32-ops", "-Wno-unused-result", "-Wno-unused-command-line-argument"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
 
 DTYPE_FLAG = {"bfloat16": "-DAXON_BF16=1", "float32": "-DAXON_BF16=0"}

@@ -37,7 +37,7 @@ _SIGNATURES = {
     "axk_rope_kv_write": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int,
                           c_int, c_int, c_int, c_int, c_int, c_void_p],
     "axk_gemm_qkv_rope_ok": [c_int, c_int, c_int, c_int, c_int],
-    "axk_gemm_qkv_rope": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_float,
+    "axk_gemm_qkv_rope": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                           c_int, c_void_p, ctypes.c_long, c_void_p],
     "axk_attention": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
@@ -52,9 +52,7 @@ _SIGNATURES = {
                  ctypes.c_long, c_void_p],
     "axk_pack_ok": [c_int, c_int, c_int],
     "axk_pack_matrix": [c_void_p, c_void_p, c_int, c_int, c_void_p],
-    "axk_gemm_norm_fold_ok": [c_int, c_int, c_int, c_int],
-    "axk_gemm_norm_fold": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                           c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+    "axk_gemm_segments": [c_int, c_int, c_int],
     "axk_gemm_then_norm_ok": [c_int, c_int, c_int],
     "axk_gemm_then_norm": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int,
                            c_float, c_void_p, c_void_p, ctypes.c_long, c_void_p],
@@ -219,12 +217,12 @@ class Kernels:
         return bool(self.lib.axk_gemm_qkv_rope_ok(m, n, k, head_dim, rotary_dim))
 
     def gemm_qkv_rope(self, x, w, bias, qkv, table, positions, seq_rows, block_table, k_cache, v_cache, n_heads,
-                      n_kv_heads, head_dim, page_size, write_kv=True, row_squares=None, eps=0.0) -> None:
+                      n_kv_heads, head_dim, page_size, write_kv=True) -> None:
         """The [q; k; v] product, the rotary encoding and the store into the pages in one launch
-        (up to 16 tokens) or with the kernel that adds a split product's parts doing the rest:
+        (up to 64 tokens) or with the kernel that adds a product's segments doing the rest:
         the same bits as `gemm` into qkv followed by `rope_kv_write`.  q lands in qkv[:, :n_heads *
         head_dim]; the k and v columns of qkv are not written.  Without write_kv, w holds the q
-        rows only.  row_squares, eps: as in `gemm`."""
+        rows only."""
         if not isinstance(w, PackedMatrix):
             raise KernelError("gemm_qkv_rope: needs a packed matrix")
         self._elem(x, "qkv x"); self._elem(w.data, "qkv w"); self._elem(qkv, "qkv out"); self._f32(table, "rope table")
@@ -239,16 +237,13 @@ class Kernels:
             raise KernelError(f"gemm_qkv_rope: table {tuple(table.shape)} or positions do not fit {M} tokens")
         if bias is not None and bias.numel() != rows:
             raise KernelError(f"gemm_qkv_rope: bias of {bias.numel()} for {rows} rows")
-        if row_squares is not None and (row_squares.dtype != torch.float32 or not row_squares.is_contiguous()
-                                        or row_squares.shape != (M, K // 16) or not row_squares.is_cuda):
-            raise KernelError(f"gemm_qkv_rope: row_squares {tuple(row_squares.shape)} is not float32 [{M}, {K // 16}]")
         if write_kv:
             self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
         need = self.lib.axk_gemm_workspace(M, rows, K, MODE_STORE)
         work = torch.empty(need // 4, dtype=torch.float32, device=x.device) if need > 0 else None
         self._check(self.lib.axk_gemm_qkv_rope(
             _ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "qkv bias"), _ptr(qkv), qkv.stride(0), M, K,
-            _ptr(row_squares), float(eps), _ptr(table), _ptr(positions), _ptr(seq_rows), _ptr(block_table),
+            _ptr(table), _ptr(positions), _ptr(seq_rows), _ptr(block_table),
             block_table.shape[-1], _ptr(k_cache if write_kv else None), _ptr(v_cache if write_kv else None), n_heads,
             n_kv_heads, head_dim, page_size, 1 if write_kv else 0, _ptr(work), need, _stream()))
 
@@ -332,10 +327,9 @@ class Kernels:
             raise KernelError(f"attention_decode: {n} tokens, q has {q.shape[0]} rows")
         if out.shape[1] != n_heads * head_dim or not out.is_contiguous():
             raise KernelError(f"attention_decode: out {tuple(out.shape)}")
-        if max_chunks > 1:
-            self._f32(partial, "attention partial")
-            if partial.numel() < self.attention_decode_workspace(n, n_heads, head_dim, max_chunks):
-                raise KernelError(f"attention_decode: workspace of {partial.numel()} floats is too small")
+        self._f32(partial, "attention partial")
+        if partial.numel() < self.attention_decode_workspace(n, n_heads, head_dim, max_chunks):
+            raise KernelError(f"attention_decode: workspace of {partial.numel()} floats is too small")
         if work is None:
             at = positions[:n] if token_index is None else positions[token_index.long()]
             work = torch.tensor(self.attention_decode_work(at.tolist(), window), dtype=torch.int32).to(q.device)
@@ -345,7 +339,7 @@ class Kernels:
         self._check(self.lib.axk_attention_decode(
             _ptr(q), q_stride, _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[-1], _ptr(positions),
             _ptr(seq_rows), _ptr(out), _ptr(token_index), n, _ptr(work), work.numel(),
-            _ptr(partial if max_chunks > 1 else None), max_chunks, n_heads, n_kv_heads, head_dim, page_size, window,
+            _ptr(partial), max_chunks, n_heads, n_kv_heads, head_dim, page_size, window,
             float(scale), _stream()))
         return out
 
@@ -372,27 +366,24 @@ class Kernels:
 
     def gemm_then_norm_ok(self, m: int, n: int, k: int) -> bool:
         """Whether the product that adds into [m, n] float32 rows can also write the RMS norm of
-        the new rows (see `gemm`: a `following_norm` without squares)."""
+        the new rows (see `gemm`: `following_norm`)."""
         return bool(self.lib.axk_gemm_then_norm_ok(m, n, k))
 
-    def gemm_norm_fold_ok(self, m: int, n: int, k: int, mode: int) -> bool:
-        """Whether the product of these sizes can take an RMS norm into itself (see `gemm`)."""
-        return bool(self.lib.axk_gemm_norm_fold_ok(m, n, k, mode))
+    def gemm_segments(self, n: int, k: int, gated: bool = False) -> int:
+        """The number of contiguous segments of K whose sums a product with a packed [n, k]
+        matrix adds in ascending order (gated: a [gate; up] matrix for n output columns).  It
+        depends on the matrix alone: a row's bits do not depend on the other rows of a step."""
+        return int(self.lib.axk_gemm_segments(n, k, 1 if gated else 0))
 
     def gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
-             mode: int = MODE_STORE, row_squares: Optional[torch.Tensor] = None, eps: float = 0.0,
-             following_norm=None) -> torch.Tensor:
+             mode: int = MODE_STORE, following_norm=None) -> torch.Tensor:
         """out = epilogue(x . w^T + bias); x [M, K] (rows may be strided), w [N, K] contiguous or
         a PackedMatrix (the matrix-core kernels; a row-major w goes to the 32-bit FMA kernel).
         MODE_SWIGLU: w is [2 N, K], gate rows then up rows; out [M, N] = silu(x gate^T) * (x up^T).
 
-        An RMS norm folded in (where `gemm_norm_fold_ok`): with `row_squares` float32 [M, K / 16],
-        x holds rows times their gain that still lack the scale 1/sqrt(sum(row_squares) / K + eps),
-        which the product applies to its result.  `following_norm` = (gain, values [M, N],
-        squares [M, ceil(N / 16)], eps) with MODE_ADD_F32: the epilogue also writes out * gain and
-        the sums of out^2 over parts of 16 columns, for the next product's `row_squares` side.
-        With squares None (where `gemm_then_norm_ok`): values = the whole norm of the new rows,
-        out / sqrt(mean(out^2) + eps) * gain."""
+        `following_norm` = (gain, values [M, N], eps) with MODE_ADD_F32, where `gemm_then_norm_ok`:
+        the kernel that finishes the product also writes the RMS norm of the new rows,
+        values = out / sqrt(mean(out^2) + eps) * gain, the same bits as `rmsnorm` after it."""
         packed = isinstance(w, PackedMatrix)
         self._elem(x, "gemm x"); self._elem(w.data if packed else w, "gemm w")
         M, K = x.shape
@@ -410,45 +401,24 @@ class Kernels:
             raise KernelError(f"gemm: mode {mode} writes {want}, out is {out.dtype}")
         if bias is not None and bias.numel() != N:
             raise KernelError(f"gemm: bias of {bias.numel()} for {N} columns")
-        if row_squares is None and following_norm is None:
-            need = self.lib.axk_gemm_workspace(M, N, K, mode) if packed else 0
-            work = torch.empty(need // 4, dtype=torch.float32, device=x.device) if need > 0 else None
+        need = self.lib.axk_gemm_workspace(M, N, K, mode) if packed else 0
+        work = torch.empty(need // 4, dtype=torch.float32, device=x.device) if need > 0 else None
+        if following_norm is None:
             self._check(self.lib.axk_gemm(_ptr(x), x.stride(0), _ptr(w), 1 if packed else 0, _ptr(bias),
                                           self._vec_flag(bias, "gemm bias"), _ptr(out), out.stride(0), M, N, K, mode,
                                           _ptr(work), need, _stream()))
             return out
-        if not packed:
-            raise KernelError("gemm: a norm is folded only into products with a packed matrix")
-        if row_squares is not None and (row_squares.dtype != torch.float32 or not row_squares.is_contiguous()
-                                        or row_squares.shape != (M, K // 16) or not row_squares.is_cuda):
-            raise KernelError(f"gemm: row_squares {tuple(row_squares.shape)} {row_squares.dtype} is not float32 "
-                              f"[{M}, {K // 16}]")
-        gain = values = squares = None
-        if following_norm is not None:
-            gain, values, squares, norm_eps = following_norm
-            self._elem(values, "gemm norm values")
-            if squares is None:
-                if row_squares is not None or mode != MODE_ADD_F32:
-                    raise KernelError("gemm: a whole norm follows only the product that adds into float32 rows")
-                if gain.numel() != N or values.shape != (M, N) or not values.is_contiguous():
-                    raise KernelError(f"gemm: the following norm's gain {tuple(gain.shape)} or values "
-                                      f"{tuple(values.shape)} do not fit [{M}, {N}]")
-                need = self.lib.axk_gemm_workspace(M, N, K, mode)
-                work = torch.empty(need // 4, dtype=torch.float32, device=x.device) if need > 0 else None
-                self._check(self.lib.axk_gemm_then_norm(
-                    _ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"), _ptr(out), out.stride(0),
-                    M, N, K, _ptr(gain), self._vec_flag(gain, "gemm norm gain"), float(norm_eps), _ptr(values), _ptr(work),
-                    need, _stream()))
-                return out
-            if (gain.numel() != N or values.shape != (M, N) or not values.is_contiguous()
-                    or squares.shape != (M, -(-N // 16)) or squares.dtype != torch.float32 or not squares.is_contiguous()
-                    or not squares.is_cuda):
-                raise KernelError(f"gemm: the following norm's gain {tuple(gain.shape)}, values {tuple(values.shape)} "
-                                  f"or squares {tuple(squares.shape)} do not fit [{M}, {N}]")
-        self._check(self.lib.axk_gemm_norm_fold(
-            _ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"), _ptr(out), out.stride(0), M, N, K,
-            mode, _ptr(row_squares), float(eps), _ptr(gain), self._vec_flag(gain, "gemm norm gain"), _ptr(values),
-            _ptr(squares), _stream()))
+        gain, values, norm_eps = following_norm
+        self._elem(values, "gemm norm values")
+        if not packed or mode != MODE_ADD_F32:
+            raise KernelError("gemm: a norm follows only the product with a packed matrix that adds into float32 rows")
+        if gain.numel() != N or values.shape != (M, N) or not values.is_contiguous():
+            raise KernelError(f"gemm: the following norm's gain {tuple(gain.shape)} or values "
+                              f"{tuple(values.shape)} do not fit [{M}, {N}]")
+        self._check(self.lib.axk_gemm_then_norm(
+            _ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "gemm bias"), _ptr(out), out.stride(0),
+            M, N, K, _ptr(gain), self._vec_flag(gain, "gemm norm gain"), float(norm_eps), _ptr(values), _ptr(work),
+            need, _stream()))
         return out
 
     def swiglu(self, gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

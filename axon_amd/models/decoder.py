@@ -110,21 +110,18 @@ class DecoderModel:
     def forward(self, ctx) -> torch.Tensor:
         """The residual stream after every run: float32 [T, hidden]."""
         x = self.embedding.forward(ctx)
-        unscaled = None      # the next block's first norm, where the block before it did its work
+        normed = None        # the next block's first norm, where the block before it did its work
         for i, (run, binding) in enumerate(zip(self.order, self.cache_plan.bindings)):
             block = self.blocks[run.layer]
-            fold = None
+            following = None
             if i + 1 < len(self.order):
                 after = self.blocks[self.order[i + 1].layer]
-                if block.finishes_following_norm(ctx):
-                    fold = after.first_norm_fold(ctx, x.shape[0], whole=True)
-                elif block.folds_following_norm(ctx):
-                    fold = after.first_norm_fold(ctx, x.shape[0])
-            if unscaled is None and fold is None:
-                block.forward(ctx, binding, x)
+                following = block.following_of(ctx, block.last_part(), after.first_norm(), x.shape[0])
+            if normed is None and following is None:
+                block.forward(ctx, binding, x)          # a block that knows nothing of this is called plainly
             else:
-                block.forward(ctx, binding, x, unscaled, fold)
-            unscaled = None if fold is None else fold.rows()
+                block.forward(ctx, binding, x, normed, following)
+            normed = None if following is None else following.values
         return x
 
     def logits(self, ctx, x: torch.Tensor, rows: torch.Tensor, out=None) -> torch.Tensor:

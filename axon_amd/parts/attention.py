@@ -21,7 +21,7 @@ import torch
 
 from ..config.base import ConfigError
 from ..kernels import MODE_ADD_F32, MODE_STORE, PackedMatrix
-from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, UnscaledRows, build_part, register_mixer
+from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, build_part, register_mixer
 
 
 PREFILL_TILE = 128     # tokens of one request per tile of the prompt kernel
@@ -69,7 +69,7 @@ class AttentionPlan:
                 at = {s.q_start: s.start_pos for s in ctx.spans if s.q_len == 1}
                 work = ctx.rt.k.attention_decode_work([at[t] for t in singles], window)
                 self.decode_work = torch.tensor(work, dtype=torch.int32).to(dev)
-        if n_single and self.max_chunks > 1:
+        if n_single:
             n = ctx.rt.k.attention_decode_workspace(n_single, n_heads, head_dim, self.max_chunks)
             self.partial = torch.empty(n, dtype=torch.float32, device=dev)
 
@@ -186,30 +186,16 @@ class GQAttention(Mixer):
             self.position.load(store, rt)
 
     # ------------------------------------------------------------------ the step
-    def takes_unscaled_rows(self, ctx) -> bool:
-        k = ctx.rt.k
-        return (isinstance(self.w_qkv, PackedMatrix)
-                and k.gemm_norm_fold_ok(ctx.n_tokens, self.q_dim + 2 * self.kv_dim, self.hidden, MODE_STORE)
-                and k.gemm_norm_fold_ok(ctx.n_tokens, self.q_dim, self.hidden, MODE_STORE))
-
-    def folds_following_norm(self, ctx) -> bool:
-        return (isinstance(self.w_o, PackedMatrix)
-                and ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.hidden, self.q_dim, MODE_ADD_F32))
-
     def finishes_following_norm(self, ctx) -> bool:
         return isinstance(self.w_o, PackedMatrix) and ctx.rt.k.gemm_then_norm_ok(ctx.n_tokens, self.hidden, self.q_dim)
 
-    def forward(self, ctx, binding: CacheBinding, h, residual, fold=None) -> None:
+    def forward(self, ctx, binding: CacheBinding, h, residual, following=None) -> None:
         k = ctx.rt.k
         T = h.shape[0]
-        scaled = {}
-        if isinstance(h, UnscaledRows):
-            h, scaled = h.values, {"row_squares": h.squares, "eps": h.eps}
         group = ctx.cache.group(binding.group)
         k_cache, v_cache = group.layer(binding.index)
         # values are kept position-contiguous: a page of them is [heads, head_dim, page_size]
         v_cache = v_cache.view(v_cache.shape[0], self.nkv, self.hd, group.page_size)
-        mark = ctx.ws.mark()
         qkv = ctx.ws.take((T, self.q_dim + 2 * self.kv_dim), ctx.rt.dtype)
         if self.position is not None:
             table, rotary = self.position.tables(ctx), self.position.rotary_dim
@@ -222,11 +208,11 @@ class GQAttention(Mixer):
             w, bias = self.w_qkv[:self.q_dim], None if self.b_qkv is None else self.b_qkv[:self.q_dim]
         if isinstance(w, PackedMatrix) and k.gemm_qkv_rope_ok(T, w.shape[0], self.hidden, self.hd, rotary):
             # product, rotation and the store into the pages in one launch (a short step) or with the
-            # rotation and the store done by the kernel that adds a split product's parts
+            # rotation and the store done by the kernel that adds the sums of the product's segments
             k.gemm_qkv_rope(h, w, bias, qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache,
-                            self.nh, self.nkv, self.hd, group.page_size, binding.writes, **scaled)
+                            self.nh, self.nkv, self.hd, group.page_size, binding.writes)
         else:
-            k.gemm(h, w, qkv[:, :w.shape[0]], bias, MODE_STORE, **scaled)
+            k.gemm(h, w, qkv[:, :w.shape[0]], bias, MODE_STORE)
             k.rope_kv_write(qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache, self.nh,
                             self.nkv, self.hd, rotary, group.page_size, binding.writes)
         att = ctx.ws.take((T, self.q_dim), ctx.rt.dtype)
@@ -243,8 +229,7 @@ class GQAttention(Mixer):
             k.attention(qkv, qkv.stride(0), k_cache, v_cache, group.block_table, ctx.positions, ctx.seq_rows, att,
                         self.nh, self.nkv, self.hd, group.page_size, self.window, self.scale)
         k.gemm(att, self.w_o, residual, self.b_o, MODE_ADD_F32,
-               following_norm=None if fold is None else fold.following_norm())
-        ctx.ws.release(mark)
+               following_norm=None if following is None else following.as_argument())
 
 
 register_mixer("gqa_attention", GQAttention)

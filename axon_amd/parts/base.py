@@ -88,45 +88,27 @@ class Part:
         (device, dtype, kernels)."""
 
 
-class UnscaledRows:
-    """Rows of a norm that still lack their scale: `values` [T, size] in the compute dtype hold
-    x * gain, `squares` float32 [T, size / 16] the sums of x^2 over the 16-column parts of each
-    row, `eps` the norm's constant.  The product that reads them multiplies its result by
-    1 / sqrt(sum(squares) / size + eps): the scale is common to a row, so it commutes with the
-    product, and the norm needs no pass of its own over the rows."""
+class FollowingNorm:
+    """A norm handed to the part that runs before it (an option, never a duty: a part that does
+    not offer it is followed by the norm's own pass).  Where the last product of a part adds into
+    the residual stream through a kernel that holds the finished rows anyway, that kernel can
+    write the norm of the new rows as well: `values` [T, size] in the compute dtype, the same
+    bits as the norm's own pass would give.  The part after the norm then reads `values`."""
 
-    def __init__(self, values, squares, eps: float):
-        self.values, self.squares, self.eps = values, squares, eps
+    def __init__(self, gain, eps: float, values):
+        self.gain, self.eps, self.values = gain, eps, values
 
-    @property
-    def shape(self):
-        return self.values.shape
-
-
-class NormFold:
-    """A norm handed to the part that runs before it: that part's last product, which adds into
-    the residual stream, does the norm's work in its epilogue, and `rows()` is then what the
-    part after the norm reads.  In parts (`squares` given): the product writes `values` =
-    residual * gain and `squares` (see UnscaledRows), and the next product applies the rows'
-    scale.  Whole (`squares` None): the product writes the finished norm into `values`."""
-
-    def __init__(self, gain, eps: float, values, squares):
-        self.gain, self.eps, self.values, self.squares = gain, eps, values, squares
-
-    def following_norm(self):
-        return (self.gain, self.values, self.squares, self.eps)
-
-    def rows(self):
-        return self.values if self.squares is None else UnscaledRows(self.values, self.squares, self.eps)
+    def as_argument(self):
+        return (self.gain, self.values, self.eps)
 
 
 class Norm(Part):
     def forward(self, ctx, x, out=None):
         raise NotImplementedError
 
-    def fold(self, ctx, n_rows: int, whole: bool = False) -> Optional[NormFold]:
-        """This norm as work for the neighbouring products (with buffers for `n_rows` rows), or
-        None if it has to run on its own.  `whole`: for a product that finishes the norm itself."""
+    def following(self, ctx, n_rows: int) -> Optional[FollowingNorm]:
+        """This norm as work for the product before it (with a buffer for `n_rows` rows), or None
+        if it always runs on its own (the default)."""
         return None
 
 
@@ -162,17 +144,9 @@ class Mixer(Part):
         this many positions each."""
         return 0
 
-    def takes_unscaled_rows(self, ctx) -> bool:
-        """Whether `h` may be UnscaledRows in this step (the first product applies the scale)."""
-        return False
-
-    def folds_following_norm(self, ctx) -> bool:
-        """Whether `forward` takes a NormFold (in parts) as a further argument in this step and fills it."""
-        return False
-
     def finishes_following_norm(self, ctx) -> bool:
-        """Whether `forward` takes a whole NormFold in this step: its last product also writes the
-        finished norm of the rows it has added into."""
+        """Whether `forward` takes a FollowingNorm as a further argument in this step: its last
+        product also writes the finished norm of the rows it has added into.  Optional."""
         return False
 
     def forward(self, ctx, binding: CacheBinding, h, residual) -> None:
@@ -180,13 +154,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    def takes_unscaled_rows(self, ctx) -> bool:
-        return False
-
-    def folds_following_norm(self, ctx) -> bool:
-        return False
-
     def finishes_following_norm(self, ctx) -> bool:
+        """As for a mixer: optional."""
         return False
 
     def forward(self, ctx, h, residual) -> None:
@@ -194,32 +163,38 @@ class FeedForward(Part):
 
 
 class Block(Part):
-    """An arrangement: built from the layer's parts, not from a spec of its own."""
+    """An arrangement: built from the layer's parts, not from a spec of its own.
+
+    A block that wants the speed of norms finished by the product before them calls
+    `run_part` for its mixer and feed-forward and `normed` for its norms (below); one that does
+    not calls the parts plainly, and everything still works."""
 
     def __init__(self, norm_factory: Callable[[str], Norm], mixer: Mixer, feed_forward: FeedForward, prefix: str):
         super().__init__({}, prefix)
         self.mixer = mixer
         self.feed_forward = feed_forward
 
-    def first_norm_fold(self, ctx, n_rows: int, whole: bool = False) -> Optional[NormFold]:
-        """The block's first norm as work for the block before it (see NormFold; `whole` if that
-        block finishes the norm itself), or None: then `forward` is called without `unscaled`."""
+    def first_norm(self) -> Optional[Norm]:
+        """The norm this block starts with, if the block before may do its work; None: it may not."""
         return None
 
-    def folds_following_norm(self, ctx) -> bool:
-        """Whether `forward` takes the next block's first norm (in parts) as `fold_next` in this step."""
-        return False
+    def last_part(self):
+        """The part whose product ends this block (it may finish the next block's first norm)."""
+        return None
 
-    def finishes_following_norm(self, ctx) -> bool:
-        """Whether `forward` takes the next block's first norm whole as `fold_next` in this step."""
-        return False
-
-    def forward(self, ctx, binding: CacheBinding, x, unscaled: Optional[UnscaledRows] = None,
-                fold_next: Optional[NormFold] = None) -> None:
-        """Update the residual stream x in place.  `unscaled`: the first norm's rows, already left
-        by the block before; `fold_next`: to be filled for the block after (both only if this
-        block offered it)."""
+    def forward(self, ctx, binding: CacheBinding, x, normed=None, following: Optional[FollowingNorm] = None) -> None:
+        """Update the residual stream x in place.  `normed`: the first norm's rows, already left by
+        the block before; `following`: the next block's first norm, to be finished by this block's
+        last product (both only if this block offered it through `first_norm` / `last_part`)."""
         raise NotImplementedError
+
+    # what a block's `forward` is put together from
+    @staticmethod
+    def following_of(ctx, part, norm: Optional[Norm], n_rows: int) -> Optional[FollowingNorm]:
+        """`norm` as work for `part`'s last product in this step, or None."""
+        if norm is None or part is None or not part.finishes_following_norm(ctx):
+            return None
+        return norm.following(ctx, n_rows)
 
 
 # --------------------------------------------------------------------------- registries

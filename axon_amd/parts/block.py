@@ -10,9 +10,8 @@ from typing import List
 
 from .base import Block, CacheBinding, TensorDecl, register_block
 
-# A norm between two products can be folded into them where both offer it (short steps in
-# bfloat16: the products then run in kernels that take it), or done whole by the product before
-# it where that one offers it (steps whose products split K): the block asks its parts.
+# A norm behind a product whose kernel holds the finished rows anyway can be written by that
+# kernel (the same bits as the norm's own pass): the block asks its parts, step by step.
 
 
 class PreNormBlock(Block):
@@ -32,36 +31,25 @@ class PreNormBlock(Block):
         for part in (self.norm1, self.mixer, self.norm2, self.feed_forward):
             part.load(store, rt)
 
-    def first_norm_fold(self, ctx, n_rows: int, whole: bool = False):
-        if whole:
-            return self.norm1.fold(ctx, n_rows, whole=True)
-        return self.norm1.fold(ctx, n_rows) if self.mixer.takes_unscaled_rows(ctx) else None
+    def first_norm(self):
+        return self.norm1
 
-    def folds_following_norm(self, ctx) -> bool:
-        return self.feed_forward.folds_following_norm(ctx)
+    def last_part(self):
+        return self.feed_forward
 
-    def finishes_following_norm(self, ctx) -> bool:
-        return self.feed_forward.finishes_following_norm(ctx)
-
-    def forward(self, ctx, binding: CacheBinding, x, unscaled=None, fold_next=None) -> None:
-        mark = ctx.ws.mark()
-        h = unscaled if unscaled is not None else self.norm1.forward(ctx, x)
-        fold = None
-        if self.mixer.finishes_following_norm(ctx):
-            fold = self.norm2.fold(ctx, x.shape[0], whole=True)
-        elif self.mixer.folds_following_norm(ctx) and self.feed_forward.takes_unscaled_rows(ctx):
-            fold = self.norm2.fold(ctx, x.shape[0])
-        if fold is not None:
-            self.mixer.forward(ctx, binding, h, x, fold)
-            h = fold.rows()
+    def forward(self, ctx, binding: CacheBinding, x, normed=None, following=None) -> None:
+        h = normed if normed is not None else self.norm1.forward(ctx, x)
+        second = self.following_of(ctx, self.mixer, self.norm2, x.shape[0])
+        if second is not None:
+            self.mixer.forward(ctx, binding, h, x, second)
+            h = second.values
         else:
             self.mixer.forward(ctx, binding, h, x)
             h = self.norm2.forward(ctx, x)
-        if fold_next is not None:
-            self.feed_forward.forward(ctx, h, x, fold_next)
+        if following is not None:
+            self.feed_forward.forward(ctx, h, x, following)
         else:
             self.feed_forward.forward(ctx, h, x)
-        ctx.ws.release(mark)
 
 
 register_block("prenorm", PreNormBlock)

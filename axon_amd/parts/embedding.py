@@ -32,7 +32,7 @@ class TokenEmbedding(Part):
 
     def forward(self, ctx, out=None):
         if out is None:
-            out = ctx.ws.take_persistent((ctx.n_tokens, self.hidden), torch.float32)
+            out = ctx.ws.take((ctx.n_tokens, self.hidden), torch.float32)
         return ctx.rt.k.embed(ctx.tokens, self.table, out)
 
 

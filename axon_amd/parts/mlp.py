@@ -10,7 +10,7 @@ from __future__ import annotations
 from typing import List
 
 from ..kernels import MODE_ADD_F32, MODE_SWIGLU, PackedMatrix
-from .base import FeedForward, TensorDecl, UnscaledRows, register_feed_forward
+from .base import FeedForward, TensorDecl, register_feed_forward
 
 
 class SwiGLUMLP(FeedForward):
@@ -33,30 +33,15 @@ class SwiGLUMLP(FeedForward):
         self.w_down = rt.k.prepare_weight(store.matrix(self.n["down"]))
         store.forget(self.n["down"])
 
-    def takes_unscaled_rows(self, ctx) -> bool:
-        return (isinstance(self.w_gate_up, PackedMatrix)
-                and ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.ffn, self.hidden, MODE_SWIGLU))
-
-    def folds_following_norm(self, ctx) -> bool:
-        return (isinstance(self.w_down, PackedMatrix)
-                and ctx.rt.k.gemm_norm_fold_ok(ctx.n_tokens, self.hidden, self.ffn, MODE_ADD_F32))
-
     def finishes_following_norm(self, ctx) -> bool:
         return isinstance(self.w_down, PackedMatrix) and ctx.rt.k.gemm_then_norm_ok(ctx.n_tokens, self.hidden, self.ffn)
 
-    def forward(self, ctx, h, residual, fold=None) -> None:
+    def forward(self, ctx, h, residual, following=None) -> None:
         k = ctx.rt.k
-        T = h.shape[0]
-        mark = ctx.ws.mark()
-        act = ctx.ws.take((T, self.ffn), ctx.rt.dtype)
-        # silu(gate h) * up h, in the product's epilogue
-        if isinstance(h, UnscaledRows):
-            k.gemm(h.values, self.w_gate_up, act, None, MODE_SWIGLU, row_squares=h.squares, eps=h.eps)
-        else:
-            k.gemm(h, self.w_gate_up, act, None, MODE_SWIGLU)
+        act = ctx.ws.take((h.shape[0], self.ffn), ctx.rt.dtype)
+        k.gemm(h, self.w_gate_up, act, None, MODE_SWIGLU)       # silu(gate h) * up h, in the product's epilogue
         k.gemm(act, self.w_down, residual, None, MODE_ADD_F32,
-               following_norm=None if fold is None else fold.following_norm())
-        ctx.ws.release(mark)
+               following_norm=None if following is None else following.as_argument())
 
 
 register_feed_forward("swiglu_mlp", SwiGLUMLP)

@@ -9,7 +9,7 @@ from typing import List, Optional
 
 import torch
 
-from .base import Norm, NormFold, TensorDecl, register_norm
+from .base import FollowingNorm, Norm, TensorDecl, register_norm
 
 
 class RMSNorm(Norm):
@@ -34,18 +34,9 @@ class RMSNorm(Norm):
             out = ctx.ws.take((n, self.size), ctx.rt.dtype)
         return ctx.rt.k.rmsnorm(x, self.gain, self.eps, out, rows)
 
-    def fold(self, ctx, n_rows: int, whole: bool = False) -> Optional[NormFold]:
-        """In parts: the product before the norm leaves x * gain and the sums of squares, the
-        product after it applies 1/sqrt(mean + eps): the same formula, the row's scale moved
-        behind the product (it is common to the row).  Whole: the product before the norm
-        writes the finished rows."""
-        if whole:
-            return NormFold(self.gain, self.eps, ctx.ws.take((n_rows, self.size), ctx.rt.dtype), None)
-        if self.size % 16:
-            return None
-        values = ctx.ws.take((n_rows, self.size), ctx.rt.dtype)
-        squares = ctx.ws.take((n_rows, self.size // 16), torch.float32)
-        return NormFold(self.gain, self.eps, values, squares)
+    def following(self, ctx, n_rows: int) -> Optional[FollowingNorm]:
+        """The product before the norm writes the finished rows (where its kernel offers it)."""
+        return FollowingNorm(self.gain, self.eps, ctx.ws.take((n_rows, self.size), ctx.rt.dtype))
 
 
 register_norm("rmsnorm", RMSNorm)

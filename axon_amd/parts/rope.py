@@ -41,7 +41,7 @@ class RotaryEncoding(PositionEncoding):
         """float32 [T, rotary_dim / 2, 2] for the positions of this step (made once per step)."""
         t = ctx.shared.get(self.key)
         if t is None:
-            t = ctx.ws.take_persistent((ctx.n_tokens, self.rotary_dim // 2, 2), torch.float32)
+            t = ctx.ws.take((ctx.n_tokens, self.rotary_dim // 2, 2), torch.float32)
             ctx.rt.k.rope_table(ctx.positions, self._freqs, t)
             ctx.shared[self.key] = t
         return t

@@ -207,36 +207,63 @@ def test_gemm_with_the_gated_epilogue(dtype, M, F, K):
         k.gemm(x, w, out, rnd(F).cuda(), MODE_SWIGLU)
 
 
+ROW_COUNTS = (1, 2, 3, 7, 16, 17, 32, 33, 64, 65, 128, 130, 256, 257, 1000, 2049)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_rows_do_not_depend_on_the_batch(dtype):
-    """The same row of x gives the same bits whatever rows ride along.  float32: for any number
-    of rows.  bfloat16: among batches of up to 16 rows (the decoding kernel), among those of 17
-    to 64, of 65 to 256 and of 257 to 2048 (tiles with K split between blocks, by (N, K) alone)
-    and among larger ones; between the classes a row differs by the rounding of 32-bit sums."""
+    """The same row of x gives the same bits whatever rows ride along, in both builds and for any
+    number of rows (src/lm.rs:272-278): every kernel a product may meet adds in the one order its
+    matrix fixes."""
     k = kernels(dtype)
-    for N, K in [(96, 80), (256, 512), (130, 1000), (512, 1024), (300, 4096), (200, 8192)]:
+    for N, K in [(96, 80), (256, 512), (130, 1000), (512, 1024), (300, 4096), (200, 8192), (4100, 256)]:
         x, _ = as_dtype(rnd(2100, K, seed=14), dtype)
         w, _ = as_dtype(rnd(N, K, seed=15, scale=0.2), dtype)
         w = packed(k, w)
-        whole = {}
-        for rows in (16, 64, 256, 2048, 2100):
-            whole[rows] = torch.empty(rows, N, dtype=torch.float32, device="cuda")
-            k.gemm(x[:rows], w, whole[rows], None, MODE_STORE_F32)
-        for m in (1, 3, 16, 17, 33, 64, 65, 130, 256, 257, 300, 1000, 2049):
+        whole = torch.empty(2100, N, dtype=torch.float32, device="cuda")
+        k.gemm(x, w, whole, None, MODE_STORE_F32)
+        for m in ROW_COUNTS:
             part = torch.empty(m, N, dtype=torch.float32, device="cuda")
             k.gemm(x[:m], w, part, None, MODE_STORE_F32)
-            cls = 2100 if dtype == "float32" else 16 if m <= 16 else 64 if m <= 64 else 256 if m <= 256 else 2048 if m <= 2048 else 2100
-            assert torch.equal(part, whole[cls][:m]), (N, K, m)
-        for rows in (16, 64, 256, 2048):
-            assert (whole[rows] - whole[2100][:rows]).abs().max() <= 1e-5 * whole[2100].abs().max()
+            assert torch.equal(part, whole[:m]), (N, K, m)
 
 
-@pytest.mark.parametrize("M,H,F", [(17, 256, 1024), (64, 384, 2048), (100, 256, 1024), (256, 128, 512), (300, 256, 8192),
-                                   (40, 4352, 512)])
+# the products of a layer of the measured sizes (hidden, q rows, kv rows, feed-forward width, head_dim)
+LAYER_SIZES = {"7b": (3584, 3584, 512, 18944, 128), "14b": (5120, 5120, 1024, 13824, 128)}
+
+
+@pytest.mark.parametrize("sizes", sorted(LAYER_SIZES))
+def test_products_of_the_measured_sizes_give_a_row_the_same_bits_in_any_step(sizes):
+    """bfloat16, the matrices of a Qwen2.5-7B and a 14B layer, every epilogue the model uses: a
+    row's result does not depend on the number of rows in the step, from 1 to 2,049."""
+    k = kernels("bfloat16")
+    hidden, q_dim, kv_dim, ffn, hd = LAYER_SIZES[sizes]
+    most = max(ROW_COUNTS)
+    cases = [("qkv", q_dim + 2 * kv_dim, hidden, MODE_STORE), ("o", hidden, q_dim, MODE_ADD_F32),
+             ("gate_up", ffn, hidden, MODE_SWIGLU), ("down", hidden, ffn, MODE_ADD_F32), ("head", 4096 + 40, hidden, MODE_STORE_F32)]
+    for name, N, K, mode in cases:
+        x, _ = as_dtype(rnd(most, K, seed=16), "bfloat16")
+        w, _ = as_dtype(rnd(2 * N if mode == MODE_SWIGLU else N, K, seed=17, scale=0.05), "bfloat16")
+        w = packed(k, w, gated=mode == MODE_SWIGLU)
+        assert k.gemm_segments(N, K, mode == MODE_SWIGLU) in (1, 2, 4, 8)
+        bias = rnd(N, seed=18).cuda() if name == "qkv" else None
+        dt = torch.float32 if mode in (MODE_ADD_F32, MODE_STORE_F32) else torch.bfloat16
+        base = rnd(most, N, seed=19).to(dt).cuda()
+        whole = base.clone()
+        k.gemm(x, w, whole, bias, mode)
+        for m in ROW_COUNTS:
+            part = base[:m].clone()
+            k.gemm(x[:m], w, part, bias, mode)
+            assert torch.equal(part, whole[:m]), (sizes, name, m)
+
+
+@pytest.mark.parametrize("M,H,F", [(65, 384, 2048), (100, 256, 1024), (256, 128, 512), (300, 256, 8192),
+                                   (128, 4352, 512)])
 def test_gemm_followed_by_the_whole_norm(M, H, F):
     """residual += a . Wo^T + bias; h = rmsnorm(residual) * gain, the norm written by the kernel
-    that adds the split product's sums: the same bits as the product and the norm one after the
-    other, and right against the plain formulas.  Where K is not split the kernels refuse."""
+    that adds the sums of the product's segments: the same bits as the product and the norm one
+    after the other, and right against the plain formulas.  Where no such kernel runs the
+    product refuses."""
     k = kernels("bfloat16")
     eps = 2e-5
     assert k.gemm_then_norm_ok(M, H, F)
@@ -253,52 +280,18 @@ def test_gemm_followed_by_the_whole_norm(M, H, F):
         h1 = k.rmsnorm(x1, gain, eps, torch.empty(M, H, dtype=torch.bfloat16, device="cuda"))
         x2 = res.clone().cuda()
         h2 = torch.full((M, H), float("nan"), dtype=torch.bfloat16, device="cuda")
-        k.gemm(a, w, x2, b, MODE_ADD_F32, following_norm=(gain, h2, None, eps))
+        k.gemm(a, w, x2, b, MODE_ADD_F32, following_norm=(gain, h2, eps))
         assert torch.equal(x1, x2) and torch.equal(h1, h2)
         x_ref = res.double() + ar @ wor.T + (0 if b is None else bias.double())
         h_ref = P.rms_norm(x_ref, gain.cpu().double(), eps)
         assert (h2.cpu().double() - h_ref).abs().max() <= tol("bfloat16", h_ref, bf16=1.5e-2)
-    assert not k.gemm_then_norm_ok(8, H, F) and not k.gemm_then_norm_ok(3000, H, F)
+        # and the rows are those of a step of eight
+        x3 = res[:8].clone().cuda()
+        k.gemm(a[:8], w, x3, b, MODE_ADD_F32)
+        assert torch.equal(x3, x2[:8])
+    assert not k.gemm_then_norm_ok(8, H, F) and not k.gemm_then_norm_ok(3000, 16384, F)
     with pytest.raises(KernelError):
-        k.gemm(a[:8], w, res[:8].clone().cuda(), None, MODE_ADD_F32, following_norm=(gain, h2[:8], None, eps))
-
-
-@pytest.mark.parametrize("M,H,F", [(1, 64, 128), (8, 192, 320), (16, 448, 64), (5, 4608, 64), (13, 128, 192)])
-def test_gemm_with_a_norm_folded_in(M, H, F):
-    """residual += a . Wo^T; h = rmsnorm(residual) * gain; out = h . W^T + bias, with the norm done
-    by the two products: the first leaves residual * gain and the rows' sums of squares, the
-    second scales its result.  Against the plain norm between plain products."""
-    k = kernels("bfloat16")
-    eps = 3e-5
-    a, ar = as_dtype(rnd(M, F, seed=40), "bfloat16")
-    wo, wor = as_dtype(rnd(H, F, seed=41, scale=0.3), "bfloat16")
-    res = rnd(M, H, seed=42, scale=2.0)
-    res[0] *= 40.0                                        # a row of another magnitude: the scale is per row
-    for gain_dt in (torch.float32, torch.bfloat16):
-        gain = (1.0 + 0.3 * rnd(H, seed=43)).to(gain_dt)
-        x_ref = res.double() + ar @ wor.T
-        h_ref = P.rms_norm(x_ref, gain.double(), eps)
-        assert k.gemm_norm_fold_ok(M, H, F, MODE_ADD_F32)
-        x = res.clone().cuda()
-        values = torch.empty(M, H, dtype=torch.bfloat16, device="cuda")
-        squares = torch.full((M, H // 16), float("nan"), dtype=torch.float32, device="cuda")
-        k.gemm(a, packed(k, wo), x, None, MODE_ADD_F32, following_norm=(gain.cuda(), values, squares, eps))
-        assert (x.cpu().double() - x_ref).abs().max() <= 2e-5 * math.sqrt(F) * x_ref.abs().max()
-        got_sq = squares.cpu().double().sum(1)
-        assert ((got_sq - (x_ref ** 2).sum(1)).abs() <= 1e-5 * (x_ref ** 2).sum(1)).all()
-        # the consumer: a plain product with bias, and the gated one
-        for N in (48, 272):
-            w, wr = as_dtype(rnd(N, H, seed=44, scale=0.2), "bfloat16")
-            bias = rnd(N, seed=45)
-            out = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
-            k.gemm(values, packed(k, w), out, bias.cuda(), MODE_STORE, row_squares=squares, eps=eps)
-            want = h_ref @ wr.T + bias.double()
-            assert (out.cpu().double() - want).abs().max() <= tol("bfloat16", want, 0, 1e-2)
-        wg, wgr = as_dtype(rnd(2 * 80, H, seed=46, scale=0.2), "bfloat16")
-        out = torch.empty(M, 80, dtype=torch.bfloat16, device="cuda")
-        k.gemm(values, packed(k, wg, gated=True), out, None, MODE_SWIGLU, row_squares=squares, eps=eps)
-        want = P.swiglu(h_ref @ wgr[:80].T, h_ref @ wgr[80:].T)
-        assert (out.cpu().double() - want).abs().max() <= tol("bfloat16", want, 0, 1e-2)
+        k.gemm(a[:8], w, res[:8].clone().cuda(), None, MODE_ADD_F32, following_norm=(gain, h2[:8], eps))
 
 
 @pytest.mark.parametrize("M,nh,nkv,hd,hidden,page", [(1, 4, 2, 32, 64, 8), (8, 6, 2, 64, 192, 16), (16, 7, 1, 128, 256, 8),
@@ -311,7 +304,7 @@ def test_qkv_product_with_rotation_and_cache_store_in_one(M, nh, nkv, hd, hidden
     k = kernels("bfloat16")
     width = (nh + 2 * nkv) * hd
     assert k.gemm_qkv_rope_ok(M, width, hidden, hd, hd) and k.gemm_qkv_rope_ok(M, nh * hd, hidden, hd, hd)
-    assert not k.gemm_qkv_rope_ok(M, width, hidden, hd, hd // 2) and not k.gemm_qkv_rope_ok(17, width, 64, hd, hd)
+    assert not k.gemm_qkv_rope_ok(M, width, hidden, hd, hd // 2) and not k.gemm_qkv_rope_ok(100, width, 64, hd, hd)
     assert not k.gemm_qkv_rope_ok(M, 48 * (nh + 2 * nkv), hidden, 48, 48)
     assert not kernels("float32").gemm_qkv_rope_ok(M, width, hidden, hd, hd)
     x, _ = as_dtype(rnd(M, hidden, seed=50), "bfloat16")
@@ -345,20 +338,6 @@ def test_qkv_product_with_rotation_and_cache_store_in_one(M, nh, nkv, hd, hidden
         for a, b in zip(got, want):
             assert torch.equal(a, b)
         assert write_kv == bool((got[1] != 7.0).any())
-
-
-def test_gemm_refuses_a_norm_it_cannot_fold():
-    k = kernels("bfloat16")
-    assert not k.gemm_norm_fold_ok(17, 64, 64, MODE_STORE)          # more rows than a folded step takes
-    assert not k.gemm_norm_fold_ok(8, 64, 70, MODE_STORE)           # K that the matrix-core kernels refuse
-    assert not kernels("float32").gemm_norm_fold_ok(8, 64, 64, MODE_STORE)
-    x = torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda")
-    w = k.pack_matrix(torch.zeros(64, 64, dtype=torch.bfloat16, device="cuda"))
-    out = torch.zeros(17, 64, dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(KernelError):
-        k.gemm(x, w, out, None, MODE_STORE, row_squares=torch.zeros(17, 4, device="cuda"), eps=1e-6)
-    with pytest.raises(KernelError):                                 # sums of squares of the wrong shape
-        k.gemm(x[:8], w, out[:8], None, MODE_STORE, row_squares=torch.zeros(8, 5, device="cuda"), eps=1e-6)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -528,6 +507,36 @@ def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
     assert torch.equal(named, plain) and (plain[:first].cpu().double() - ref[:first]).abs().max() <= tol("bfloat16", ref, bf16=1.5e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page,T,window", [
+    (28, 4, 128, 16, 700, 0), (40, 8, 128, 16, 300, 0), (4, 2, 64, 8, 333, 0), (6, 1, 128, 64, 600, 150),
+    (32, 1, 64, 16, 200, 0), (3, 3, 128, 32, 1100, 0)])
+def test_a_position_gets_the_same_bits_from_the_prompt_kernel_and_the_decoding_kernel(nh, nkv, hd, page, T, window):
+    """Every position of a sequence once as a row of a prompt portion (tiles cut at several places)
+    and once as a single decoding token: bit for bit the same result, whatever the cut, because
+    both kernels fold the same blocks of 64 positions with the same instructions
+    (src/lm.rs:272-278; docs/determinism.md:53-57 of the reference)."""
+    k = kernels("bfloat16")
+    assert k.attention_fast_ok(hd, page, nh, nkv)
+    q, kc, vc, table, ref = _mfma_case(nh, nkv, hd, page, T, window, seed=11)
+    pos = torch.arange(T, dtype=torch.int32).cuda()
+    rows = torch.zeros(T, dtype=torch.int32).cuda()
+    scale = 1.0 / math.sqrt(hd)
+    ch = k.attention_decode_chunk
+    chunks = max((p - ((max(0, p + 1 - window) if window else 0) // ch * ch)) // ch + 1 for p in range(T))
+    partial = torch.empty(k.attention_decode_workspace(T, nh, hd, chunks), dtype=torch.float32, device="cuda")
+    decoded = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+    k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, decoded, T, partial, chunks, nh, nkv, hd, page, window, scale)
+    assert (decoded.cpu().double() - ref).abs().max() <= tol("bfloat16", ref, bf16=1.5e-2)
+    for cuts in ([0], [0, 2, 7, 64, 130, 131], [0, 63, 129, 190]):
+        cuts = [c for c in cuts if c < T] + [T]
+        tiles = [(a + o, min(128, b - a - o)) for a, b in zip(cuts, cuts[1:]) for o in range(0, b - a, 128)]
+        tiles = [t for t in tiles if t[1] >= 1]
+        prompt = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+        k.attention_prefill(q, nh * hd, kc, vc, table, pos, rows, prompt, torch.tensor(tiles, dtype=torch.int32).cuda(),
+                            nh, nkv, hd, page, window, scale)
+        assert torch.equal(prompt, decoded), cuts
+
+
 def test_matrix_core_attention_finds_a_far_key_and_respects_the_windows_edge():
     k = kernels("bfloat16")
     nh, nkv, hd, page, T = 4, 2, 128, 16, 700
@@ -566,7 +575,7 @@ def test_matrix_core_attention_finds_a_far_key_and_respects_the_windows_edge():
 def test_matrix_core_attention_refuses_other_sizes():
     k = kernels("bfloat16")
     assert not k.attention_fast_ok(80, 16, 4, 2) and not k.attention_fast_ok(128, 5, 4, 2)
-    assert not k.attention_fast_ok(128, 16, 34, 2)             # a group of 17 heads
+    assert not k.attention_fast_ok(128, 16, 66, 2)             # a group of 33 heads
     assert not kernels("float32").attention_fast_ok(128, 16, 4, 2)
     q = torch.zeros(4, 160, dtype=torch.bfloat16, device="cuda")
     kc = torch.zeros(2, 1, 16, 80, dtype=torch.bfloat16, device="cuda")

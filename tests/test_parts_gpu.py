@@ -140,66 +140,13 @@ def test_prenorm_block_arrangement(dtype):
     assert (x.cpu().double() - r).abs().max() <= tol(dtype, r, 1e-5, 3e-2)
 
 
-def test_prenorm_block_with_the_norms_folded_into_the_products():
-    """A short step in bfloat16 whose widths the matrix-core kernels take: the block runs no norm
-    of its own (the products around each norm do its work), takes its first norm's rows from
-    the block before and leaves the next block's; against the plain formulas."""
-    dtype = "bfloat16"
-    hidden, nh, nkv, hd, ffn, eps, T = 128, 4, 2, 32, 192, 1e-3, 9
-    mixer = build_part("mixer", PartSpec("gqa_attention", {
-        "hidden_size": hidden, "num_heads": nh, "num_kv_heads": nkv, "head_dim": hd, "qkv_bias": True,
-        "position": PartSpec("rope", {"head_dim": hd, "theta": 100.0})}), "model.layers.0.")
-    ffn_part = build_part("feed_forward", PartSpec("swiglu_mlp", {"hidden_size": hidden, "intermediate_size": ffn}),
-                          "model.layers.0.")
-    block = build_block("prenorm", PartSpec("rmsnorm", {"size": hidden, "eps": eps}), mixer, ffn_part, "model.layers.0.")
-    from test_plain import random_weights
-    cfg = P.PlainConfig(1, hidden, nh, nkv, hd, 100.0, eps, True)
-    w = {k: rounded(v.float(), dtype) for k, v in random_weights(cfg, ffn, 10, 0.3).items() if "layers.0" in k}
-    p = "model.layers.0."
-    w[p + "input_layernorm.weight"] = 1.0 + 0.5 * rnd(hidden, seed=3)         # gains that matter
-    w[p + "post_attention_layernorm.weight"] = 1.0 + 0.5 * rnd(hidden, seed=4)
-    h = PartHarness(dtype, mixer.cache_spec())
-    load(block, w, h)
-    ctx = h.ctx([0] * T)
-    assert block.folds_following_norm(ctx) and mixer.takes_unscaled_rows(ctx) and mixer.folds_following_norm(ctx)
-    x0 = rnd(T, hidden, seed=9, scale=3.0)
-    x0[2] *= 30.0                                                             # rows of different magnitudes
-    wd = {k: v.double() for k, v in w.items()}
-    # what the block before would have left: the first norm's rows without their scale
-    first = block.first_norm_fold(ctx, T)
-    assert first is not None
-    first.values.copy_((x0 * w[p + "input_layernorm.weight"]).to(torch.bfloat16))
-    first.squares.copy_((x0.double() ** 2).view(T, hidden // 16, 16).sum(-1).float())
-    next_gain = (1.0 + 0.5 * rnd(hidden, seed=5)).cuda()
-    nxt = first.__class__(next_gain, 1e-5, torch.empty(T, hidden, dtype=torch.bfloat16, device="cuda"),
-                          torch.empty(T, hidden // 16, dtype=torch.float32, device="cuda"))
-    calls = []
-    real = h.rt.k.rmsnorm
-    h.rt.k.rmsnorm = lambda *a, **kw: (calls.append(1), real(*a, **kw))[1]
-    try:
-        x = x0.clone().cuda()
-        block.forward(ctx, CacheBinding(0, 0, True), x, first.rows(), nxt)
-    finally:
-        h.rt.k.rmsnorm = real
-    assert not calls                                                          # no norm ran on its own
-    r = x0.double()
-    r = r + P.attention_block(cfg, wd, 0, P.rms_norm(r, wd[p + "input_layernorm.weight"], eps), torch.arange(T))
-    r = r + P.mlp_block(wd, 0, P.rms_norm(r, wd[p + "post_attention_layernorm.weight"], eps))
-    assert (x.cpu().double() - r).abs().max() <= tol(dtype, r, 1e-5, 3e-2)
-    rows = nxt.rows()
-    assert (rows.values.cpu().double() - r * next_gain.cpu().double()).abs().max() <= tol(dtype, r, 0, 3e-2)
-    assert ((rows.squares.cpu().double().sum(1) - (r ** 2).sum(1)).abs() <= 2e-2 * (r ** 2).sum(1)).all()
-    # more rows than a folded step takes: the parts say so and the block runs its norms itself
-    big = PartHarness(dtype, mixer.cache_spec())
-    assert not mixer.takes_unscaled_rows(big.ctx([0] * 17)) and block.first_norm_fold(big.ctx([0] * 17), 17) is None
-
-
 def test_prenorm_block_whose_products_finish_the_norms_behind_them():
-    """A step of some tens of rows in bfloat16 with products wide enough to split K: the output
-    projection writes the second norm's rows and the down projection the next block's first
-    norm, whole; only a norm nobody did for the block runs on its own.  Against the plain formulas."""
+    """A step of some tens of rows in bfloat16 with narrow products, whose segments of K run in
+    blocks of their own: the output projection writes the second norm's rows and the down
+    projection the next block's first norm; only a norm nobody did for the block runs on its
+    own.  Against the plain formulas, and the same bits as with every norm on its own."""
     dtype = "bfloat16"
-    hidden, nh, nkv, hd, ffn, eps, T = 256, 8, 2, 64, 512, 1e-3, 40
+    hidden, nh, nkv, hd, ffn, eps, T = 256, 8, 2, 64, 512, 1e-3, 80
     mixer = build_part("mixer", PartSpec("gqa_attention", {
         "hidden_size": hidden, "num_heads": nh, "num_kv_heads": nkv, "head_dim": hd, "qkv_bias": True,
         "position": PartSpec("rope", {"head_dim": hd, "theta": 100.0})}), "model.layers.0.")
@@ -215,12 +162,11 @@ def test_prenorm_block_whose_products_finish_the_norms_behind_them():
     h = PartHarness(dtype, mixer.cache_spec())
     load(block, w, h)
     ctx = h.ctx([0] * T)
-    assert mixer.finishes_following_norm(ctx) and block.finishes_following_norm(ctx)
-    assert not mixer.takes_unscaled_rows(ctx) and not mixer.folds_following_norm(ctx)
+    assert mixer.finishes_following_norm(ctx) and block.last_part().finishes_following_norm(ctx)
     x0 = rnd(T, hidden, seed=9, scale=3.0)
     x0[2] *= 30.0
     next_gain = (1.0 + 0.5 * rnd(hidden, seed=5)).cuda()
-    nxt = block.first_norm_fold(ctx, T, whole=True)
+    nxt = block.following_of(ctx, block.last_part(), block.first_norm(), T)
     nxt.gain, nxt.eps = next_gain, 1e-5
     calls = []
     real = h.rt.k.rmsnorm
@@ -236,14 +182,17 @@ def test_prenorm_block_whose_products_finish_the_norms_behind_them():
     r = r + P.attention_block(cfg, wd, 0, P.rms_norm(r, wd[p + "input_layernorm.weight"], eps), torch.arange(T))
     r = r + P.mlp_block(wd, 0, P.rms_norm(r, wd[p + "post_attention_layernorm.weight"], eps))
     assert (x.cpu().double() - r).abs().max() <= tol(dtype, r, 1e-5, 3e-2)
-    rows = nxt.rows()
+    rows = nxt.values
     want = P.rms_norm(r, next_gain.cpu().double(), 1e-5)
-    assert isinstance(rows, torch.Tensor) and (rows.cpu().double() - want).abs().max() <= tol(dtype, want, 0, 3e-2)
+    assert (rows.cpu().double() - want).abs().max() <= tol(dtype, want, 0, 3e-2)
     # the same block and rows with every norm on its own: the same bits
     x2 = x0.clone().cuda()
     block.forward(ctx, CacheBinding(0, 0, True), x2)
     assert torch.equal(x2, x)
     assert torch.equal(real(x2, next_gain, 1e-5, torch.empty(T, hidden, dtype=torch.bfloat16, device="cuda")), rows)
+    # a short step: no product offers it, the block runs its norms itself
+    small = PartHarness(dtype, mixer.cache_spec())
+    assert not mixer.finishes_following_norm(small.ctx([0] * 9))
 
 
 def test_tied_head_and_embedding_share_the_packed_matrix(tmp_path):
