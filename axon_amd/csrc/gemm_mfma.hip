@@ -511,28 +511,24 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
 }
 
 // ---------------------------------------------------------------------------- gemm_stream
-// Up to 64 rows of X: the product is bound by reading W once.  A wave owns one tile of 32 rows
-// of W (two packed row tiles, A0 and A1) and one of the S segments of K.  Per step of 16 k it
-// loads 1 KB of W (the A operand of a 32x32x16 MFMA: lane l holds row l % 32, the 8 consecutive
-// k from 8 (l / 32); two pieces of 512 consecutive bytes, one in each packed tile) and, per 32
-// rows of X, 1 KB of X (the B operand: lane l holds row l % 32 of X, the same 8 k), and
-// multiplies; a ring of DEPTH steps is in flight, refilled as soon as a step is multiplied, so
-// the memory pipe never drains.  The waves of a block are TILES tiles x SEGS segments; the
-// segments' sums meet in LDS and are added in segment order, the 16 registers of a lane shared
-// out between the tile's waves in units of 4 consecutive output columns.
-//
-// The accumulator of a 32 x 32 tile: lane l, register e holds W row 8 (e / 4) + 4 (l / 32) + e % 4
-// and X row l % 32.  Rows 0..15 come from packed tile A0, rows 16..31 from A1, so register e + 8
-// is the same row of A1 as register e of A0: the paired epilogues put partners there.
-// * plain: A0, A1 = tiles 2t, 2t + 1: 32 consecutive columns of the output.
-// * GLU: A0 = gate rows 16t .., A1 = the up rows of the same columns (W holds 2 N rows); the
-//   output is silu(gate) * up.
-// * ROPE (the attention's fused [q; k; v] matrix; W's rows are heads of head_dim): A0 = dims
-//   16j .. of a head, A1 = their rotation partners 16j + half ..; q heads go rotated to `out`,
-//   k heads rotated into the request's page of keys, v heads as they are into its page of
-//   values (kept position-contiguous, [dim][slot]).  The arithmetic is that of the rotary kernel
-//   after a plain product: the sums are rounded to bfloat16 first, and each product and sum of
-//   the rotation is rounded on its own.
+// Up to 64 rows of X: the product is bound by reading W once.  A block owns NT16 row tiles (of
+// 16) of W; its waves are the S segments of K, each streaming its share of the tiles from memory
+// straight into 16x16x32 MFMA operands (a packed block as it lies in memory, 1 KB an
+// instruction), keeping a ring of steps in flight so that the memory pipe never drains, and
+// multiplying with up to 64 rows of X (the B operand: lane l holds row l % 16, 8 consecutive k
+// from (l / 16) * 8).  C[n][m] tiles of 16 x 16: a lane ends with 4 consecutive n of one m, one
+// vector store.  The segments' sums meet in LDS and are added in segment order.  A 16x16x32 MFMA
+// gives the bits of two chained 32x32x16 MFMAs over the same 32 k (measured over wide ranges of
+// exponents; the tests compare the kernels bit for bit), so the chain is the tile kernel's.
+// * GLU (NT16 = 2): the block's two tiles are the gate rows n0 .. n0 + 15 and the up rows of the
+//   same columns (W holds 2 N rows), and the output is silu(gate) * up.
+// * ROPE (NT16 = 2; the attention's fused [q; k; v] matrix, W's rows are heads of head_dim): a
+//   block owns dims d0 .. d0 + 15 of one head and their rotation partners d0 + half .., so that a
+//   lane ends with both values of a pair.  q heads go rotated to `out`, k heads rotated into the
+//   request's page of keys, v heads as they are into its page of values (kept
+//   position-contiguous, [dim][slot]).  The arithmetic is that of the rotary kernel after a
+//   plain product: the sums are rounded to bfloat16 first, and each product and sum of the
+//   rotation is rounded on its own.
 struct RopeStore {
   const float* table;            // [M, half, 2]: sin, cos of each token's angles
   const int32_t* positions;      // [M]
@@ -600,72 +596,78 @@ static int launch_split_reduce_rope(const float* partial, int splits, int m, int
   return 0;
 }
 
-template <int MT32, int SEGS, int TILES, int DEPTH, int EPI>
-__global__ void __launch_bounds__(SEGS * TILES * 64)
+template <int NT16, int MT16, int SEGS, int DEPTH, int EPI>
+__global__ void __launch_bounds__(SEGS * 64)
 gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w,
                    const void* __restrict__ bias, int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N,
-                   int K, int mode, int n_tiles, RopeStore rope) {
+                   int K, int mode, RopeStore rope) {
   constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE;
-  constexpr int WAVES = SEGS * TILES;
-  // [wave][32 rows of X][4 groups of 4 registers][lane]: a lane's 4 consecutive registers are one 16-byte slot
-  __shared__ float4 sums[SEGS > 1 ? WAVES * MT32 * 4 * 64 : 1];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int tile = blockIdx.x * TILES + wave / SEGS, seg = wave % SEGS;
-  const bool live = tile < n_tiles;                  // the last block may have tiles to spare
-  const int t = live ? tile : n_tiles - 1;
-  const int l32 = lane & 31, half = lane >> 5;
+  static_assert(EPI == EPI_PLAIN || NT16 == 2, "the paired epilogues own two tiles of W rows");
+  __shared__ float partial[SEGS > 1 ? SEGS : 1][NT16 * MT16][64][4];
+  const int tid = threadIdx.x, lane = tid & 63, seg = tid >> 6;
+  const int n0 = blockIdx.x * (GLU ? 16 : NT16 * 16);
+  const int r16 = lane & 15, kq = (lane >> 4) * 8;
 
-  // the two packed row tiles of this tile of 32 rows
+  // the packed blocks of this block's row tiles: [row tile][k block of 32][lane][8]
   const int KB = K / 32;
-  int a0, a1;
-  if (GLU) {
-    a0 = t;
-    a1 = N / 16 + t;
-  } else if (ROPE) {
-    const int per_head = rope.head_dim / 32;
-    a0 = (t / per_head) * (rope.head_dim / 16) + t % per_head;
-    a1 = a0 + rope.head_dim / 32;
-  } else {
-    const int last = (N + 15) / 16 - 1;              // past the matrix: its last tile (columns dropped below)
-    a0 = min(2 * t, last);
-    a1 = min(2 * t + 1, last);
+  const bf16_t* wtile[NT16];
+#pragma unroll
+  for (int i = 0; i < NT16; ++i) {
+    int tile;
+    if (GLU) tile = i * (N / 16) + blockIdx.x;                 // gate rows, then the up rows of the same columns
+    else if (ROPE) {
+      const int half = rope.head_dim / 2, per_head = half / 16;
+      tile = ((blockIdx.x / per_head) * rope.head_dim + i * half) / 16 + blockIdx.x % per_head;
+    } else tile = min(n0 / 16 + i, (N + 15) / 16 - 1);         // past the matrix: its last tile (columns dropped below)
+    wtile[i] = w + (size_t)tile * KB * 512 + lane * 8;
   }
-  // step q (16 k from 16 q) of a packed row tile: the 512 bytes from 512 q; this lane's 16 of them
-  const bf16_t* wp = w + (size_t)((lane & 16) ? a1 : a0) * KB * 512 + (half * 16 + (lane & 15)) * 8;
-  const bf16_t* xp[MT32];
+  const bf16_t* xrow[MT16];
 #pragma unroll
-  for (int j = 0; j < MT32; ++j) xp[j] = x + (size_t)min(j * 32 + l32, M - 1) * x_stride + half * 8;
+  for (int j = 0; j < MT16; ++j) xrow[j] = x + (size_t)min(j * 16 + r16, M - 1) * x_stride + kq;
 
-  // this wave's segment: the K tiles (of 64) nk seg / SEGS .. nk (seg + 1) / SEGS - 1, in steps of 16
+  f32x4 acc[NT16][MT16];
+#pragma unroll
+  for (int i = 0; i < NT16; ++i)
+#pragma unroll
+    for (int j = 0; j < MT16; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  // This wave's segment: the K tiles (of 64) nk seg / SEGS .. nk (seg + 1) / SEGS - 1, one chain
+  // in ascending k.  A ring of DEPTH steps (of 64 k) is kept in flight: a step is multiplied as
+  // soon as ITS loads have landed (loads return in order), and its place in the ring is refilled
+  // at once, so the memory pipe never drains.
   const int nk = K / 64;
-  const int q0 = (int)((long)seg * nk / SEGS) * 4;
-  const int steps = live ? (int)((long)(seg + 1) * nk / SEGS) * 4 - q0 : 0;
-
-  f32x16 acc[MT32];
-#pragma unroll
-  for (int j = 0; j < MT32; ++j)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) acc[j][e] = 0.0f;
-
-  uint4 wf[DEPTH], xf[DEPTH][MT32];
+  const int first = (int)((long)seg * nk / SEGS);
+  const int mine = (int)((long)(seg + 1) * nk / SEGS) - first;
+  uint4 wf[DEPTH][NT16][2], xf[DEPTH][MT16][2];
   auto load = [&](int slot, int local) {
-    const int q = q0 + local;
-    wf[slot] = *reinterpret_cast<const uint4*>(wp + (size_t)q * 256);
+    const int k0 = (first + local) * 64;
 #pragma unroll
-    for (int j = 0; j < MT32; ++j) xf[slot][j] = *reinterpret_cast<const uint4*>(xp[j] + q * 16);
+    for (int i = 0; i < NT16; ++i) {
+      wf[slot][i][0] = *reinterpret_cast<const uint4*>(wtile[i] + k0 * 16);          // k block k0 / 32: 512 elements each
+      wf[slot][i][1] = *reinterpret_cast<const uint4*>(wtile[i] + k0 * 16 + 512);
+    }
+#pragma unroll
+    for (int j = 0; j < MT16; ++j) {
+      xf[slot][j][0] = *reinterpret_cast<const uint4*>(xrow[j] + k0);
+      xf[slot][j][1] = *reinterpret_cast<const uint4*>(xrow[j] + k0 + 32);
+    }
   };
+  // one 16x16x32 MFMA is two chained 32x32x16 ones over the same k, bit for bit (the tile kernel's)
   auto multiply = [&](int slot) {
 #pragma unroll
-    for (int j = 0; j < MT32; ++j)
-      acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(wf[slot]), as_frag(xf[slot][j]), acc[j], 0, 0, 0);
-  };
-  if (steps > 0) {
-    // The ring holds steps base .. base + DEPTH - 1: a step is multiplied as soon as ITS loads
-    // have landed (loads return in order), and its place is refilled at once.
+    for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) load(d, min(d, steps - 1));    // beyond the segment: a valid step again
-    int base = 0;
-    for (; base + 2 * DEPTH <= steps; base += DEPTH) {
+      for (int i = 0; i < NT16; ++i)
+#pragma unroll
+        for (int j = 0; j < MT16; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[slot][i][h]), as_frag(xf[slot][j][h]), acc[i][j],
+                                                              0, 0, 0);
+  };
+  if (mine > 0) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) load(d, min(d, mine - 1));   // beyond this wave's steps: a valid step again
+    int base = 0;  // the ring holds local steps base .. base + DEPTH - 1
+    for (; base + 2 * DEPTH <= mine; base += DEPTH) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
         multiply(d);
@@ -675,62 +677,49 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
     // the tail: what the ring holds, refilled only where a step is left, then those
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      if (base + d < steps) multiply(d);
-      if (base + DEPTH + d < steps) load(d, base + DEPTH + d);
+      if (base + d < mine) multiply(d);
+      if (base + DEPTH + d < mine) load(d, base + DEPTH + d);
     }
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d)
-      if (base + DEPTH + d < steps) multiply(d);
+      if (base + DEPTH + d < mine) multiply(d);
   }
 
   if (SEGS > 1) {
 #pragma unroll
-    for (int j = 0; j < MT32; ++j)
+    for (int i = 0; i < NT16; ++i)
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
-        sums[((wave * MT32 + j) * 4 + g) * 64 + lane] =
-            make_float4(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
+      for (int j = 0; j < MT16; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) partial[seg][i * MT16 + j][lane][e] = acc[i][j][e];
     __syncthreads();
   }
-  if (!live) return;
-
-  // Units of work: 4 registers (4 consecutive W rows 8 g + 4 half ..) of one 32-row part of X;
-  // the paired epilogues take group g (rows of A0) together with group g + 2 (the same rows of A1).
-  // The tile's waves share the units out; each adds the segments' sums in segment order.
-  constexpr int GROUPS = EPI == EPI_PLAIN ? 4 : 2;
-  const int first_wave = (wave / SEGS) * SEGS;
-  auto summed = [&](int j, int g) {
-    if (SEGS == 1) return make_float4(acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]);
-    float4 v = sums[(((first_wave + 0) * MT32 + j) * 4 + g) * 64 + lane];
+  // the segments' sums in segment order; lane: X row 16 j + r16, W rows 4 (lane / 16) .. + 3 of tile i
+  auto summed = [&](int t, int e) {
+    if (SEGS == 1) return acc[t / MT16][t % MT16][e];
+    float sum = partial[0][t][lane][e];
 #pragma unroll
-    for (int s = 1; s < SEGS; ++s) {
-      const float4 p = sums[(((first_wave + s) * MT32 + j) * 4 + g) * 64 + lane];
-      v.x += p.x; v.y += p.y; v.z += p.z; v.w += p.w;
-    }
-    return v;
+    for (int q = 1; q < SEGS; ++q) sum += partial[q][t][lane][e];
+    return sum;
   };
+
+  if (ROPE) {
+    const int hd = rope.head_dim, half = hd / 2, per_head = half / 16;
+    const int slot = blockIdx.x / per_head;                  // q heads, then k heads, then v heads
+    const int d = (blockIdx.x % per_head) * 16 + (lane >> 4) * 4;
 #pragma unroll
-  for (int u0 = 0; u0 < MT32 * GROUPS; u0 += SEGS) {
-    const int u = u0 + seg;
-    if (u >= MT32 * GROUPS) break;
-    // SEGS == 1: u is a compile-time constant, so the registers are indexed statically
-    const int j = u / GROUPS, g = u % GROUPS;
-    const int m = j * 32 + l32;
-    const int r = 8 * g + 4 * half;               // first of the 4 rows, within the 32 of the tile (or the 16 of A0)
-    if (m >= M) continue;
-    if (ROPE) {
-      const int hd = rope.head_dim, hh = hd / 2, per_head = hd / 32;
-      const int slot = tile / per_head;             // q heads, then k heads, then v heads
-      const int d = (tile % per_head) * 16 + r;
-      const float4 lo4 = summed(j, g), hi4 = summed(j, g + 2);
-      const float lo_s[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, hi_s[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
+    for (int j0 = 0; j0 < MT16; j0 += SEGS) {
+      const int j = j0 + seg;
+      if (j >= MT16) break;
+      const int m = j * 16 + r16;
+      if (m >= M) continue;
       float a[4], b[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float lo = lo_s[e], hi = hi_s[e];
+        float lo = summed(j, e), hi = summed(MT16 + j, e);
         if (bias) {
           lo += load_vec(bias, bias_is_f32, slot * hd + d + e);
-          hi += load_vec(bias, bias_is_f32, slot * hd + hh + d + e);
+          hi += load_vec(bias, bias_is_f32, slot * hd + half + d + e);
         }
         a[e] = bf16_to_float(float_to_bf16(lo));
         b[e] = bf16_to_float(float_to_bf16(hi));
@@ -748,14 +737,14 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             vdst[(size_t)(d + e) * rope.page_size] = float_to_bf16(a[e]);
-            vdst[(size_t)(hh + d + e) * rope.page_size] = float_to_bf16(b[e]);
+            vdst[(size_t)(half + d + e) * rope.page_size] = float_to_bf16(b[e]);
           }
           continue;
         }
         const int kvh = slot - rope.n_heads;
         dst = rope.k_cache + (((size_t)page * rope.n_kv_heads + kvh) * rope.page_size + in_page) * hd;
       }
-      const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * hh + d) * 2);
+      const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * half + d) * 2);
       const float4 t0 = tab[0], t1 = tab[1];
       const float sn[4] = {t0.x, t0.z, t1.x, t1.z}, cs[4] = {t0.y, t0.w, t1.y, t1.w};
       float lo[4], hi[4];
@@ -770,31 +759,50 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
       *reinterpret_cast<uint2*>(dst + d) = pk;
       pk.x = pack2_bf16(hi[0], hi[1]);
       pk.y = pack2_bf16(hi[2], hi[3]);
-      *reinterpret_cast<uint2*>(dst + hh + d) = pk;
-      continue;
+      *reinterpret_cast<uint2*>(dst + half + d) = pk;
     }
-    if (GLU) {
-      const int n = tile * 16 + r;                  // N is a multiple of 16: the unit's 4 columns exist
-      const float4 g4 = summed(j, g), u4 = summed(j, g + 2);
-      uint2 pk;
-      pk.x = pack2_bf16(swiglu1(g4.x, u4.x), swiglu1(g4.y, u4.y));
-      pk.y = pack2_bf16(swiglu1(g4.z, u4.z), swiglu1(g4.w, u4.w));
-      bf16_t* dst = reinterpret_cast<bf16_t*>(out) + (size_t)m * out_stride + n;
-      if (out_stride % 4 == 0 && ((uintptr_t)out & 7) == 0) *reinterpret_cast<uint2*>(dst) = pk;
-      else {
-        dst[0].bits = (uint16_t)pk.x; dst[1].bits = (uint16_t)(pk.x >> 16);
-        dst[2].bits = (uint16_t)pk.y; dst[3].bits = (uint16_t)(pk.y >> 16);
-      }
-      continue;
-    }
-    const int n = tile * 32 + r;
-    if (n >= N) continue;
-    const float4 v4 = summed(j, g);
-    float v[4] = {v4.x, v4.y, v4.z, v4.w};
-    if (bias) {
+    return;
+  }
+  if (GLU) {
+    // a wave takes both tiles of a column block: gate (tile j) and up (tile MT16 + j)
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (n + e < N) v[e] += load_vec(bias, bias_is_f32, n + e);
+    for (int j0 = 0; j0 < MT16; j0 += SEGS) {
+      const int j = j0 + seg;
+      if (j >= MT16) break;
+      const int m = j * 16 + r16;
+      const int n = n0 + (lane >> 4) * 4;
+      if (m >= M) continue;
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = swiglu1(summed(j, e), summed(MT16 + j, e));
+      bf16_t* dst = reinterpret_cast<bf16_t*>(out) + (size_t)m * out_stride + n;
+      if (n + 3 < N && out_stride % 4 == 0 && ((uintptr_t)out & 7) == 0) {
+        uint2 pk;
+        pk.x = pack2_bf16(v[0], v[1]);
+        pk.y = pack2_bf16(v[2], v[3]);
+        *reinterpret_cast<uint2*>(dst) = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) dst[e] = float_to_bf16(v[e]);
+      }
+    }
+    return;
+  }
+  // tiles are shared out between the waves
+#pragma unroll
+  for (int t0 = 0; t0 < NT16 * MT16; t0 += SEGS) {
+    const int t = t0 + seg;
+    if (t >= NT16 * MT16) break;
+    const int i = t / MT16, j = t % MT16;
+    const int m = j * 16 + r16;
+    const int n = n0 + i * 16 + (lane >> 4) * 4;
+    if (m >= M || n >= N) continue;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[e] = summed(t, e);
+      if (bias && n + e < N) v[e] += load_vec(bias, bias_is_f32, n + e);
     }
     const size_t at = (size_t)m * out_stride + n;
     const bool whole = n + 3 < N && out_stride % 4 == 0;
@@ -828,42 +836,52 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
   }
 }
 
-template <int MT32, int SEGS, int EPI>
+#ifndef AXON_STREAM_DEPTH
+#define AXON_STREAM_DEPTH 8
+#endif
+
+template <int NT16, int MT16, int SEGS, int EPI>
 static int launch_stream(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                         int out_stride, int m, int n, int k, int mode, hipStream_t stream, int n_tiles,
-                         const RopeStore& rope) {
-  // eight waves a block where the segments allow it; the ring as deep as the registers allow
-  constexpr int TILES = SEGS >= 8 ? 1 : SEGS == 4 ? 2 : 4;
-  constexpr int DEPTH = MT32 == 1 ? 16 : 10;
-  gemm_stream_kernel<MT32, SEGS, TILES, DEPTH, EPI><<<ceil_div(n_tiles, TILES), SEGS * TILES * 64, 0, stream>>>(
-      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, n_tiles, rope);
+                         int out_stride, int m, int n, int k, int mode, hipStream_t stream, const RopeStore& rope) {
+  // the ring as deep as the registers allow: (NT16 + MT16) 8 registers a step; eight waves a block
+  // leave each 256 registers, fewer waves 512
+  constexpr int BUDGET = SEGS == 8 ? 160 : 384, FIT = BUDGET / ((NT16 + MT16) * 8);
+  constexpr int DEPTH = FIT < AXON_STREAM_DEPTH ? FIT : AXON_STREAM_DEPTH;
+  gemm_stream_kernel<NT16, MT16, SEGS, DEPTH, EPI><<<ceil_div(n, EPI == EPI_GLU ? 16 : NT16 * 16), SEGS * 64, 0, stream>>>(
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, rope);
   AXK_LAUNCH_CHECK("gemm_stream");
   return 0;
 }
 
-template <int EPI>
-static int launch_stream_any(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
-                             int out_stride, int m, int n, int k, int mode, hipStream_t stream, int n_tiles, int segs,
-                             const RopeStore& rope) {
-#define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, n_tiles, rope
-  if (m <= 32) {
-    switch (segs) {
-      case 1: return launch_stream<1, 1, EPI>(ARGS);
-      case 2: return launch_stream<1, 2, EPI>(ARGS);
-      case 4: return launch_stream<1, 4, EPI>(ARGS);
-      case 8: return launch_stream<1, 8, EPI>(ARGS);
-    }
-  } else {
-    switch (segs) {
-      case 1: return launch_stream<2, 1, EPI>(ARGS);
-      case 2: return launch_stream<2, 2, EPI>(ARGS);
-      case 4: return launch_stream<2, 4, EPI>(ARGS);
-      case 8: return launch_stream<2, 8, EPI>(ARGS);
-    }
+template <int NT16, int EPI>
+static int launch_stream_rows(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                              int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs,
+                              const RopeStore& rope) {
+#define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, rope
+#define BY_SEGS(MT16)                                                   \
+  switch (segs) {                                                       \
+    case 1: return launch_stream<NT16, MT16, 1, EPI>(ARGS);             \
+    case 2: return launch_stream<NT16, MT16, 2, EPI>(ARGS);             \
+    case 4: return launch_stream<NT16, MT16, 4, EPI>(ARGS);             \
+    case 8: return launch_stream<NT16, MT16, 8, EPI>(ARGS);             \
   }
+  if (m <= 16) { BY_SEGS(1) } else { BY_SEGS(2) }
+#undef BY_SEGS
 #undef ARGS
   axk_set_error("gemm_stream: %d segments", segs);
   return -1;
+}
+
+// Two row tiles a block where the matrix is large (the paired epilogues always), one where that
+// gives the chip more blocks.
+template <int EPI>
+static int launch_stream_any(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                             int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs,
+                             const RopeStore& rope) {
+  if (EPI != EPI_PLAIN || n >= 32 * 512)
+    return launch_stream_rows<2, EPI>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, segs, rope);
+  return launch_stream_rows<EPI == EPI_PLAIN ? 1 : 2, EPI>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode,
+                                                           stream, segs, rope);
 }
 
 // Shapes the MFMA kernels take: K a multiple of 64 and 16-byte aligned rows.  Decided by (N, K)
@@ -901,31 +919,38 @@ int launch_pack_matrix(const bf16_t* src, bf16_t* dst, int rows, int k, hipStrea
 
 
 // ---------------------------------------------------------------------------- the order and the dispatch
-// The number of segments K is cut into for a matrix of `tiles32` tiles of 32 rows (as gemm_stream
-// counts them: ceil(N / 32); N / 16 for a [gate; up] matrix of 2 N rows) and K columns: a power
-// of two up to 8, so that a step of few rows still gives some 768 waves a chain of their own,
-// with at least 4 K tiles (256 k) a segment.  It is a property of the matrix: it fixes the order
-// of addition of every product with it.
+// The number of segments K is cut into for a matrix of `tiles32` tiles of 32 rows (ceil(N / 32);
+// N / 16 for a [gate; up] matrix of 2 N rows) and K columns: 1, 2 or 4, so that a step of few rows
+// still gives some 768 waves a chain of their own, with at least 4 K tiles (256 k) a segment.
+// It is a property of the matrix: it fixes the order of addition of every product with it.
+// Measured on the 7B and 14B widths: more segments help steps of 33 to 256 rows (more blocks)
+// and cost long prompts (more sums through the workspace); 4 is the balance.
 int gemm_segments(int tiles32, int k) {
   const int nk = k / 64;
   int s = 1;
-  while (s < 8 && tiles32 * s < 768 && nk / (2 * s) >= 4) s *= 2;
+  while (s < 4 && tiles32 * s < 768 && nk / (2 * s) >= 4) s *= 2;
   return s;
 }
 
 static int tiles32_of(int n, int mode) { return mode == MODE_SWIGLU ? n / 16 : (n + 31) / 32; }
 
-// M > 64 with S > 1 segments: kept apart in registers by blocks that walk all of K where the output
-// alone gives enough tiles of 128 x 128 (or 128 x 256) to occupy the chip, else a block a segment
-// and the sums through a workspace.  Decided by the sizes alone.
+// The most rows the streaming kernel takes: beyond, every block would read more of X than of W.
+#ifndef AXON_STREAM_MAX_M
+#define AXON_STREAM_MAX_M 32
+#endif
+
+// More rows than the streaming kernel takes, S > 1 segments: a block a segment (the blocks' sums
+// go through a workspace and are added in segment order by a second kernel; measured faster for
+// every product of the 7B and 14B layers up to 2,048 rows, and the only way to occupy the chip
+// when the output is small), unless the workspace would pass 256 MB: then blocks walk all of K
+// and keep the segments apart in registers.  Decided by the sizes alone.
 static bool segments_across_blocks(int m, int n, int k, int mode, int segs) {
   if (segs <= 1 || n % 4 != 0) return false;
-  const long blocks = (long)ceil_div(m, 128) * ceil_div(n, mode == MODE_SWIGLU ? 64 : 128);
-  return blocks < 100;
+  return (size_t)segs * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float) <= ((size_t)256 << 20);
 }
 
 size_t gemm_workspace_bytes(int m, int n, int k, int mode) {
-  if (k % 64 != 0 || m <= 64) return 0;
+  if (k % 64 != 0 || m <= AXON_STREAM_MAX_M) return 0;
   const int s = gemm_segments(tiles32_of(n, mode), k);
   if (!segments_across_blocks(m, n, k, mode, s)) return 0;
   return (size_t)s * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float);
@@ -935,7 +960,7 @@ size_t gemm_workspace_bytes(int m, int n, int k, int mode) {
 // adds the segments' sums can also norm the finished rows (gemm_split_reduce_norm_kernel: rows of
 // up to SRN_MAX_N columns).
 int gemm_then_norm_ok(int m, int n, int k) {
-  return gemm_pack_ok(n, k, 0) && m > 64 && n <= SRN_MAX_N &&
+  return gemm_pack_ok(n, k, 0) && m > AXON_STREAM_MAX_M && n <= SRN_MAX_N &&
          segments_across_blocks(m, n, k, MODE_ADD_F32, gemm_segments(tiles32_of(n, MODE_ADD_F32), k));
 }
 
@@ -952,16 +977,15 @@ static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, co
                   "(stride %d, M=%d)", x_stride, m);
     return -1;
   }
-  const int tiles32 = tiles32_of(n, mode);
-  const int segs = gemm_segments(tiles32, k);
+  const int segs = gemm_segments(tiles32_of(n, mode), k);
 #define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream
-  if (m <= 64) {
+  if (m <= AXON_STREAM_MAX_M) {
     if (norm || rope_after) {
       axk_set_error("gemm: M=%d goes to the streaming kernel, which has these epilogues of its own", m);
       return -1;
     }
-    if (mode == MODE_SWIGLU) return launch_stream_any<EPI_GLU>(ARGS, tiles32, segs, RopeStore());
-    return launch_stream_any<EPI_PLAIN>(ARGS, tiles32, segs, RopeStore());
+    if (mode == MODE_SWIGLU) return launch_stream_any<EPI_GLU>(ARGS, segs, RopeStore());
+    return launch_stream_any<EPI_PLAIN>(ARGS, segs, RopeStore());
   }
   const bool across = segments_across_blocks(m, n, k, mode, segs);
   if ((norm || rope_after) && (!across || mode != (norm ? MODE_ADD_F32 : MODE_STORE))) {
@@ -977,6 +1001,16 @@ static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, co
   }
   float* ws = (float*)workspace;
   const bool glu = mode == MODE_SWIGLU;
+  if (m <= 64) {
+    // one tile of 64 rows; the segments in registers only where the sums cannot go through the workspace
+    if (segs > 1 && !across) {
+      if (glu) return launch_tile<64, 256, 1, 4, true, true>(ARGS, segs);
+      return launch_tile<64, 128, 1, 4, false, true, 64, 3>(ARGS, segs);
+    }
+    if (glu) return launch_tile<64, 256, 1, 4, true>(ARGS, segs, ws);
+    if (n >= 8192) return launch_tile<64, 256, 1, 4, false>(ARGS, segs, ws, norm, rope_after);
+    return launch_tile<64, 128, 1, 4, false, false, 64, 3>(ARGS, segs, ws, norm, rope_after);
+  }
   if (segs > 1 && !across) {
     // the segments in registers: 128 x 256 tiles (8 waves) where they occupy the chip, else 128 x 128
     const long wide = (long)ceil_div(m, 128) * ceil_div(n, glu ? 128 : 256);
@@ -1030,7 +1064,7 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
 int gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotary_dim) {
   if (m < 1 || k % 64 != 0 || rotary_dim != head_dim || head_dim % 32 != 0 || n % head_dim != 0) return 0;
   if (!gemm_pack_ok(n, k, 0)) return 0;
-  if (m <= 64) return 1;
+  if (m <= AXON_STREAM_MAX_M) return 1;
   return segments_across_blocks(m, n, k, MODE_STORE, gemm_segments(tiles32_of(n, MODE_STORE), k));
 }
 
@@ -1041,12 +1075,11 @@ int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const v
                          size_t workspace_bytes, hipStream_t stream) {
   const RopeStore rope = {table, positions, seq_rows, block_table, table_stride, k_cache, v_cache,
                           n_heads, n_kv_heads, head_dim, page_size};
-  if (m > 64)
+  if (m > AXON_STREAM_MAX_M)
     return gemm_mfma_dispatch(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream, nullptr,
                               workspace, workspace_bytes, &rope);
-  const int tiles32 = n / 32;
   return launch_stream_any<EPI_ROPE>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream,
-                                     tiles32, gemm_segments(tiles32, k), rope);
+                                     gemm_segments(n / 32, k), rope);
 }
 
 #endif  // AXON_BF16
