@@ -64,6 +64,7 @@ def _through_every_class_of_rows(dtype, page, case):
     eng = llm.engine
     fed = {rid: 0 for rid in prompts}
     worst = 0.0
+    seen = {}
 
     def step(parts, end=()):
         """parts: (request, tokens to feed, wanted places among them)"""
@@ -77,6 +78,8 @@ def _through_every_class_of_rows(dtype, page, case):
         logits = eng.step(entries, end=end)
         if where:
             got = logits.cpu().double()
+            for row, (rid, pos) in zip(logits.cpu(), where):
+                seen[(rid, pos)] = row.clone()
             for row, (rid, pos) in zip(got, where):
                 ref = oracle[rid][pos]
                 err = float((row - ref).abs().max())
@@ -96,5 +99,11 @@ def _through_every_class_of_rows(dtype, page, case):
         step([("a", 1, [0])])                                      # over 600 positions: three chunks
     assert fed == {"a": 620, "b": 150, "c": 61}
     eng.release_all()
+    # every row again with its request alone and whole in one step: the same bits, in both precisions
+    for rid in prompts:
+        places = sorted(pos for r, pos in seen if r == rid)
+        alone = eng.step([StepEntry(rid + "!", prompts[rid], places)], end=[rid + "!"]).cpu()
+        for row, pos in zip(alone, places):
+            assert torch.equal(row, seen[(rid, pos)]), (rid, pos)
     eng.cache.check()
     assert eng.cache.free_pages() == n_pages

@@ -119,24 +119,62 @@ def test_stop_tokens_end_a_request_and_are_not_returned(model_dirs):
     assert llm.generate(p, max_new_tokens=0) == [[]]
 
 
-def test_under_page_pressure_requests_give_way_and_continue_with_the_same_tokens(model_dirs):
-    d = model_dirs("B")
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_under_page_pressure_requests_give_way_and_continue_with_the_same_tokens(dtype, model_dirs):
+    d = model_dirs("B", "float32" if dtype == "float32" else "bfloat16")
     cfg, w = P.load_plain(d)
     prompts = prompts_for("B", [20, 25, 18, 30, 22], seed=6)
-    roomy = axon_amd.load(d, dtype="float32", page_size=16, num_pages=64, max_seqs=4, max_batch_tokens=32)
+    roomy = axon_amd.load(d, dtype=dtype, page_size=16, num_pages=64, max_seqs=4, max_batch_tokens=32)
     want = roomy.generate(prompts, max_new_tokens=40)
     assert roomy.last_stats.preemptions == 0
     # 9 pages of 16: one request needs up to 70 tokens = 5 pages, so two cannot both finish
-    tight = axon_amd.load(d, dtype="float32", page_size=16, num_pages=9, max_seqs=4, max_batch_tokens=32)
+    tight = axon_amd.load(d, dtype=dtype, page_size=16, num_pages=9, max_seqs=4, max_batch_tokens=32)
     got = tight.generate(prompts, max_new_tokens=40)
     assert tight.last_stats.preemptions > 0
-    assert got == want == [P.greedy_generate(cfg, w, p, 40) for p in prompts]
+    # a request that gave way is fed again from its first token (prompt and generated tokens) and goes
+    # on with the same tokens: feeding again gives the cache the same bits, in both precisions
+    assert got == want
+    if dtype == "float32":
+        assert got == [P.greedy_generate(cfg, w, p, 40) for p in prompts]
     tight.engine.cache.check()
     assert tight.engine.cache.free_pages() == 9
-    # sampled requests keep their random stream across a preemption
+    # sampled requests keep their random stream across a preemption; a stop token ends one of them early
     s_want = roomy.generate(prompts, max_new_tokens=30, temperature=0.9, seed=3)
     s_got = tight.generate(prompts, max_new_tokens=30, temperature=0.9, seed=3)
     assert s_got == s_want
+    stop = s_want[1][7]
+    cut = tight.generate(prompts, max_new_tokens=30, temperature=0.9, seed=3, stop=[stop])
+    for full, part in zip(s_want, cut):
+        assert part == (full[:full.index(stop)] if stop in full else full)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["D", "E"])
+def test_a_requests_tokens_do_not_depend_on_the_batch(name, dtype, model_dirs):
+    """Eighteen requests of different lengths that finish one after the other, so that the
+    decoding batch shrinks 18, 17, 16, ... and prompt portions share steps with decoding tokens:
+    every request gets the tokens it gets when it runs alone, greedy and sampled with a seed,
+    in float32 and in bfloat16 (the matrix-core kernels: head sizes 64 and 128)."""
+    d = model_dirs(name, "float32" if dtype == "float32" else "bfloat16")
+    lengths = [3, 70, 9, 130, 17, 33, 64, 65, 2, 40, 100, 5, 21, 90, 12, 150, 7, 48]
+    prompts = prompts_for(name, lengths, seed=21)
+    page = TINY[name]["page_size"]
+    llm = axon_amd.load(d, dtype=dtype, page_size=page, num_pages=18 * (200 // page + 2), max_seqs=18, max_batch_tokens=96)
+    for kw in (dict(), dict(temperature=0.8, top_k=40, top_p=0.9, repeat_penalty=1.1, seed=100)):
+        news = [4 + 2 * i for i in range(len(prompts))]
+        full = llm.generate(prompts, max_new_tokens=max(news), **kw)
+        for i, (p, o) in enumerate(zip(prompts, full)):
+            solo_kw = dict(kw)
+            if "seed" in kw:
+                solo_kw["seed"] = kw["seed"] + i            # request i of a call draws from the stream seeded seed + i
+            alone = llm.generate([p], max_new_tokens=news[i], **solo_kw)[0]
+            assert alone == o[:news[i]], (name, dtype, i, kw)
+        # other company, another token budget and so other portions: the same tokens
+        llm.cfg.max_batch_tokens = 40
+        some = llm.generate(prompts[3:9], max_new_tokens=10, **({**kw, "seed": kw["seed"] + 3} if "seed" in kw else kw))
+        llm.cfg.max_batch_tokens = 96
+        assert some == [o[:10] for o in full[3:9]]
+    llm.engine.cache.check()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

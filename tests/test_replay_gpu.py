@@ -1,7 +1,9 @@
 """Trace replay through bin/trace_run, as a user drives it: the same requests whole, with the
-last 32 tokens decoded one by one, in portions of changing size down to two tokens, and mixed
-with other requests in a pool so small that pages are used again; float32 and bfloat16; all
-compared with the plain implementation."""
+last 32 tokens decoded one by one, in portions of changing size down to two tokens, mixed
+with other requests in a pool so small that pages are used again, and given up half way and fed
+again from their first token; float32 and bfloat16; all compared with the plain implementation,
+and with each other bit for bit (src/lm.rs:272-278: a row's result is what it is alone, whatever
+else is in the step)."""
 import numpy as np
 import pytest
 import torch
@@ -20,9 +22,15 @@ def oracle(model_dir, prompts):
     return [P.forward_logits(cfg, w, p).float().numpy() for p in prompts]
 
 
+def first_life(rid):
+    """The request a row belongs to: a request fed again after it was given up carries a mark."""
+    return rid.rstrip("~")
+
+
 def check(rows, refs, ids, dtype):
     worst = 0.0
     for (rid, pos), got in rows.items():
+        rid = first_life(rid)
         ref = refs[ids.index(rid)][pos]
         tol = tolerance(dtype, torch.from_numpy(refs[ids.index(rid)]))
         err = float(np.abs(got - ref).max())
@@ -88,6 +96,38 @@ def mixed(prompts, seed=0, live_at_most=4):
     return tb
 
 
+def given_up_and_fed_again(prompts, seed=0, live_at_most=3):
+    """What a scheduler does when pages run out (src/serve/engine.rs:2244-2276): a request that
+    has been fed part of its prompt and has decoded a few tokens is ended, its pages go to the
+    others, and later it is fed again from its first token (here under its name with a mark), in
+    other portions, up to its end.  Both lives' rows must be those of the whole request."""
+    rng = np.random.default_rng(seed)
+    tb = TraceBuilder()
+    waiting = [(i, f"r{i}") for i in range(len(prompts))]
+    live = {}
+    while waiting or live:
+        while waiting and len(live) < live_at_most:
+            i, rid = waiting.pop(0)
+            live[rid] = (i, 0)
+        entries, end = [], []
+        for rid in list(live):
+            i, at = live[rid]
+            p = prompts[i]
+            n = int(min(rng.choice([1, 1, 2, 5, 16, 40]), len(p) - at))
+            entries.append((rid, p[at:at + n], list(range(n))))
+            at += n
+            live[rid] = (i, at)
+            if at == len(p):
+                end.append(rid)
+                del live[rid]
+            elif not rid.endswith("~") and at >= len(p) // 2:
+                end.append(rid)                                  # given up half way ...
+                del live[rid]
+                waiting.append((i, rid + "~"))                   # ... and back in the queue, from token 0
+        tb.step(entries, end)
+    return tb
+
+
 def max_tokens_for(tb, prompts_by_id):
     """The most tokens live requests hold at any time, each rounded up to 64."""
     live, most = {}, 0
@@ -110,7 +150,8 @@ def test_every_schedule_matches_the_plain_implementation(name, dtype, model_dirs
     page = ["--page-size", str(TINY[name]["page_size"])]
     results = {}
     for label, tb in (("whole", whole(prompts)), ("last32", last_32_one_by_one(prompts)),
-                      ("portions", changing_portions(prompts)), ("mixed", mixed(prompts, seed=len(name)))):
+                      ("portions", changing_portions(prompts)), ("mixed", mixed(prompts, seed=len(name))),
+                      ("refed", given_up_and_fed_again(prompts, seed=len(name)))):
         budget = max_tokens_for(tb, None)
         out = run_trace(model_dir, dtype, tb.steps, str(tmp_path / label), budget, extra=page)
         rows = tb.collect(out)
@@ -118,11 +159,11 @@ def test_every_schedule_matches_the_plain_implementation(name, dtype, model_dirs
         results[label] = rows
     # every position was asked for in the whole and portions schedules
     assert len(results["whole"]) == sum(len(p) for p in prompts) == len(results["portions"])
-    if dtype == "float32":
-        # beyond the tolerance: however the tokens were cut, the float32 logits are the same bits
-        for label in ("last32", "portions", "mixed"):
-            for key, row in results[label].items():
-                assert np.array_equal(row, results["whole"][key]), (label, key)
+    # beyond the tolerance: however the tokens were cut and whatever shared their steps, the logits
+    # are the same bits, in float32 and in bfloat16
+    for label in ("last32", "portions", "mixed", "refed"):
+        for (rid, pos), row in results[label].items():
+            assert np.array_equal(row, results["whole"][(first_life(rid), pos)]), (label, rid, pos)
 
 
 def test_a_step_that_wants_nothing_writes_nothing_and_requests_can_pause(model_dirs, tmp_path):
