@@ -55,6 +55,7 @@ def host_lib():
             "axh_cache_open": (c_int, [c_void_p]),
             "axh_cache_close": (c_int, [c_void_p, c_int]),
             "axh_cache_reserve": (c_int, [c_void_p, c_int, c_long]),
+            "axh_cache_reserve_many": (c_int, [c_void_p, c_int, IP, LP]),
             "axh_cache_trim": (c_int, [c_void_p, c_int, c_long]),
             "axh_cache_row": (c_int, [c_void_p, c_int, c_int, c_void_p, c_int]),
             "axh_cache_free_pages": (c_int, [c_void_p, c_int]),
@@ -193,6 +194,28 @@ class CacheManager:
             raise CacheError(self._error())
         else:
             raise OutOfPages(-rc, f"the cache is full: {-rc} pages short for {n_tokens} positions of slot {slot}")
+
+    def reserve_many(self, needs: Sequence[Tuple[int, int]]) -> None:
+        """Pages for every (slot, positions) of a step, in every group: for all of them or, with
+        OutOfPages, for none (what a step reserves is what all of its entries need)."""
+        if not needs:
+            return
+        for slot, n_tokens in needs:
+            if n_tokens > self.max_seq_len:
+                raise CacheError(f"{n_tokens} positions exceed the {self.max_seq_len} a request may reach")
+        n_groups = len(self.groups)
+        held = [[self.lib.axh_cache_pages_of(self._h, g, slot) for g in range(n_groups)] for slot, _ in needs]
+        slots = (c_int * len(needs))(*[s for s, _ in needs])
+        tokens = (c_long * len(needs))(*[n for _, n in needs])
+        rc = self.lib.axh_cache_reserve_many(self._h, len(needs), slots, tokens)
+        if rc == 0:
+            for (slot, _), before in zip(needs, held):
+                if any(self.lib.axh_cache_pages_of(self._h, g, slot) != before[g] for g in range(n_groups)):
+                    self._dirty.add(slot)
+        elif rc <= -1000000:
+            raise CacheError(self._error())
+        else:
+            raise OutOfPages(-rc, f"the cache is full: {-rc} pages short for the {len(needs)} requests of the step")
 
     def trim(self, slot: int, n_cached: int) -> int:
         freed = self.lib.axh_cache_trim(self._h, slot, n_cached)

@@ -71,6 +71,9 @@ def read_config_json(model_dir: str) -> Dict[str, Any]:
         raise ConfigError(f"{path} is not JSON: {e}") from None
     if not isinstance(cfg, dict):
         raise ConfigError("config.json is not a JSON object")
+    if os.path.isfile(os.path.join(model_dir, "hf_quant_config.json")):
+        # src/safetensors.rs:1444-1449: a quantized export names itself in a file of its own
+        raise ConfigError("quantized checkpoint (hf_quant_config.json): quantized weights are not supported")
     return cfg
 
 

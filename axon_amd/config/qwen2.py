@@ -8,11 +8,16 @@ head_dim to hidden_size / heads (src/model.rs:1782-1783), tie_word_embeddings to
 """
 from __future__ import annotations
 
+import struct
 from dataclasses import dataclass
 from typing import Any, Dict, Optional
 
 from .base import (ConfigError, LayerSpec, ModelConfig, ModelSpec, PartSpec, Run, get_flag, get_number,
                    get_whole)
+
+
+def _as_float32(x: float) -> float:
+    return struct.unpack("<f", struct.pack("<f", x))[0]
 
 
 @dataclass(frozen=True)
@@ -83,7 +88,8 @@ class Qwen2Config(ModelConfig):
             head_dim=hd,
             vocab_size=get_whole(cfg, "vocab_size", None),
             max_position_embeddings=get_whole(cfg, "max_position_embeddings"),
-            rope_theta=get_number(theta_src, "rope_theta", 10000.0),
+            # kept as the 32-bit float nearest to the file's value, then widened (src/safetensors.rs:649-651)
+            rope_theta=_as_float32(get_number(theta_src, "rope_theta", 10000.0)),
             rms_norm_eps=get_number(cfg, "rms_norm_eps", 1e-6),
             tie_word_embeddings=get_flag(cfg, "tie_word_embeddings", False),
             head_dim_given=given,

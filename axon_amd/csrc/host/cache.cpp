@@ -165,6 +165,51 @@ int axh_cache_reserve(void* h, int slot, long n_tokens) {
   return 0;
 }
 
+// Pages for several requests at once (slot i up to n_tokens[i] positions), for all of them in
+// every group or for none: a step's entries are reserved together, so that a step that does not
+// fit leaves the cache as it found it.  Returns 0, or -(pages short), or -1000000 for a bad call.
+int axh_cache_reserve_many(void* h, int n, const int* slots, const long* n_tokens) {
+  Cache& c = *(Cache*)h;
+  for (int i = 0; i < n; ++i) {
+    const int slot = slots[i];
+    if (slot < 0 || slot >= c.max_seqs || !c.open[slot] || n_tokens[i] < 0) {
+      c.error = "reserve: slot " + std::to_string(slot) + " is not open";
+      return -1000000;
+    }
+    for (int j = 0; j < i; ++j)
+      if (slots[j] == slot) {
+        c.error = "reserve: slot " + std::to_string(slot) + " is named twice";
+        return -1000000;
+      }
+  }
+  int short_by = 0;
+  for (Group& g : c.groups) {
+    long need = 0;
+    for (int i = 0; i < n; ++i) {
+      const int want = pages_covering(g.geo, n_tokens[i]);
+      if (want > c.max_pages_per_seq) {
+        c.error = "reserve: " + std::to_string(n_tokens[i]) + " tokens need " + std::to_string(want) +
+                  " pages, a request may hold " + std::to_string(c.max_pages_per_seq);
+        return -1000000;
+      }
+      need += std::max(0, want - (int)g.pages[slots[i]].size());
+    }
+    if (need > (long)g.free_list.size()) short_by += (int)(need - (long)g.free_list.size());
+  }
+  if (short_by > 0) {
+    c.error = "reserve: " + std::to_string(short_by) + " pages short";
+    return -short_by;
+  }
+  for (int i = 0; i < n; ++i) {
+    for (Group& g : c.groups) {
+      const int want = pages_covering(g.geo, n_tokens[i]);
+      while ((int)g.pages[slots[i]].size() < want) g.pages[slots[i]].push_back(take_page(c, g));
+    }
+    if (n_tokens[i] > c.length[slots[i]]) c.length[slots[i]] = n_tokens[i];
+  }
+  return 0;
+}
+
 // After a step: `n_cached` tokens are in the cache.  Windowed groups give back the pages the
 // window has passed.  Returns the pages freed.
 int axh_cache_trim(void* h, int slot, long n_cached) {

@@ -6,6 +6,10 @@
 // comes here.  Everything after the candidates is float64, as in the reference
 // (src/sample.rs:465-556).  Exactly one number is taken from the stream per decided token
 // (src/sample.rs:272-277), so a seed gives the same tokens however requests are batched.
+//
+// `kept`, `draw` and `pick_sorted` below follow src/sample.rs:465-556 operation by operation, on
+// purpose: the same tokens for the same seed need the same float64 operations in the same order,
+// so here the reference's algorithm is the specification, not one choice among several.
 #include <math.h>
 #include <stdint.h>
 #include <string.h>

@@ -193,12 +193,12 @@ class LLM:
     # ------------------------------------------------------------------ logits
     def logits(self, token_ids: Sequence[int], all_positions: bool = False) -> torch.Tensor:
         """float32 logits after `token_ids`: at the last position [vocab], or at every position
-        [len, vocab].  The cache is left as it was."""
+        [len, vocab], as a tensor of the caller's own.  The cache is left as it was."""
         ids = list(token_ids)
         rid = ("logits", self._next_id)
         self._next_id += 1
         want = list(range(len(ids))) if all_positions else [len(ids) - 1]
-        out = self.engine.step([StepEntry(rid, ids, want)], end=[rid])
+        out = self.engine.step([StepEntry(rid, ids, want)], end=[rid]).clone()     # a one-token step returns a view
         return out if all_positions else out[0]
 
 

@@ -100,6 +100,10 @@ class Engine:
         self.rt = rt
         self.cfg = cfg
         self.max_seq_len = cfg.max_seq_len or model.max_positions
+        for b in model.blocks:
+            limit = b.mixer.max_context()
+            if limit is not None and self.max_seq_len > limit:
+                raise StepError(f"max_seq_len {self.max_seq_len}: a mixer of this model takes contexts of up to {limit}")
         self.ws = Workspace(rt.device)
         plans = model.group_plans(cfg.page_size, self._pool_size)
         self.cache = CacheManager(plans, model.cache_plan.state_elems, cfg.max_seqs, self.max_seq_len, rt.device,
@@ -204,14 +208,14 @@ class Engine:
     def step(self, entries: Sequence[StepEntry], end: Iterable[Hashable] = ()) -> Optional[torch.Tensor]:
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         self._validate(entries)
+        # pages for every entry or for none: a step that does not fit leaves the cache as it was
         opened = []
         try:
             for e in entries:
                 if e.id not in self.live:
                     self.live[e.id] = LiveRequest(self.cache.open())
                     opened.append(e.id)
-                req = self.live[e.id]
-                self.cache.reserve(req.slot, req.n_cached + len(e.tokens))
+            self.cache.reserve_many([(self.live[e.id].slot, self.live[e.id].n_cached + len(e.tokens)) for e in entries])
         except Exception:
             for rid in opened:
                 self.release(rid)
@@ -267,8 +271,7 @@ class Engine:
         for rid, req in zip(ids, reqs):
             if req.n_cached + 1 > self.max_seq_len:
                 raise StepError(f"request {rid!r} would reach {req.n_cached + 1} positions, at most {self.max_seq_len}")
-        for req in reqs:
-            self.cache.reserve(req.slot, req.n_cached + 1)      # OutOfPages: nothing has run
+        self.cache.reserve_many([(req.slot, req.n_cached + 1) for req in reqs])      # OutOfPages: nothing taken, nothing run
         positions = [req.n_cached for req in reqs]
         rows = [req.slot for req in reqs]
         spans = [Span(req.slot, i, 1, req.n_cached) for i, req in enumerate(reqs)]

@@ -291,6 +291,11 @@ class Kernels:
         holds the window's first position, or 0) is cut into chunks of this size."""
         return int(self.lib.axk_attention_decode_chunk())
 
+    @property
+    def attention_decode_max_context(self) -> int:
+        """The longest context the decoding kernel's work list can name."""
+        return self.attention_decode_chunk * int(self.lib.axk_attention_decode_item_factor())
+
     def attention_decode_workspace(self, n_tokens: int, n_heads: int, head_dim: int, max_chunks: int) -> int:
         return int(self.lib.axk_attention_decode_workspace(n_tokens, n_heads, head_dim, max_chunks))
 

@@ -130,6 +130,7 @@ class GQAttention(Mixer):
         base = prefix + names.get("scope", "self_attn.")
         self.n = {k: base + names.get(k, k + "_proj") for k in ("q", "k", "v", "o")}
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+        self._max_context = None
         self.decode_chunk = 1 << 30          # until `load` has asked the kernels: one chunk
         self._work_list = lambda positions, window: list(range(len(positions)))
 
@@ -151,6 +152,9 @@ class GQAttention(Mixer):
     def cache_spec(self) -> Optional[CacheSpec]:
         return CacheSpec(entries=2, heads=self.nkv, head_dim=self.hd, window=self.window)
 
+    def max_context(self):
+        return self._max_context
+
     def decode_shape(self, positions):
         """The decoding kernel's workspace is laid out by the longest context of the step, in
         chunks of the kernel's size, rounded up to a power of two so that few shapes exist (the
@@ -171,6 +175,7 @@ class GQAttention(Mixer):
     def load(self, store, rt) -> None:
         self.decode_chunk = rt.k.attention_decode_chunk
         self._work_list = rt.k.attention_decode_work
+        self._max_context = rt.k.attention_decode_max_context
         self.w_qkv = rt.k.prepare_weight(store.fused_matrix([self.n[k] + ".weight" for k in ("q", "k", "v")]))
         biases = [store.vector(self.n[k] + ".bias", optional=True) for k in ("q", "k", "v")] if self.qkv_bias else []
         present = [b is not None for b in biases]

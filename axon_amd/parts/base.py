@@ -124,6 +124,11 @@ class Mixer(Part):
     def state_spec(self) -> Optional[StateSpec]:
         return None
 
+    def max_context(self) -> Optional[int]:
+        """The most positions of a request this mixer's kernels take (None: no limit of its own).
+        The engine refuses a longer `max_seq_len` when it is built, not in the middle of a step."""
+        return None
+
     def decode_shape(self, positions) -> Optional[Tuple[Any, Any]]:
         """For a step of single tokens at `positions`: (name, value) if the launches of this
         mixer depend on more than the number of tokens (say, on how long the contexts are), so

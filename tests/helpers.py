@@ -72,8 +72,8 @@ def engine_for(model_dir: str, dtype: str, page_size: int, num_pages: int, max_s
     from axon_amd.engine.loading import load_model
     rt = Runtime(dtype)
     model = load_model(model_dir, rt)
-    return Engine(model, rt, EngineConfig(dtype=dtype, page_size=page_size, num_pages=num_pages, max_seqs=max_seqs,
-                                          use_graphs=False, **kw))
+    kw.setdefault("use_graphs", False)
+    return Engine(model, rt, EngineConfig(dtype=dtype, page_size=page_size, num_pages=num_pages, max_seqs=max_seqs, **kw))
 
 
 # --------------------------------------------------------------------------- trace replay

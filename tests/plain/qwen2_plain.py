@@ -46,7 +46,8 @@ class PlainConfig:
             # head_dim is optional: hidden_size / heads without it (src/model.rs:1782-1783)
             head_dim=c.get("head_dim") or c["hidden_size"] // nh,
             # theta defaults to 10000 (src/model.rs:639), eps to 1e-6 (src/model.rs:1784)
-            rope_theta=float(c.get("rope_theta", 10000.0)),
+            # the loader keeps theta as a 32-bit float and widens it (src/safetensors.rs:649-651)
+            rope_theta=float(torch.tensor(float(c.get("rope_theta", 10000.0)), dtype=torch.float32)),
             rms_norm_eps=float(c.get("rms_norm_eps", 1e-6)),
             # tie_word_embeddings defaults to false (src/safetensors.rs:1608-1609)
             tie_word_embeddings=bool(c.get("tie_word_embeddings", False)),

@@ -128,3 +128,32 @@ def test_random_orders_keep_the_invariants(seed):
         m.close(s)
     assert m.free_pages() == m.plans[0].n_pages and m.free_slots() == 5
     m.check()
+
+
+def test_a_steps_reservation_is_for_all_of_its_requests_or_for_none():
+    """Two live requests and a new one, the pool one page short of what the three need together:
+    nothing is taken (the live requests keep exactly their pages), and with one page less to
+    ask for all three get theirs."""
+    spec = CacheSpec(entries=2, heads=2, head_dim=16)
+    cm = CacheManager([GroupPlan(spec, 2, 8, 10)], [], 4, 256)
+    a, b = cm.open(), cm.open()
+    cm.reserve(a, 20)      # 3 pages
+    cm.reserve(b, 9)       # 2 pages
+    c = cm.open()
+    free = cm.free_pages(0)
+    assert free == 5
+    before = [(cm.pages_of(0, s), cm.row(0, s)) for s in (a, b, c)]
+    with pytest.raises(OutOfPages) as info:
+        cm.reserve_many([(a, 33), (b, 17), (c, 17)])          # 2 + 1 + 3 = 6 pages, 5 free
+    assert info.value.short == 1
+    assert cm.free_pages(0) == free and [(cm.pages_of(0, s), cm.row(0, s)) for s in (a, b, c)] == before
+    cm.check()
+    cm.reserve_many([(a, 33), (b, 17), (c, 16)])              # 2 + 1 + 2
+    assert cm.free_pages(0) == 0 and [cm.pages_of(0, s) for s in (a, b, c)] == [5, 3, 2]
+    cm.check()
+    with pytest.raises(CacheError):
+        cm.reserve_many([(a, 34), (a, 35)])                    # a slot twice
+    for s in (a, b, c):
+        cm.close(s)
+    cm.check()
+    assert cm.free_pages(0) == 10

@@ -89,3 +89,22 @@ def test_engine_config():
         EngineConfig(dtype="float16")
     with pytest.raises(ConfigError):
         EngineConfig(page_size=0)
+
+
+def test_theta_is_kept_as_a_32_bit_float_and_a_quantized_export_is_refused(tmp_path):
+    import json
+    import struct
+    from axon_amd.config import ConfigError, config_from_dict, read_config_json
+    base = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=1, hidden_size=64, intermediate_size=64,
+                num_attention_heads=2, num_key_value_heads=1, vocab_size=32, max_position_embeddings=64)
+    # src/safetensors.rs:649-651: a base that 32 bits cannot hold is rounded to the nearest that they can
+    theta = 1000003.7
+    c = config_from_dict(dict(base, rope_theta=theta))
+    assert c.rope_theta == struct.unpack("<f", struct.pack("<f", theta))[0] != theta
+    assert config_from_dict(dict(base, rope_theta=1000000.0)).rope_theta == 1000000.0
+    # src/safetensors.rs:1444-1449
+    (tmp_path / "config.json").write_text(json.dumps(base))
+    assert read_config_json(str(tmp_path))["hidden_size"] == 64
+    (tmp_path / "hf_quant_config.json").write_text("{}")
+    with pytest.raises(ConfigError, match="hf_quant_config.json"):
+        read_config_json(str(tmp_path))

@@ -221,6 +221,47 @@ def test_the_first_tokens_of_a_sequence(dtype, model_dirs):
         assert torch.equal(one, got[-1])
 
 
+def test_a_step_that_does_not_fit_takes_nothing(model_dirs):
+    """Two live requests and a new one in a step whose pages do not all fit: the step is refused,
+    the live requests hold what they held, the new one was never opened, and the step's tokens
+    fed afterwards in two steps give the logits of an undisturbed engine."""
+    from axon_amd.cache import OutOfPages
+    from axon_amd.engine import StepEntry
+    from helpers import engine_for
+    d = model_dirs("A")
+    p = prompts_for("A", [25, 17, 17], seed=13)
+    eng = engine_for(d, "float32", page_size=8, num_pages=6)
+    eng.step([StepEntry("a", p[0][:20], []), StepEntry("b", p[1][:9], [])])            # 3 + 2 pages of 6
+    cache = eng.cache
+    held = lambda: (cache.free_pages(0), {r: (eng.live[r].n_cached, cache.pages_of(0, eng.live[r].slot),
+                                               cache.row(0, eng.live[r].slot)) for r in eng.live})
+    before = held()
+    with pytest.raises(OutOfPages):                                                      # 1 + 1 + 3 pages, 1 free
+        eng.step([StepEntry("a", p[0][20:], [4]), StepEntry("b", p[1][9:], [7]), StepEntry("c", p[2], [16])])
+    assert held() == before and "c" not in eng.live and cache.free_slots() == 2
+    cache.check()
+    la = eng.step([StepEntry("a", p[0][20:], [4])], end=["a"]).clone()
+    lb = eng.step([StepEntry("b", p[1][9:], [7])], end=["b"]).clone()
+    lc = eng.step([StepEntry("c", p[2], [16])], end=["c"]).clone()
+    fresh = engine_for(d, "float32", page_size=8, num_pages=16)
+    for rid, prompt, got in (("a", p[0], la), ("b", p[1], lb), ("c", p[2], lc)):
+        want = fresh.step([StepEntry(rid, prompt, [len(prompt) - 1])], end=[rid])
+        assert torch.equal(got, want)
+    assert cache.free_pages(0) == 6
+    with pytest.raises(Exception):                                                       # longer than any kernel's list of work
+        engine_for(d, "bfloat16", page_size=8, num_pages=6, max_seq_len=1 << 20)
+
+
+def test_logits_are_the_callers_own(model_dirs):
+    """A one-token step answers from a buffer the next one-token step writes again: `logits`
+    hands out a copy."""
+    llm = axon_amd.load(model_dirs("A"), dtype="float32", page_size=8, num_pages=8, max_seqs=2)
+    a = llm.logits([5])
+    kept = a.clone()
+    b = llm.logits([7])
+    assert torch.equal(a, kept) and not torch.equal(a, b)
+
+
 def test_command_line_gen_and_logits(model_dirs):
     d = model_dirs("A")
     cfg, w = P.load_plain(d)

@@ -251,6 +251,88 @@ def test_wrong_attention_variants_move_the_logits(monkeypatch):
         assert moved > 100 * tolerance("float32", good), (name, moved)
 
 
+# --------------------------------------------------------------------------- the arrangement of a layer
+
+def _uniform_attention_weights():
+    """The whole-model fixture with q and k projections and their biases zeroed: every score is 0,
+    so attention is the running mean of the values over positions 0..t, which library routines
+    give (cumsum), whatever the rotation does to the zero vectors."""
+    cfg, w, tokens = _setup()
+    w = dict(w)
+    for l in range(cfg.num_hidden_layers):
+        for n in ("q_proj.weight", "q_proj.bias", "k_proj.weight", "k_proj.bias"):
+            w[f"model.layers.{l}.self_attn.{n}"] = torch.zeros_like(w[f"model.layers.{l}.self_attn.{n}"])
+    return cfg, w, tokens
+
+
+def _by_library_routines(cfg, w, tokens, order="reference"):
+    """The whole model as straight-line calls of torch's own routines (F.embedding, F.rms_norm,
+    F.linear, F.silu, cumsum), valid when every attention score is 0.  `order` names the
+    arrangement: the reference's (src/model.rs:2967-3059: x += attention(norm1 x); x +=
+    feed_forward(norm2 x), norm2 reading the sum; final norm, then the head) or a wrong one."""
+    d = cfg.hidden_size
+    group = cfg.num_attention_heads // cfg.num_key_value_heads
+    T = len(tokens)
+    x = F.embedding(torch.tensor(tokens), w["model.embed_tokens.weight"])
+    steps = torch.arange(1, T + 1, dtype=torch.float64)[:, None]
+
+    def attention(h, p):
+        v = F.linear(h, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"])
+        mean = torch.cumsum(v, dim=0) / steps                                  # uniform weights over 0..t
+        heads = mean.view(T, cfg.num_key_value_heads, cfg.head_dim).repeat_interleave(group, dim=1)
+        return F.linear(heads.reshape(T, -1), w[p + "self_attn.o_proj.weight"])
+
+    def feed_forward(h, p):
+        return F.linear(F.silu(F.linear(h, w[p + "mlp.gate_proj.weight"])) * F.linear(h, w[p + "mlp.up_proj.weight"]),
+                        w[p + "mlp.down_proj.weight"])
+
+    for l in range(cfg.num_hidden_layers):
+        p = f"model.layers.{l}."
+        n1 = lambda t: F.rms_norm(t, (d,), w[p + "input_layernorm.weight"], cfg.rms_norm_eps)
+        n2 = lambda t: F.rms_norm(t, (d,), w[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps)
+        if order == "reference":
+            x = x + attention(n1(x), p)
+            x = x + feed_forward(n2(x), p)
+        elif order == "parallel":                      # both parts read the same stream
+            x = x + attention(n1(x), p) + feed_forward(n2(x), p)
+        elif order == "no residual after attention":
+            x = attention(n1(x), p)
+            x = x + feed_forward(n2(x), p)
+        elif order == "no residual after the feed-forward":
+            x = x + attention(n1(x), p)
+            x = feed_forward(n2(x), p)
+        elif order == "norms after the parts":        # post-norm
+            x = n1(x + attention(x, p))
+            x = n2(x + feed_forward(x, p))
+        elif order == "norms swapped":
+            x = x + attention(n2(x), p)
+            x = x + feed_forward(n1(x), p)
+    if order != "no final norm":
+        x = F.rms_norm(x, (d,), w["model.norm.weight"], cfg.rms_norm_eps)
+    return F.linear(x, w["lm_head.weight"])
+
+
+def test_the_arrangement_of_a_layer_reduces_to_library_routines():
+    """What no part's own test pins: the order of norm, attention, sum, norm, feed-forward, sum
+    and the final norm before the head.  With uniform attention the whole model is a few lines of
+    library calls; the plain implementation equals them in the reference's order and in no other."""
+    cfg, w, tokens = _uniform_attention_weights()
+    got = P.forward_logits(cfg, w, tokens)
+    want = _by_library_routines(cfg, w, tokens)
+    assert (got - want).abs().max() <= 1e-10 * want.abs().max()
+    for wrong in ("parallel", "no residual after attention", "no residual after the feed-forward",
+                  "norms after the parts", "norms swapped", "no final norm"):
+        off = (_by_library_routines(cfg, w, tokens, wrong) - got).abs().max().item()
+        assert off > 100 * tolerance("float32", got) and off > 2 * tolerance("bfloat16", got), (wrong, off)
+    # with both output projections zero the residual stream carries the embedding through, unscaled
+    for l in range(cfg.num_hidden_layers):
+        for n in ("self_attn.o_proj.weight", "mlp.down_proj.weight"):
+            w[f"model.layers.{l}.{n}"] = torch.zeros_like(w[f"model.layers.{l}.{n}"])
+    bare = F.linear(F.rms_norm(F.embedding(torch.tensor(tokens), w["model.embed_tokens.weight"]), (cfg.hidden_size,),
+                               w["model.norm.weight"], cfg.rms_norm_eps), w["lm_head.weight"])
+    assert (P.forward_logits(cfg, w, tokens) - bare).abs().max() <= 1e-12 * bare.abs().max()
+
+
 # --------------------------------------------------------------------------- picking
 
 def test_argmax_rules():
