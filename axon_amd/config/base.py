@@ -142,5 +142,19 @@ class ModelConfig:
     def to_dict(self) -> Dict[str, Any]:
         raise NotImplementedError
 
+    # ---- what a checkpoint of this architecture may look like (hooks; the defaults fit most)
+    def vocab_tensor(self) -> Optional[str]:
+        """If config.json may lack the vocabulary's size: the tensor whose first dimension is it
+        (the loader then calls `with_vocab`).  None: the configuration always knows it."""
+        return None
+
+    def with_vocab(self, vocab_size: int) -> "ModelConfig":
+        raise NotImplementedError
+
+    def ignores_tensor(self, name: str) -> bool:
+        """Tensors a checkpoint may hold that the model does not read (tables that are
+        recomputed, say): they are neither unexpected nor loaded."""
+        return False
+
     def model_spec(self) -> ModelSpec:
         raise NotImplementedError

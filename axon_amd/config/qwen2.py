@@ -116,11 +116,18 @@ class Qwen2Config(ModelConfig):
             d["head_dim"] = self.head_dim
         return d
 
+    embedding_tensor = "model.embed_tokens.weight"
+
+    def vocab_tensor(self):
+        # the reference takes the vocabulary from the embedding's rows, not from vocab_size (src/model.rs:1797-1798)
+        return self.embedding_tensor if self.vocab_size is None else None
+
     def with_vocab(self, vocab_size: int) -> "Qwen2Config":
         from dataclasses import replace
         return replace(self, vocab_size=vocab_size)
 
-    embedding_tensor = "model.embed_tokens.weight"
+    def ignores_tensor(self, name: str) -> bool:
+        return name.endswith("rotary_emb.inv_freq")          # src/safetensors.rs:1157-1159
 
     # ------------------------------------------------------------------ the model as data
     def model_spec(self) -> ModelSpec:

@@ -262,6 +262,23 @@ __device__ __forceinline__ void attention_values(unsigned st, const bf16x8 (&pf)
   }
 }
 
+// The same chains with the V^T fragments in registers (the decoding kernel loads them straight
+// from the pages): vf[dt][s2] is what attention_values reads from the stage for tile dt, k step s2.
+template <int HD, typename Consume>
+__device__ __forceinline__ void attention_values_of(const uint4 (&vf)[HD / 32][4], const bf16x8 (&pf)[4], Consume consume) {
+  constexpr int DT = HD / 32;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    f32x16 tile;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) tile[e] = 0.0f;
+#pragma unroll
+    for (int s2 = 0; s2 < 4; ++s2)
+      tile = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_of(vf[dt][s2]), pf[s2], tile, 0, 0, 0);
+    consume(dt, tile);
+  }
+}
+
 // The fold of a block into the running state: the factors of the old state and of the block.
 __device__ __forceinline__ void attention_fold(float& m, float& l, float m_b, float l_b, float& a, float& b) {
   const float mn = fmaxf(m, m_b);
@@ -434,9 +451,10 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
 
 // ============================================================================ decoding tokens
 // grid (work items x kv heads): a block of four waves per (token, kv head, chunk of 256
-// positions); a wave takes one block of 64 of them, on its own: it brings the block's K and V^T
-// into a stage of LDS of its own (every load issued at once, 32 KB in flight per wave), runs
-// attention_block with the query heads of the group as the columns (a group of up to 32 heads)
+// positions); a wave takes one block of 64 of them, on its own: it brings the block's K into a
+// stage of LDS of its own and its V^T straight into registers as MFMA operands (every load
+// issued at once, 32 KB in flight per wave), runs attention_scores and the chains of
+// attention_values with the query heads of the group as the columns (a group of up to 32 heads)
 // and leaves (o_b, m_b, l_b) of every head in `partial`.  The work list names the chunks that
 // exist, token by token (item = token slot * CMB_MAX_CHUNKS + chunk, -1: nothing), so that a
 // batch of short and long contexts launches no block without work.  How a token's range is cut
@@ -444,7 +462,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
 // partial [token slot][head][block][HD + 2]: o_b, then m_b and l_b; blocks counted from the
 // chunk that holds the window's first position (or 0).
 template <int HD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
                         const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
@@ -452,7 +470,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
                         float* __restrict__ partial, int max_chunks, int n_heads, int n_kv_heads, int page_size,
                         int window, float scale) {
   using S = AttStage<HD>;
-  constexpr int KS = HD / 16;
+  constexpr int KS = HD / 16, DT = HD / 32;
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int item = work[blockIdx.x / n_kv_heads];    // the kv heads of a chunk side by side: they share its pages
@@ -473,18 +491,32 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
   const size_t page_stride = (size_t)n_kv_heads * HD * page_size;
   const bf16_t* k_head = k_cache + (size_t)kvh * HD * page_size;
   const bf16_t* v_head = v_cache + (size_t)kvh * HD * page_size;
-  unsigned char* stage = smem + wave * S::BYTES;
+  unsigned char* stage = smem + wave * S::K_BYTES;   // keys only
 
-  // every page first, then every load: nothing waits behind a table entry
-  int k_page[S::K_INSTR], v_page[S::V_INSTR];
+  // every page first, then every load: nothing waits behind a table entry.  V^T: k step s2 takes
+  // the lane's positions p0 + 8 c .. + 7, c = 4 (s2 / 2) + 2 (s2 % 2) + half, of dim 32 dt + l32:
+  // 16 bytes of one page (a page holds a multiple of 8 positions); the two halves of a wave read
+  // neighbouring chunks, so an instruction reads whole rows of a page of 16 positions.
+  int k_page[S::K_INSTR], v_page[4], v_at[4], keep[4];
 #pragma unroll
   for (int n = 0; n < S::K_INSTR; ++n) k_page[n] = att_k_page<HD>(n, lane, p0, pos, table_row, page_size);
 #pragma unroll
-  for (int n = 0; n < S::V_INSTR; ++n) v_page[n] = att_v_page<HD>(n, lane, p0, pos, table_row, page_size);
+  for (int s2 = 0; s2 < 4; ++s2) {
+    const int pa = p0 + 8 * (4 * (s2 >> 1) + 2 * (s2 & 1) + half);
+    keep[s2] = max(0, min(pos - pa + 1, 8));          // positions past the token were never written
+    const int pa_c = min(pa, pos);
+    v_page[s2] = table_row[pa_c / page_size];
+    v_at[s2] = (pa_c % page_size) & ~7;
+  }
 #pragma unroll
   for (int n = 0; n < S::K_INSTR; ++n) att_issue_k<HD>(stage, n, lane, k_page[n], p0, pos, k_head, page_stride, page_size);
+  uint4 vf[DT][4];
 #pragma unroll
-  for (int n = 0; n < S::V_INSTR; ++n) att_issue_v<HD>(stage, n, lane, v_page[n], p0, pos, v_head, page_stride, page_size);
+  for (int s2 = 0; s2 < 4; ++s2) {
+    const bf16_t* va = v_head + (size_t)v_page[s2] * page_stride + v_at[s2];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vf[dt][s2] = *reinterpret_cast<const uint4*>(va + (size_t)(dt * 32 + l32) * page_size);
+  }
 
   // Q^T (B operand): column = head of the group (zero beyond it), 8 consecutive dims from 16 ks + 8 half
   bf16x8 qf[KS];
@@ -498,10 +530,20 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
     }
   }
   wait_vmcnt<0>();                    // the stage is this wave's alone: what it loaded is what it reads
-  if (p0 + ATT_BLOCK - 1 > pos) {
-    att_clear_unwritten<HD>(stage, p0, pos, lane, 64);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    wait_lgkmcnt<0>();
+  // weights of unwritten positions are zero, and zero times whatever a page holds must stay zero
+#pragma unroll
+  for (int s2 = 0; s2 < 4; ++s2) {
+    if (keep[s2] < 8) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        uint32_t* w = reinterpret_cast<uint32_t*>(&vf[dt][s2]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (keep[s2] <= 2 * i) w[i] = 0;
+          else if (keep[s2] == 2 * i + 1) w[i] &= 0xffffu;
+        }
+      }
+    }
   }
   const bool whole = p0 + ATT_BLOCK - 1 <= pos && p0 >= lo;
   float m_b, l_b;
@@ -512,7 +554,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
   float* dst = partial + (((size_t)slot * n_heads + kvh * group + min(l32, group - 1)) *
                               (max_chunks * (DC_CHUNK / ATT_BLOCK)) + block) * (HD + 2);
   const bool head_live = l32 < group;
-  attention_values<HD>(st, pf, lane, [&](int dt, const f32x16& tile) {
+  attention_values_of<HD>(vf, pf, [&](int dt, const f32x16& tile) {
     if (!head_live) return;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
@@ -663,7 +705,7 @@ extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_c
 #define LAUNCH(HD)                                                                                                   \
   {                                                                                                                  \
     static bool configured = false;                                                                                  \
-    constexpr int lds = 4 * (ATT_BLOCK * HD * 2 + HD * ATT_BLOCK * 2);          /* a stage a wave */                  \
+    constexpr int lds = 4 * ATT_BLOCK * HD * 2;                              /* a wave its block's keys */        \
     if (!configured) {                                                                                               \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_kernel<HD>),                \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);                           \

@@ -7,6 +7,9 @@ they are batched continuously by the scheduler.
 """
 from __future__ import annotations
 
+import json
+import os
+import sys
 import time
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Union
@@ -44,6 +47,40 @@ class _Request:
     sampler: Optional[Sampler]
     out: List[int] = field(default_factory=list)
     done: bool = False
+
+
+class StepTrace:
+    """AXON_STEP_TRACE=FILE: one JSON line per scheduler step appended to FILE, a measurement aid
+    that changes no output (the reference's AXON_SERVE_TRACE, src/serve/engine.rs:682-773,
+    2011-2034): `t_ms` since the trace opened, the step's wall `ms` (the device is waited for, so
+    running ahead is off while tracing), its prompt portions (`feeds`, `fed` tokens), its
+    decoding rows (`rows`, their mean `depth` in positions; null without any), then the requests
+    `waiting` and `running` and the `preempted` ones of this step."""
+
+    def __init__(self, path: str):
+        self.out = open(path, "a", buffering=1)
+        self.t0 = time.time()
+
+    @classmethod
+    def from_env(cls) -> Optional["StepTrace"]:
+        path = os.environ.get("AXON_STEP_TRACE", "")
+        if not path:
+            return None
+        try:
+            trace = cls(path)
+        except OSError as e:
+            print(f"axon: AXON_STEP_TRACE {path}: {e}", file=sys.stderr)
+            return None
+        print(f"axon: step trace to {path}", file=sys.stderr)
+        return trace
+
+    def line(self, started: float, ms: float, plan, waiting: int, running: int, preempted: int) -> None:
+        feeds = [p for p in plan if p.count > 1 or p.start == 0]
+        rows = [p for p in plan if p.count == 1 and p.start > 0]
+        depth = round(sum(p.start for p in rows) / len(rows), 1) if rows else None
+        self.out.write(json.dumps({"t_ms": round((started - self.t0) * 1e3, 3), "ms": round(ms, 3), "feeds": len(feeds),
+                                   "fed": sum(p.count for p in feeds), "rows": len(rows), "depth": depth,
+                                   "waiting": waiting, "running": running, "preempted": preempted}) + "\n")
 
 
 class LLM:
@@ -100,7 +137,8 @@ class LLM:
         # tokens from the picks of the step before on the device (Engine.step_from_picks), and the
         # picks are read a step late, while the next step runs.  Until they are read the requests'
         # lists hold None in their place.  What ends a request is then known without the token.
-        ahead_ok = not stop
+        trace = StepTrace.from_env()
+        ahead_ok = not stop and trace is None
         behind = None            # (picks on their way, the requests they belong to)
 
         def settle(behind):
@@ -171,6 +209,10 @@ class LLM:
                         self.engine.release(p.id)
                 if late is not None:
                     behind = (late, [p.id for p in plan])
+                if trace is not None:
+                    torch.cuda.synchronize()
+                    waiting, running, _ = sched.counts()
+                    trace.line(t_step, (time.time() - t_step) * 1e3, plan, waiting, running, len(preempted))
                 dt = time.time() - t_step
                 if all(p.count == 1 and p.start > 0 for p in plan):
                     stats.decode_seconds += dt

@@ -12,12 +12,12 @@ from .runtime import Runtime
 
 
 def read_model_config(model_dir: str, checkpoint: Optional[Checkpoint] = None) -> ModelConfig:
-    """config.json through the registry.  A configuration without vocab_size takes it from the
-    embedding tensor, as the reference does (src/model.rs:1797-1798)."""
+    """config.json through the registry.  A configuration that does not know its vocabulary yet
+    names the tensor that does (`ModelConfig.vocab_tensor`)."""
     config = config_from_dict(read_config_json(model_dir))
-    if getattr(config, "vocab_size", 0) is None:
+    name = config.vocab_tensor()
+    if name is not None:
         ck = checkpoint or Checkpoint(model_dir)
-        name = config.embedding_tensor
         if name not in ck:
             from ..weights import WeightError
             raise WeightError([name], [], [])
@@ -30,7 +30,7 @@ def load_model(model_dir: str, rt: Runtime) -> DecoderModel:
     config = read_model_config(model_dir, ck)
     model = build_model_description(config)
     source = CheckpointSource(ck)
-    check_tensors(model.tensors(), source)
+    check_tensors(model.tensors(), source, config.ignores_tensor)
     model.load(WeightStore(source, rt.device, rt.dtype), rt)
     _release_staging(rt)
     return model

@@ -258,6 +258,36 @@ class Engine:
             self.release(rid)
         return logits
 
+    def profile(self, entries: Sequence[StepEntry], end: Iterable[Hashable] = ()):
+        """One step launched kernel by kernel (no graph) with an event after every launch:
+        ([{name, ms, launches, bytes}] in first-launch order, total ms), as the reference's
+        profile of a step (src/cuda/qwen2.rs:3338-3397).  `bytes`: the weight matrices those
+        launches read.  The events between the kernels also keep them from overlapping, so this
+        is each kernel alone; the step itself is a real one (the cache moves on)."""
+        events = []
+
+        def mark(name, nbytes):
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            events.append((name, ev, nbytes))
+
+        graphs, self.graphs_ok = self.graphs_ok, False
+        self.rt.k.set_launch_hook(mark)
+        try:
+            mark("start", 0)
+            self.step(entries, end)
+        finally:
+            self.rt.k.set_launch_hook(None)
+            self.graphs_ok = graphs
+        torch.cuda.synchronize()
+        rows: Dict[str, dict] = {}
+        for (_, before, _), (name, after, nbytes) in zip(events, events[1:]):
+            row = rows.setdefault(name, dict(name=name, ms=0.0, launches=0, bytes=0))
+            row["ms"] += before.elapsed_time(after)
+            row["launches"] += 1
+            row["bytes"] += nbytes
+        return list(rows.values()), events[0][1].elapsed_time(events[-1][1])
+
     def step_from_picks(self, ids: Sequence[Hashable]) -> torch.Tensor:
         """One more decoding step for exactly the requests of the last decoding step, in its
         order: each takes as its token the greedy pick that step made for it.  The pick is taken

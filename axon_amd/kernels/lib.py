@@ -123,6 +123,33 @@ class Kernels:
         if rc != 0:
             raise KernelError(self.lib.axk_last_error().decode())
 
+    # what launches kernels: wrapped while a step is profiled
+    _LAUNCHING = ("embed", "rmsnorm", "rope_table", "rope_kv_write", "gemm_qkv_rope", "attention", "attention_prefill",
+                  "attention_decode", "gemm", "swiglu", "argmax", "topk", "fill_i32", "fill_f32")
+
+    def set_launch_hook(self, hook) -> None:
+        """`hook(name, matrix_bytes)` is told of every call that has launched kernels, with the
+        bytes of the weight matrix it read (0 if none), as the reference's launch sites tell
+        theirs (src/cuda/qwen2.rs:2294, 2361-2449); None: off."""
+        for name in self._LAUNCHING:
+            self.__dict__.pop(name, None)
+        if hook is None:
+            return
+        for name in self._LAUNCHING:
+            plain = getattr(type(self), name)
+
+            def told(*a, _plain=plain, _name=name, **kw):
+                out = _plain(self, *a, **kw)
+                label, nbytes = _name, 0
+                if _name in ("gemm", "gemm_qkv_rope"):
+                    w = a[1]
+                    data = w.data if isinstance(w, PackedMatrix) else w
+                    nbytes = data.numel() * data.element_size()
+                    label = f"{_name} {w.shape[0]}x{w.shape[1]}"
+                hook(label, nbytes)
+                return out
+            self.__dict__[name] = told
+
     def _elem(self, t: torch.Tensor, what: str) -> None:
         if t.dtype != self.dtype or not t.is_cuda:
             raise KernelError(f"{what}: expected a {self.dtype_name} device tensor, got {t.dtype} on {t.device}")

@@ -3,7 +3,8 @@
 `check_tensors` compares the declared tensors with a checkpoint and raises ONE error that
 lists every missing tensor, every unexpected one and every wrong shape or unusable dtype
 (the reference checks the same things up front: src/model.rs:1491-1541, 1581-1607;
-src/safetensors.rs:1553-1558; `*.rotary_emb.inv_freq` is skipped: src/safetensors.rs:1157-1159).
+src/safetensors.rs:1553-1558; what the architecture says it does not read is skipped, as
+`*.rotary_emb.inv_freq` is there: src/safetensors.rs:1157-1159).
 
 `WeightStore` hands tensors to the parts on the device.  Storage rule: a matrix is kept in the
 compute dtype (bfloat16 for serving; float32 for the 32-bit path, where a bfloat16 checkpoint
@@ -38,17 +39,14 @@ class WeightError(ValueError):
         super().__init__("\n".join(lines))
 
 
-def _skipped(name: str) -> bool:
-    return name.endswith("rotary_emb.inv_freq")
-
-
-def check_tensors(decls: Iterable[TensorDecl], source) -> None:
-    """`source` offers names(), shape(name), dtype(name)."""
+def check_tensors(decls: Iterable[TensorDecl], source, ignored=None) -> None:
+    """`source` offers names(), shape(name), dtype(name); `ignored(name)` says which of its
+    tensors the architecture knows and does not read (`ModelConfig.ignores_tensor`)."""
     decls = list(decls)
     declared: Dict[str, TensorDecl] = {}
     for d in decls:
         declared.setdefault(d.name, d)
-    have = [n for n in source.names() if not _skipped(n)]
+    have = [n for n in source.names() if not (ignored is not None and ignored(n))]
     have_set = set(have)
     missing = [d.name for d in declared.values() if not d.optional and d.name not in have_set]
     unexpected = sorted(n for n in have if n not in declared)

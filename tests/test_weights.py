@@ -85,9 +85,10 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(model_dirs, tmp_pat
     d = tmp_path / "bad"
     d.mkdir()
     write_safetensors(str(d / "model.safetensors"), tensors.items())
-    model = build_model_description(config_from_dict(TINY["A"]["config"]))
+    config = config_from_dict(TINY["A"]["config"])
+    model = build_model_description(config)
     with pytest.raises(WeightError) as e:
-        check_tensors(model.tensors(), CheckpointSource(Checkpoint(str(d))))
+        check_tensors(model.tensors(), CheckpointSource(Checkpoint(str(d))), config.ignores_tensor)
     err = e.value
     assert sorted(err.missing) == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
     assert err.unexpected == ["model.layers.0.self_attn.o_proj.bias"]
