@@ -98,6 +98,9 @@ class GroupPlan:
     n_pages: int
 
     def bytes_per_page(self, elem_size: int) -> int:
+        """`elem_size`: of the compute dtype, which a group that names no dtype of its own stores."""
+        if self.spec.dtype is not None:
+            elem_size = torch.empty((), dtype=getattr(torch, self.spec.dtype)).element_size()
         return self.n_layers * self.spec.entries * self.spec.heads * self.page_size * self.spec.head_dim * elem_size
 
 
@@ -115,7 +118,7 @@ class CacheGroup:
         if device is not None:
             s = plan.spec
             self.storage = torch.zeros((plan.n_layers, s.entries, plan.n_pages, s.heads, plan.page_size, s.head_dim),
-                                       dtype=dtype, device=device)
+                                       dtype=dtype if s.dtype is None else getattr(torch, s.dtype), device=device)
             self.block_table = torch.zeros((max_seqs, max_pages_per_seq), dtype=torch.int32, device=device)
 
     def layer(self, index: int) -> Tuple[torch.Tensor, ...]:
@@ -142,8 +145,10 @@ class CacheManager:
             raise CacheError(f"bad cache geometry: {[(g.n_pages, g.page_size, g.spec.window) for g in groups]}")
         self.plans = list(groups)
         self.groups = [CacheGroup(g, max_seqs, self.max_pages_per_seq, device, dtype) for g in groups]
-        self.states = [torch.zeros((max_seqs, max(e, 1)), dtype=torch.float32, device=device) if device is not None
-                       else None for e in state_elems]
+        # a state arena per run with state: `state_elems` holds sizes, or (size, dtype name) pairs
+        sized = [(e, "float32") if isinstance(e, int) else (int(e[0]), str(e[1])) for e in state_elems]
+        self.states = [torch.zeros((max_seqs, max(e, 1)), dtype=getattr(torch, dt), device=device) if device is not None
+                       else None for e, dt in sized]
         self._dirty: set = set()
 
     def __del__(self):

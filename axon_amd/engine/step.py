@@ -15,6 +15,7 @@ The reference runs prompt portions and decode rows as two passes of one schedule
 """
 from __future__ import annotations
 
+from collections import ChainMap
 from dataclasses import dataclass
 from typing import Dict, Hashable, Iterable, List, Optional, Sequence
 
@@ -111,10 +112,21 @@ class Engine:
         self.live: Dict[Hashable, LiveRequest] = {}
         self.has_window = any(p.spec.window > 0 for p in plans)
         self.steps = 0
-        # decoding steps replayed from HIP graphs: static inputs and outputs, one graph per shape
-        parts = [model.embedding, model.final_norm, model.head] + list(model.blocks) + [b.mixer for b in model.blocks] \
-            + [b.feed_forward for b in model.blocks]
-        self.graphs_ok = cfg.use_graphs and all(getattr(p, "graph_safe", False) for p in parts)
+        # Decoding steps replayed from HIP graphs: static inputs and outputs, graphs per shape.  The
+        # step is cut into segments: the runs whose parts are graph_safe are captured, together
+        # with as much of the embedding, the final norm, the head and the pick as is; a part that
+        # is not (it branches on host values or keeps state) runs launch by launch between two
+        # graphs, once a step.
+        n_runs = len(model.order)
+        safe = [model.run_is_graph_safe(i) for i in range(n_runs)]
+        self._ends_safe = all(getattr(p, "graph_safe", False) for p in (model.embedding, model.final_norm, model.head))
+        self._segments = []                 # (captured?, first run, end run)
+        for i, ok in enumerate(safe):
+            if self._segments and self._segments[-1][0] == ok:
+                self._segments[-1] = (ok, self._segments[-1][1], i + 1)
+            else:
+                self._segments.append((ok, i, i + 1))
+        self.graphs_ok = cfg.use_graphs and self._ends_safe and any(safe)
         self._graphs: Dict = {}
         self._graph_pool = None
         self._shape_mixers = []         # one mixer for each distinct thing a decoding step's shape depends on
@@ -160,7 +172,8 @@ class Engine:
         # from the memory that is free now: every group gets an equal share of the fraction
         free, _ = torch.cuda.mem_get_info(self.rt.device)
         n_groups = max(1, len(self.model.cache_plan.group_specs))
-        per_page = n_layers * spec.entries * spec.heads * page_size * spec.head_dim * self.rt.elem_size
+        elem = self.rt.elem_size if spec.dtype is None else torch.empty((), dtype=getattr(torch, spec.dtype)).element_size()
+        per_page = n_layers * spec.entries * spec.heads * page_size * spec.head_dim * elem
         pages = int(free * cfg.memory_fraction / n_groups) // max(per_page, 1)
         cap = cfg.max_seqs * -(-self.max_seq_len // page_size)
         return max(1, min(pages, cap))
@@ -320,18 +333,71 @@ class Engine:
         return self._pending
 
     # ------------------------------------------------------------------ decoding steps
-    def _decode_forward(self, T: int, spans: List[Span], shapes: Dict, inputs: Dict):
-        """A step of T single tokens whose tokens, positions and slots are in `self._meta`: the
-        launches that a graph captures.  Logits go to the static buffer, greedy picks beside them."""
+    def _decode_context(self, T: int, spans: List[Span], shapes: Dict, inputs: Dict) -> StepContext:
         ctx = StepContext(self.rt, self.cache, self.ws, self._meta, T, spans)
         ctx.decode_only = True
         ctx.decode_index = self._index[:T]
         ctx.decode_shapes = shapes
         ctx.decode_inputs = inputs
+        return ctx
+
+    def _decode_forward(self, T: int, spans: List[Span], shapes: Dict, inputs: Dict):
+        """A step of T single tokens whose tokens, positions and slots are in `self._meta`,
+        launch by launch.  Logits go to the static buffer, greedy picks beside them."""
+        ctx = self._decode_context(T, spans, shapes, inputs)
         x = self.model.forward(ctx)
         logits = self.model.logits(ctx, x, ctx.decode_index, out=self._logits[:T])
         self.rt.k.argmax(logits, self._picks[:T])
         return logits
+
+    def _segment(self, ctx: StepContext, x: torch.Tensor, index: int) -> None:
+        """Segment `index` of a decoding step on the residual stream x, in place: its runs, with
+        the embedding before the first run and the final norm, the head and the pick behind the
+        last (logits into the static buffer)."""
+        _, first, end = self._segments[index]
+        if first == 0:
+            self.model.embedding.forward(ctx, out=x)
+        self.model.forward_runs(ctx, x, first, end)
+        if end == len(self.model.order):
+            logits = self.model.logits(ctx, x, ctx.decode_index, out=self._logits[:ctx.n_tokens])
+            self.rt.k.argmax(logits, self._picks[:ctx.n_tokens])
+
+    def _decode_graphs(self, key, T: int, spans: List[Span], shapes: Dict, inputs: Dict) -> torch.Tensor:
+        """Replay (at the first step of a shape: set up and capture) the step's segments.  What
+        the parts share within a step (`ctx.shared`: tables, plans) is kept from the captured
+        segments, whose graphs refresh it at every replay; what a segment that runs launch by
+        launch adds is the step's own and is dropped after it."""
+        entry = self._graphs.get(key)
+        if entry is None:
+            entry = self._graphs[key] = dict(
+                x=torch.empty((T, self.model.hidden_size), dtype=torch.float32, device=self.rt.device), shared={},
+                graphs=[None] * len(self._segments))
+        x = entry["x"]
+
+        def context(shared):
+            ctx = self._decode_context(T, spans, shapes, inputs)
+            ctx.shared = shared
+            return ctx
+
+        of_step = ChainMap({}, entry["shared"])
+        for index, (captured, _, _) in enumerate(self._segments):
+            if not captured:
+                self._segment(context(of_step), x, index)
+                continue
+            if entry["graphs"][index] is None:
+                # Once without capture, on a copy of the stream: kernels set themselves up at their
+                # first launch, and a captured segment writes the same cache rows however often it
+                # runs.  Then the capture itself, which runs nothing; the replay below is the step.
+                self._segment(context(ChainMap({}, entry["shared"])), x.clone(), index)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                if self._graph_pool is None:
+                    self._graph_pool = torch.cuda.graph_pool_handle()
+                with torch.cuda.graph(graph, pool=self._graph_pool):
+                    self._segment(context(entry["shared"]), x, index)
+                entry["graphs"][index] = graph
+            entry["graphs"][index].replay()
+        return self._logits[:T]
 
     def _decode_step(self, tokens, positions, rows, spans) -> torch.Tensor:
         """Every entry brings one token and wants its logits.  Inputs are copied into static
@@ -374,21 +440,7 @@ class Engine:
         if not self.graphs_ok:
             logits = self._decode_forward(T, spans, shapes, inputs)
         else:
-            key = (T, tuple(sorted(shapes.items(), key=repr)))
-            entry = self._graphs.get(key)
-            if entry is None:
-                # once without capture: kernels set themselves up at their first launch, and a
-                # decoding step writes the same cache rows however often it runs
-                self._decode_forward(T, spans, shapes, inputs)
-                torch.cuda.synchronize()
-                graph = torch.cuda.CUDAGraph()
-                if self._graph_pool is None:
-                    self._graph_pool = torch.cuda.graph_pool_handle()
-                with torch.cuda.graph(graph, pool=self._graph_pool):
-                    logits = self._decode_forward(T, spans, shapes, inputs)
-                entry = self._graphs[key] = (graph, logits)
-            entry[0].replay()
-            logits = entry[1]
+            logits = self._decode_graphs((T, tuple(sorted(shapes.items(), key=repr))), T, spans, shapes, inputs)
         self.last_picks = self._picks[:T]
         # the picks start their way to the host behind the step
         self._pick_hosts[at][:T].copy_(self._picks[:T], non_blocking=True)

@@ -83,7 +83,7 @@ class DecoderModel:
                 b.group, b.index = where[run.cache]
             if ss is not None:
                 b.state_index = len(state_elems)
-                state_elems.append(ss.elems)
+                state_elems.append((ss.elems, ss.dtype))
             bindings.append(b)
         return CachePlan(specs, counts, bindings, state_elems)
 
@@ -110,11 +110,17 @@ class DecoderModel:
     def forward(self, ctx) -> torch.Tensor:
         """The residual stream after every run: float32 [T, hidden]."""
         x = self.embedding.forward(ctx)
+        self.forward_runs(ctx, x, 0, len(self.order))
+        return x
+
+    def forward_runs(self, ctx, x: torch.Tensor, first: int, end: int) -> None:
+        """Runs first .. end - 1 of the execution order on the residual stream x, in place."""
         normed = None        # the next block's first norm, where the block before it did its work
-        for i, (run, binding) in enumerate(zip(self.order, self.cache_plan.bindings)):
+        for i in range(first, end):
+            run, binding = self.order[i], self.cache_plan.bindings[i]
             block = self.blocks[run.layer]
             following = None
-            if i + 1 < len(self.order):
+            if i + 1 < end:
                 after = self.blocks[self.order[i + 1].layer]
                 following = block.following_of(ctx, block.last_part(), after.first_norm(), x.shape[0])
             if normed is None and following is None:
@@ -122,7 +128,11 @@ class DecoderModel:
             else:
                 block.forward(ctx, binding, x, normed, following)
             normed = None if following is None else following.values
-        return x
+
+    def run_is_graph_safe(self, i: int) -> bool:
+        """Whether run i's block and its parts are all fixed launch sequences (see Part.graph_safe)."""
+        block = self.blocks[self.order[i].layer]
+        return all(getattr(p, "graph_safe", False) for p in (block, block.mixer, block.feed_forward))
 
     def logits(self, ctx, x: torch.Tensor, rows: torch.Tensor, out=None) -> torch.Tensor:
         """Final norm and head at the rows asked for: float32 [len(rows), vocab]."""

@@ -40,21 +40,24 @@ class TensorDecl:
 class CacheSpec:
     """Paged per-token storage a mixer wants for one run: `entries` arrays (keys and values:
     2) of `heads` x `head_dim` elements per position.  `window` > 0: only the last `window`
-    positions are ever read, so earlier pages can be given back."""
+    positions are ever read, so earlier pages can be given back.  `dtype`: the element type of
+    the pages ("float32", "bfloat16", "int8", ...); None: the engine's compute dtype."""
     entries: int
     heads: int
     head_dim: int
     window: int = 0
+    dtype: Optional[str] = None
 
     def group_key(self):
-        return (self.entries, self.heads, self.head_dim, self.window)
+        return (self.entries, self.heads, self.head_dim, self.window, self.dtype)
 
 
 @dataclass(frozen=True)
 class StateSpec:
-    """Fixed-size per-request state a mixer wants for one run: `elems` 32-bit floats, zeroed
-    when a request starts."""
+    """Fixed-size per-request state a mixer wants for one run: `elems` elements of `dtype`
+    (32-bit floats unless it says otherwise), zeroed when a request starts."""
     elems: int
+    dtype: str = "float32"
 
 
 @dataclass

@@ -222,7 +222,7 @@ def test_the_toy_architecture_is_described_by_its_parts(toy_dir):
     # two cache groups with pages of their own: the windowed runs (two of them: layer 0 twice)
     # and the full one (layer 2 once; its second run stores nothing); one state arena
     assert [(s.window, n) for s, n in zip(plan.group_specs, plan.group_layers)] == [(11, 2), (0, 1)]
-    assert plan.state_elems == [24]
+    assert plan.state_elems == [(24, "float32")]                 # the state's size and its element type
     assert [(b.group, b.index, b.writes, b.state_index) for b in plan.bindings] == [
         (0, 0, True, -1), (-1, -1, True, 0), (1, 0, True, -1), (0, 1, True, -1), (1, 0, False, -1)]
     names = {d.name for d in model.tensors()}
@@ -280,6 +280,11 @@ def test_the_toy_model_steps_like_its_plain_twin(toy_dir, dtype):
     # and generation works through the same entry point
     out = llm.generate([seqs[0][:9], seqs[1][:5]], max_new_tokens=6)
     assert [len(o) for o in out] == [6, 6]
+    # decoding steps replay graphs for the runs whose parts allow it; the toy mixer's run, which
+    # keeps state and reads host values, is launched between two graphs, once a step
+    assert eng.graphs_ok and [(c, a, b) for c, a, b in eng._segments] == [(True, 0, 1), (False, 1, 2), (True, 2, 5)]
+    assert eng._graphs and all(g is not None for e in eng._graphs.values() for g, (c, _, _) in
+                               zip(e["graphs"], eng._segments) if c)
     # what the toy mixer asked to have on the device in the last step of single tokens
     decay = next(b.mixer for b in llm.model.blocks if isinstance(b.mixer, DecayMixer))
     assert decay.seen_on_device.tolist() == [13, 9, -1, -1]
