@@ -47,6 +47,7 @@ class _Request:
     sampler: Optional[Sampler]
     out: List[int] = field(default_factory=list)
     done: bool = False
+    stopped: bool = False        # it picked a stop token (learnt a step late when decoding runs ahead)
 
 
 class StepTrace:
@@ -133,41 +134,65 @@ class LLM:
         stop = set(int(s) for s in stop)
         cache = self.engine.cache
         n_groups = len(cache.groups)
-        # Greedy decoding without stop tokens runs one step ahead of the host: a step takes its
-        # tokens from the picks of the step before on the device (Engine.step_from_picks), and the
-        # picks are read a step late, while the next step runs.  Until they are read the requests'
-        # lists hold None in their place.  What ends a request is then known without the token.
+        # Greedy decoding runs one step ahead of the host: a step takes its tokens from the picks
+        # of the step before on the device (Engine.step_from_picks), and the picks are read a step
+        # late, while the next step runs.  Until they are read the requests' lists hold None in
+        # their place.  That a request has reached its length is known without the token; that it
+        # picked a stop token is learnt a step late: the token is taken back, the request ends,
+        # and the row that the step ahead ran for it is dropped unread.
         trace = StepTrace.from_env()
-        ahead_ok = not stop and trace is None
+        ahead_ok = trace is None
         behind = None            # (picks on their way, the requests they belong to)
 
-        def settle(behind):
+        def settle(behind) -> List[int]:
+            """Fill in the picks that were on their way; the requests that picked a stop token."""
             picks, ids = behind
+            stopped = []
             for rid, tok in zip(ids, picks.tolist()):
                 r = reqs[rid]
+                if r.stopped:                        # a row that ran ahead of its request's end
+                    continue
                 at = len(r.tokens) - 1
                 while r.tokens[at] is not None:      # the one place that is still open
                     at -= 1
+                if int(tok) in stop:
+                    del r.tokens[at:], r.out[at - r.prompt_len:]
+                    r.stopped = True
+                    stopped.append(rid)
+                    continue
                 r.tokens[at] = int(tok)
                 r.out[at - r.prompt_len] = int(tok)
+            return stopped
 
         try:
             while any(not r.done for r in reqs.values()):
                 plan, preempted = sched.plan([cache.free_pages(g) for g in range(n_groups)])
                 feed = (behind is not None and not preempted and [p.id for p in plan] == behind[1]
                         and all(p.count == 1 and p.wants_logits for p in plan))
+                stopped = []
                 if behind is not None and not feed:
-                    settle(behind)
+                    stopped = settle(behind)
                     behind = None
                 for rid in preempted:
                     self.engine.release(rid)
                     stats.preemptions += 1
+                if stopped:
+                    # learnt before the step was launched: those requests leave it
+                    for rid in stopped:
+                        if not reqs[rid].done:
+                            reqs[rid].done = True
+                            sched.remove(rid)
+                            self.engine.release(rid)
+                    plan = [p for p in plan if not reqs[p.id].stopped]
+                    stopped = []
+                    if not plan:
+                        continue
                 if not plan:
                     raise RuntimeError("the scheduler has requests but planned nothing: the cache pool is too small")
                 t_step = time.time()
                 if feed:
                     logits = self.engine.step_from_picks([p.id for p in plan])
-                    settle(behind)               # the step before: read while this one runs
+                    stopped = settle(behind)     # the step before: read while this one runs
                     behind = None
                 else:
                     entries = [StepEntry(p.id, reqs[p.id].tokens[p.start:p.start + p.count],
@@ -190,7 +215,10 @@ class LLM:
                 for p in plan:
                     r = reqs[p.id]
                     appended = finished = False
-                    if p.wants_logits:
+                    if r.stopped:                    # this step ran a row for it in vain
+                        at += 1
+                        finished = not r.done
+                    elif p.wants_logits:
                         tok = None if late is not None else int(picks[at])
                         at += 1
                         stats.decided += 1

@@ -207,12 +207,13 @@ def main() -> int:
         more["prefill_8192"] = prefill(min(8192, ctx_len), 2)
         if args.sizes == "14b":
             more["mixed_step"] = mixed()
-        # generation through the entry point on the paths that cannot run ahead of the host: a
-        # stop token set (an id that random weights hardly ever pick), and sampled tokens
+        # generation through the entry point: greedy, greedy with a stop token set (an id that
+        # random weights hardly ever pick; both run a step ahead of the host), and sampled
+        # tokens, which the host draws and so cannot run ahead
         ps = [prompt(prompt_len) for _ in range(args.batch)]
         n_new = min(steps, 64)
-        llm.generate(ps[:1], max_new_tokens=2)
-        for label, kw in (("stop_token", dict(stop=[V - 1])),
+        llm.generate(ps, max_new_tokens=3)                            # graphs of this batch are captured here
+        for label, kw in (("greedy", {}), ("stop_token", dict(stop=[V - 1])),
                           ("sampled", dict(temperature=0.8, top_k=40, seed=1))):
             llm.generate(ps, max_new_tokens=n_new, **kw)
             st = llm.last_stats

@@ -60,10 +60,11 @@ def test_sampled_generation_matches_the_plain_sampler(model_dirs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_decoding_one_step_ahead_of_the_host(dtype, model_dirs):
+def test_decoding_one_step_ahead_of_the_host(dtype, model_dirs, monkeypatch, tmp_path):
     """A step fed from the previous step's picks on the device gives the logits and tokens of a
-    step fed the same tokens from the host, bit for bit; and generation that runs ahead (greedy,
-    no stop tokens) returns what generation that reads every token first returns."""
+    step fed the same tokens from the host, bit for bit; and greedy generation, which runs
+    ahead, returns what generation that reads every token first returns, with stop tokens that
+    end requests at their first token, in the middle, at their last token and never."""
     from axon_amd.engine import StepEntry
     d = model_dirs("B", dtype)
     prompts = prompts_for("B", [7, 30, 19], seed=11)
@@ -99,9 +100,19 @@ def test_decoding_one_step_ahead_of_the_host(dtype, model_dirs):
     more = prompts_for("B", [5, 40, 12, 26, 9], seed=12)
     run_ahead = llm.generate(more, max_new_tokens=21)
     steps_ahead = llm.last_stats.steps
-    one_by_one = llm.generate(more, max_new_tokens=21, stop=[-1])      # a stop token: every token is read first
-    assert run_ahead == one_by_one and steps_ahead == llm.last_stats.steps
     assert all(len(o) == 21 and None not in o for o in run_ahead)
+    stops = [run_ahead[0][0], run_ahead[1][9], run_ahead[2][20], run_ahead[3][1]]
+    cut = [o[:min([o.index(s) for s in stops if s in o], default=len(o))] for o in run_ahead]
+    assert len(set(len(o) for o in cut)) >= 3 and any(len(o) == 0 for o in cut)
+    stopped_ahead = llm.generate(more, max_new_tokens=21, stop=stops)
+    assert stopped_ahead == cut
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_pages() == 32 and not llm.engine.live
+    monkeypatch.setenv("AXON_STEP_TRACE", str(tmp_path / "steps.jsonl"))   # tracing reads every token first
+    one_by_one = llm.generate(more, max_new_tokens=21)
+    assert run_ahead == one_by_one and steps_ahead == llm.last_stats.steps
+    assert llm.generate(more, max_new_tokens=21, stop=stops) == cut
+    assert len((tmp_path / "steps.jsonl").read_text().splitlines()) == steps_ahead + llm.last_stats.steps
     llm.engine.cache.check()
     assert llm.engine.cache.free_pages() == 32 and not llm.engine.live
 
