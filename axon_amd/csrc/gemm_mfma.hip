@@ -473,6 +473,23 @@ struct RopeStore;
 static int launch_split_reduce_rope(const float* partial, int splits, int m, int n, const void* bias, int bias_is_f32,
                                     void* out, int out_stride, const RopeStore& rope, hipStream_t stream);
 
+// The second launch of a product whose blocks left a segment's sums each: the sums in segment
+// order, then the epilogue (with the rotary store, or the norm of the new rows, where asked).
+static int add_split_sums(const float* partial, int splits, int m, int n, const void* bias, int bias_is_f32, void* out,
+                          int out_stride, int mode, const SplitNorm* norm, const RopeStore* rope, hipStream_t stream) {
+  if (rope != nullptr) return launch_split_reduce_rope(partial, splits, m, n, bias, bias_is_f32, out, out_stride, *rope, stream);
+  if (norm != nullptr) {
+    gemm_split_reduce_norm_kernel<<<m, SRN_THREADS, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, (float*)out,
+                                                                 out_stride, *norm);
+    AXK_LAUNCH_CHECK("gemm_split_reduce_norm");
+    return 0;
+  }
+  gemm_split_reduce_kernel<<<ceil_div(m * (n / 4), 256), 256, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, out,
+                                                                          out_stride, mode);
+  AXK_LAUNCH_CHECK("gemm_split_reduce");
+  return 0;
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, bool SEG = false, int BK = 64, int STAGES = 2>
 static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                        int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs = 1,
@@ -497,17 +514,7 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks, splits > 1 ? partial : nullptr,
       segs);
   AXK_LAUNCH_CHECK("gemm_tile");
-  if (splits > 1 && rope != nullptr) return launch_split_reduce_rope(partial, splits, m, n, bias, bias_is_f32, out, out_stride, *rope, stream);
-  if (splits > 1 && norm != nullptr) {
-    gemm_split_reduce_norm_kernel<<<m, SRN_THREADS, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, (float*)out, out_stride,
-                                                         *norm);
-    AXK_LAUNCH_CHECK("gemm_split_reduce_norm");
-  } else if (splits > 1) {
-    gemm_split_reduce_kernel<<<ceil_div(m * (n / 4), 256), 256, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, out,
-                                                                            out_stride, mode);
-    AXK_LAUNCH_CHECK("gemm_split_reduce");
-  }
-  return 0;
+  return splits > 1 ? add_split_sums(partial, splits, m, n, bias, bias_is_f32, out, out_stride, mode, norm, rope, stream) : 0;
 }
 
 // ---------------------------------------------------------------------------- gemm_stream
@@ -594,6 +601,151 @@ static int launch_split_reduce_rope(const float* partial, int splits, int m, int
                                                           rope);
   AXK_LAUNCH_CHECK("gemm_split_reduce_rope");
   return 0;
+}
+
+// What a wave does with finished sums (`summed(t, e)`: tile t = i * MT16 + j, element e; a lane
+// holds X row 16 j + lane % 16 and W rows 4 (lane / 16) .. + 3 of tile i): the epilogue of the
+// product.  `unit` names the tiles: for PLAIN the columns from unit * NT16 * 16, for GLU gate and
+// up rows of columns unit * 16 .., for ROPE the half-pair `unit` of the [q; k; v] heads.  SHARE
+// waves (`share` = which one) divide the tiles among themselves.
+template <int NT16, int MT16, int EPI, int SHARE, class Summed>
+__device__ inline void rows_epilogue(Summed summed, int share, int unit, int lane, const void* __restrict__ bias,
+                                     int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int mode,
+                                     const RopeStore& rope) {
+  constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE;
+  const int r16 = lane & 15;
+  const int n0 = unit * (GLU ? 16 : NT16 * 16);
+  if (ROPE) {
+    const int hd = rope.head_dim, half = hd / 2, per_head = half / 16;
+    const int slot = unit / per_head;                  // q heads, then k heads, then v heads
+    const int d = (unit % per_head) * 16 + (lane >> 4) * 4;
+#pragma unroll
+    for (int j0 = 0; j0 < MT16; j0 += SHARE) {
+      const int j = j0 + share;
+      if (j >= MT16) break;
+      const int m = j * 16 + r16;
+      if (m >= M) continue;
+      float a[4], b[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float lo = summed(j, e), hi = summed(MT16 + j, e);
+        if (bias) {
+          lo += load_vec(bias, bias_is_f32, slot * hd + d + e);
+          hi += load_vec(bias, bias_is_f32, slot * hd + half + d + e);
+        }
+        a[e] = bf16_to_float(float_to_bf16(lo));
+        b[e] = bf16_to_float(float_to_bf16(hi));
+      }
+      bf16_t* dst;
+      if (slot < rope.n_heads) {
+        dst = reinterpret_cast<bf16_t*>(out) + (size_t)m * out_stride + (size_t)slot * hd;
+      } else {
+        const int pos = rope.positions[m];
+        const int page = rope.block_table[(size_t)rope.seq_rows[m] * rope.table_stride + pos / rope.page_size];
+        const int in_page = pos % rope.page_size;
+        if (slot >= rope.n_heads + rope.n_kv_heads) {
+          const int kvh = slot - rope.n_heads - rope.n_kv_heads;
+          bf16_t* vdst = rope.v_cache + ((size_t)page * rope.n_kv_heads + kvh) * hd * rope.page_size + in_page;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            vdst[(size_t)(d + e) * rope.page_size] = float_to_bf16(a[e]);
+            vdst[(size_t)(half + d + e) * rope.page_size] = float_to_bf16(b[e]);
+          }
+          continue;
+        }
+        const int kvh = slot - rope.n_heads;
+        dst = rope.k_cache + (((size_t)page * rope.n_kv_heads + kvh) * rope.page_size + in_page) * hd;
+      }
+      const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * half + d) * 2);
+      const float4 t0 = tab[0], t1 = tab[1];
+      const float sn[4] = {t0.x, t0.z, t1.x, t1.z}, cs[4] = {t0.y, t0.w, t1.y, t1.w};
+      float lo[4], hi[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo[e] = __fsub_rn(__fmul_rn(a[e], cs[e]), __fmul_rn(b[e], sn[e]));
+        hi[e] = __fadd_rn(__fmul_rn(a[e], sn[e]), __fmul_rn(b[e], cs[e]));
+      }
+      uint2 pk;
+      pk.x = pack2_bf16(lo[0], lo[1]);
+      pk.y = pack2_bf16(lo[2], lo[3]);
+      *reinterpret_cast<uint2*>(dst + d) = pk;
+      pk.x = pack2_bf16(hi[0], hi[1]);
+      pk.y = pack2_bf16(hi[2], hi[3]);
+      *reinterpret_cast<uint2*>(dst + half + d) = pk;
+    }
+    return;
+  }
+  if (GLU) {
+    // a wave takes both tiles of a column block: gate (tile j) and up (tile MT16 + j)
+#pragma unroll
+    for (int j0 = 0; j0 < MT16; j0 += SHARE) {
+      const int j = j0 + share;
+      if (j >= MT16) break;
+      const int m = j * 16 + r16;
+      const int n = n0 + (lane >> 4) * 4;
+      if (m >= M) continue;
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = swiglu1(summed(j, e), summed(MT16 + j, e));
+      bf16_t* dst = reinterpret_cast<bf16_t*>(out) + (size_t)m * out_stride + n;
+      if (n + 3 < N && out_stride % 4 == 0 && ((uintptr_t)out & 7) == 0) {
+        uint2 pk;
+        pk.x = pack2_bf16(v[0], v[1]);
+        pk.y = pack2_bf16(v[2], v[3]);
+        *reinterpret_cast<uint2*>(dst) = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) dst[e] = float_to_bf16(v[e]);
+      }
+    }
+    return;
+  }
+  // tiles are shared out between the waves
+#pragma unroll
+  for (int t0 = 0; t0 < NT16 * MT16; t0 += SHARE) {
+    const int t = t0 + share;
+    if (t >= NT16 * MT16) break;
+    const int i = t / MT16, j = t % MT16;
+    const int m = j * 16 + r16;
+    const int n = n0 + i * 16 + (lane >> 4) * 4;
+    if (m >= M || n >= N) continue;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[e] = summed(t, e);
+      if (bias && n + e < N) v[e] += load_vec(bias, bias_is_f32, n + e);
+    }
+    const size_t at = (size_t)m * out_stride + n;
+    const bool whole = n + 3 < N && out_stride % 4 == 0;
+    if (mode == MODE_STORE) {
+      bf16_t* dst = reinterpret_cast<bf16_t*>(out) + at;
+      if (whole && ((uintptr_t)out & 7) == 0) {
+        uint2 pk;
+        pk.x = pack2_bf16(v[0], v[1]);
+        pk.y = pack2_bf16(v[2], v[3]);
+        *reinterpret_cast<uint2*>(dst) = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) dst[e] = float_to_bf16(v[e]);
+      }
+    } else {
+      float* dst = reinterpret_cast<float*>(out) + at;
+      if (whole && ((uintptr_t)out & 15) == 0) {
+        float4 o = make_float4(v[0], v[1], v[2], v[3]);
+        if (mode == MODE_ADD_F32) {
+          const float4 old = *reinterpret_cast<const float4*>(dst);
+          o.x = old.x + v[0]; o.y = old.y + v[1]; o.z = old.z + v[2]; o.w = old.w + v[3];
+        }
+        *reinterpret_cast<float4*>(dst) = o;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) dst[e] = mode == MODE_ADD_F32 ? dst[e] + v[e] : v[e];
+      }
+    }
+  }
 }
 
 template <int NT16, int MT16, int SEGS, int DEPTH, int EPI>
@@ -703,150 +855,191 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
     return sum;
   };
 
-  if (ROPE) {
-    const int hd = rope.head_dim, half = hd / 2, per_head = half / 16;
-    const int slot = blockIdx.x / per_head;                  // q heads, then k heads, then v heads
-    const int d = (blockIdx.x % per_head) * 16 + (lane >> 4) * 4;
-#pragma unroll
-    for (int j0 = 0; j0 < MT16; j0 += SEGS) {
-      const int j = j0 + seg;
-      if (j >= MT16) break;
-      const int m = j * 16 + r16;
-      if (m >= M) continue;
-      float a[4], b[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float lo = summed(j, e), hi = summed(MT16 + j, e);
-        if (bias) {
-          lo += load_vec(bias, bias_is_f32, slot * hd + d + e);
-          hi += load_vec(bias, bias_is_f32, slot * hd + half + d + e);
-        }
-        a[e] = bf16_to_float(float_to_bf16(lo));
-        b[e] = bf16_to_float(float_to_bf16(hi));
-      }
-      bf16_t* dst;
-      if (slot < rope.n_heads) {
-        dst = reinterpret_cast<bf16_t*>(out) + (size_t)m * out_stride + (size_t)slot * hd;
-      } else {
-        const int pos = rope.positions[m];
-        const int page = rope.block_table[(size_t)rope.seq_rows[m] * rope.table_stride + pos / rope.page_size];
-        const int in_page = pos % rope.page_size;
-        if (slot >= rope.n_heads + rope.n_kv_heads) {
-          const int kvh = slot - rope.n_heads - rope.n_kv_heads;
-          bf16_t* vdst = rope.v_cache + ((size_t)page * rope.n_kv_heads + kvh) * hd * rope.page_size + in_page;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            vdst[(size_t)(d + e) * rope.page_size] = float_to_bf16(a[e]);
-            vdst[(size_t)(half + d + e) * rope.page_size] = float_to_bf16(b[e]);
-          }
-          continue;
-        }
-        const int kvh = slot - rope.n_heads;
-        dst = rope.k_cache + (((size_t)page * rope.n_kv_heads + kvh) * rope.page_size + in_page) * hd;
-      }
-      const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * half + d) * 2);
-      const float4 t0 = tab[0], t1 = tab[1];
-      const float sn[4] = {t0.x, t0.z, t1.x, t1.z}, cs[4] = {t0.y, t0.w, t1.y, t1.w};
-      float lo[4], hi[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        lo[e] = __fsub_rn(__fmul_rn(a[e], cs[e]), __fmul_rn(b[e], sn[e]));
-        hi[e] = __fadd_rn(__fmul_rn(a[e], sn[e]), __fmul_rn(b[e], cs[e]));
-      }
-      uint2 pk;
-      pk.x = pack2_bf16(lo[0], lo[1]);
-      pk.y = pack2_bf16(lo[2], lo[3]);
-      *reinterpret_cast<uint2*>(dst + d) = pk;
-      pk.x = pack2_bf16(hi[0], hi[1]);
-      pk.y = pack2_bf16(hi[2], hi[3]);
-      *reinterpret_cast<uint2*>(dst + half + d) = pk;
-    }
-    return;
-  }
-  if (GLU) {
-    // a wave takes both tiles of a column block: gate (tile j) and up (tile MT16 + j)
-#pragma unroll
-    for (int j0 = 0; j0 < MT16; j0 += SEGS) {
-      const int j = j0 + seg;
-      if (j >= MT16) break;
-      const int m = j * 16 + r16;
-      const int n = n0 + (lane >> 4) * 4;
-      if (m >= M) continue;
-      float v[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = swiglu1(summed(j, e), summed(MT16 + j, e));
-      bf16_t* dst = reinterpret_cast<bf16_t*>(out) + (size_t)m * out_stride + n;
-      if (n + 3 < N && out_stride % 4 == 0 && ((uintptr_t)out & 7) == 0) {
-        uint2 pk;
-        pk.x = pack2_bf16(v[0], v[1]);
-        pk.y = pack2_bf16(v[2], v[3]);
-        *reinterpret_cast<uint2*>(dst) = pk;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (n + e < N) dst[e] = float_to_bf16(v[e]);
-      }
-    }
-    return;
-  }
-  // tiles are shared out between the waves
-#pragma unroll
-  for (int t0 = 0; t0 < NT16 * MT16; t0 += SEGS) {
-    const int t = t0 + seg;
-    if (t >= NT16 * MT16) break;
-    const int i = t / MT16, j = t % MT16;
-    const int m = j * 16 + r16;
-    const int n = n0 + i * 16 + (lane >> 4) * 4;
-    if (m >= M || n >= N) continue;
-    float v[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      v[e] = summed(t, e);
-      if (bias && n + e < N) v[e] += load_vec(bias, bias_is_f32, n + e);
-    }
-    const size_t at = (size_t)m * out_stride + n;
-    const bool whole = n + 3 < N && out_stride % 4 == 0;
-    if (mode == MODE_STORE) {
-      bf16_t* dst = reinterpret_cast<bf16_t*>(out) + at;
-      if (whole && ((uintptr_t)out & 7) == 0) {
-        uint2 pk;
-        pk.x = pack2_bf16(v[0], v[1]);
-        pk.y = pack2_bf16(v[2], v[3]);
-        *reinterpret_cast<uint2*>(dst) = pk;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (n + e < N) dst[e] = float_to_bf16(v[e]);
-      }
-    } else {
-      float* dst = reinterpret_cast<float*>(out) + at;
-      if (whole && ((uintptr_t)out & 15) == 0) {
-        float4 o = make_float4(v[0], v[1], v[2], v[3]);
-        if (mode == MODE_ADD_F32) {
-          const float4 old = *reinterpret_cast<const float4*>(dst);
-          o.x = old.x + v[0]; o.y = old.y + v[1]; o.z = old.z + v[2]; o.w = old.w + v[3];
-        }
-        *reinterpret_cast<float4*>(dst) = o;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (n + e < N) dst[e] = mode == MODE_ADD_F32 ? dst[e] + v[e] : v[e];
-      }
-    }
-  }
+  rows_epilogue<NT16, MT16, EPI, SEGS>(summed, seg, blockIdx.x, lane, bias, bias_is_f32, out, out_stride, M, N, mode, rope);
 }
 
-#ifndef AXON_STREAM_DEPTH
-#define AXON_STREAM_DEPTH 8
-#endif
+// ---------------------------------------------------------------------------- gemm_rows
+// 17 to 64 rows of X: still bound by reading W once, but X is now as large as a tile of W, and a
+// wave that fetched its own X for every step (as gemm_stream does) would ask the caches for as
+// many bytes of X as of W.  Here the WAVES waves of a block walk the same K together, each
+// with its own NT16 row tiles of W streamed from memory straight into MFMA operands (a ring of
+// NS - 1 steps of 64 k in flight), and share X: a step's X (64 rows x 64 k, 8 KB) goes straight
+// into LDS once a block, in the blocks of 1 KB that one LDS read of a wave takes (16 rows x 32 k,
+// lane l: row l % 16, 8 k from 8 (l / 16)), each wave fetching its share.  One barrier a step:
+// behind it the step's X is there for everyone and the step before is read by everyone, so its
+// place can be filled again.  A block works on one segment of K (blockIdx.y): with one segment
+// it ends with the product's epilogue, with more it leaves its sums in `partial`
+// [segment][gate | up][M][N] and the kernels that add such sums in segment order finish the
+// product.  The chain of an output element is the same as in every other kernel: 16x16x32
+// MFMAs in ascending k from zero over its segment.
+template <int NT16, int WAVES, int NS, int EPI>
+__global__ void __launch_bounds__(WAVES * 64, WAVES > 4 ? 1 : 8 / WAVES)      // up to two waves a SIMD: 256 registers each
+gemm_rows_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const void* __restrict__ bias,
+                 int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode,
+                 float* __restrict__ partial, int n_units) {
+  constexpr bool GLU = EPI == EPI_GLU;
+  // every wave fetches XI blocks of X a step (where the waves do not divide the blocks, some
+  // twice: the same bytes to the same place), so that every wave counts the same loads
+  constexpr int MT16 = 4, XB = MT16 * 2, XI = (XB + WAVES - 1) / WAVES, WI = NT16 * 2, LOADS = XI + WI;
+  static_assert(EPI == EPI_PLAIN || (EPI == EPI_GLU && NT16 == 2), "plain tiles, or gate and up tiles of the same columns");
+  static_assert((NS - 2) * LOADS < 64, "the counter of loads in flight has six bits");
+  extern __shared__ __align__(16) unsigned char x_ring[];      // [NS][XB][1 KB]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int unit = min((int)blockIdx.x * WAVES + wave, n_units - 1);     // past the last: the last again, nothing stored
+  const bool live = (int)blockIdx.x * WAVES + wave < n_units;
+  const int segs = gridDim.y, seg = blockIdx.y;
+  const int KB = K / 32;
+  const bf16_t* wtile[NT16];
+#pragma unroll
+  for (int i = 0; i < NT16; ++i) {
+    int tile;
+    if (GLU) tile = i * (N / 16) + unit;
+    else tile = min(unit * NT16 + i, (N + 15) / 16 - 1);
+    wtile[i] = w + (size_t)tile * KB * 512 + lane * 8;
+  }
+  // this wave's blocks of X: block b = (16 rows j, 32 k h), lane: row 16 j + lane % 16, 8 k from 8 (lane / 16)
+  const bf16_t* xsrc[XI];
+  int xdst[XI];
+#pragma unroll
+  for (int q = 0; q < XI; ++q) {
+    const int b = (wave * XI + q) % XB;
+    xsrc[q] = x + (size_t)min((b >> 1) * 16 + (lane & 15), M - 1) * x_stride + (b & 1) * 32 + (lane >> 4) * 8;
+    xdst[q] = b * 1024;
+  }
+  const int nk = K / 64;
+  const int first = (int)((long)seg * nk / segs);
+  const int mine = (int)((long)(seg + 1) * nk / segs) - first;      // the same for every wave of the block
+  const unsigned ring0 = (unsigned)(size_t)(lds_ptr_t)x_ring;
+
+  f32x4 acc[NT16][MT16];
+#pragma unroll
+  for (int i = 0; i < NT16; ++i)
+#pragma unroll
+    for (int j = 0; j < MT16; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  // In whole rounds of the ring every step issues the loads of the step NS - 1 ahead, also past
+  // the segment's end (then its last step again, which the cache still holds, into places nobody
+  // reads); the steps left after the last whole round issue nothing.  So the number of loads in
+  // flight at every wait is fixed by the code alone, for the kernel's count and for the compiler's.
+  uint4 wf[NS][NT16][2];
+  auto issue = [&](int slot, int local) {
+    const int k0 = (first + min(local, mine - 1)) * 64;
+    // X straight into LDS, written as an instruction (M0: where the wave's 1 KB goes): the compiler,
+    // seeing such a load in a loop, would wait for every load in flight once a round of the ring.
+    // It then counts the loads of W alone and waits a little earlier than it must: never too late.
+#pragma unroll
+    for (int q = 0; q < XI; ++q) {
+      const bf16_t* src = xsrc[q] + k0;
+      const unsigned dst = __builtin_amdgcn_readfirstlane(ring0 + slot * XB * 1024 + xdst[q]);
+      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(dst) : "memory", "m0");
+    }
+#pragma unroll
+    for (int i = 0; i < NT16; ++i) {
+      wf[slot][i][0] = *reinterpret_cast<const uint4*>(wtile[i] + k0 * 16);          // k block k0 / 32: 512 elements each
+      wf[slot][i][1] = *reinterpret_cast<const uint4*>(wtile[i] + k0 * 16 + 512);
+    }
+  };
+  // one step: behind the barrier its X is in LDS for every wave and nobody reads the step before
+  // any more (the bare barrier: the fence of __syncthreads would wait for every load under way)
+  auto multiply = [&](int d) {
+    u32x4 xf[XB];
+    read_frags<XB, 1024>(xf, ring0 + d * (XB * 1024) + lane * 16);
+    wait_lgkmcnt<0>();
+    use_frags<XB>(xf);
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < NT16; ++i)
+#pragma unroll
+        for (int j = 0; j < MT16; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[d][i][h]), as_frag(xf[j * 2 + h]), acc[i][j], 0, 0, 0);
+  };
+  static_assert(NS >= 4 && NS <= 8, "the ring of steps");
+#pragma unroll
+  for (int d = 0; d < NS - 1; ++d) issue(d, d);
+  int base = 0;
+  for (; base + NS <= mine; base += NS) {
+#pragma unroll
+    for (int d = 0; d < NS; ++d) {
+      wait_vmcnt<(NS - 2) * LOADS>();      // this step's loads have landed (loads return in order)
+      __builtin_amdgcn_s_barrier();
+      issue((d + NS - 1) % NS, base + d + NS - 1);
+      multiply(d);
+    }
+  }
+  const int left = mine - base;            // 0 .. NS - 1 steps, their loads under way already; the same for every wave
+#define ROWS_LAST(T)                                                \
+  if (T < NS - 1 && left > T) {                                     \
+    wait_vmcnt<(NS - 2 - (T < NS - 2 ? T : NS - 2)) * LOADS>();     \
+    __builtin_amdgcn_s_barrier();                                   \
+    multiply(T);                                                    \
+  }
+  ROWS_LAST(0) ROWS_LAST(1) ROWS_LAST(2) ROWS_LAST(3) ROWS_LAST(4) ROWS_LAST(5) ROWS_LAST(6)
+#undef ROWS_LAST
+  wait_vmcnt<0>();                         // the loads past the end: nothing of this block is in flight when it leaves
+  if (!live) return;
+  if (partial) {
+    // [segment][gate | up][M][N], 32-bit sums as they are; a lane: 4 consecutive columns of a row
+    constexpr int PARTS = GLU ? 2 : 1;
+#pragma unroll
+    for (int i = 0; i < NT16; ++i) {
+      const int part = GLU ? i : 0;
+      const int n = (GLU ? unit : unit * NT16 + i) * 16 + (lane >> 4) * 4;
+      if (n >= N) continue;
+      float* dst = partial + ((size_t)seg * PARTS + part) * M * N + n;
+#pragma unroll
+      for (int j = 0; j < MT16; ++j) {
+        const int m = j * 16 + (lane & 15);
+        if (m < M) *reinterpret_cast<float4*>(dst + (size_t)m * N) = make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+      }
+    }
+    return;
+  }
+  auto summed = [&](int t, int e) { return acc[t / MT16][t % MT16][e]; };
+  rows_epilogue<NT16, MT16, EPI, 1>(summed, 0, unit, lane, bias, bias_is_f32, out, out_stride, M, N, mode, RopeStore());
+}
+
+#define ROWS_NS 8
+
+template <int NT16, int WAVES, int EPI>
+static int launch_rows_of(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                          int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs, float* partial, int units) {
+  constexpr int lds_bytes = ROWS_NS * 8 * 1024;
+  gemm_rows_kernel<NT16, WAVES, ROWS_NS, EPI><<<dim3(ceil_div(units, WAVES), segs), WAVES * 64, lds_bytes, stream>>>(
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, segs > 1 ? partial : nullptr, units);
+  AXK_LAUNCH_CHECK("gemm_rows");
+  return 0;
+}
+
+// A CU streams at its own pace however many blocks it holds, so the waves of a block are as many
+// as it takes to give each of the chip's 256 CUs one block (at most eight: two a SIMD).
+template <int NT16, int EPI>
+static int launch_rows(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                       int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs, float* partial,
+                       const SplitNorm* norm, const RopeStore* rope) {
+  const int units = EPI == EPI_GLU ? n / 16 : ceil_div(ceil_div(n, 16), NT16);
+  int waves = ceil_div(units * segs, 256);
+  waves = waves < 2 ? 2 : waves > 8 ? 8 : waves;
+#define ARGS_ROWS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, segs, partial, units
+  int rc = -1;
+  switch (waves) {
+    case 2: rc = launch_rows_of<NT16, 2, EPI>(ARGS_ROWS); break;
+    case 3: rc = launch_rows_of<NT16, 3, EPI>(ARGS_ROWS); break;
+    case 4: rc = launch_rows_of<NT16, 4, EPI>(ARGS_ROWS); break;
+    case 5: rc = launch_rows_of<NT16, 5, EPI>(ARGS_ROWS); break;
+    case 6: rc = launch_rows_of<NT16, 6, EPI>(ARGS_ROWS); break;
+    case 7: rc = launch_rows_of<NT16, 7, EPI>(ARGS_ROWS); break;
+    default: rc = launch_rows_of<NT16, 8, EPI>(ARGS_ROWS); break;
+  }
+#undef ARGS_ROWS
+  if (rc != 0) return rc;
+  return segs > 1 ? add_split_sums(partial, segs, m, n, bias, bias_is_f32, out, out_stride, mode, norm, rope, stream) : 0;
+}
 
 template <int NT16, int MT16, int SEGS, int EPI>
 static int launch_stream(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                          int out_stride, int m, int n, int k, int mode, hipStream_t stream, const RopeStore& rope) {
-  // the ring as deep as the registers allow: (NT16 + MT16) 8 registers a step; eight waves a block
-  // leave each 256 registers, fewer waves 512
-  constexpr int BUDGET = SEGS == 8 ? 160 : 384, FIT = BUDGET / ((NT16 + MT16) * 8);
-  constexpr int DEPTH = FIT < AXON_STREAM_DEPTH ? FIT : AXON_STREAM_DEPTH;
+  // the ring as deep as the registers allow: (NT16 + MT16) 8 registers a step
+  constexpr int FIT = 384 / ((NT16 + MT16) * 8), DEPTH = FIT < 8 ? FIT : 8;
   gemm_stream_kernel<NT16, MT16, SEGS, DEPTH, EPI><<<ceil_div(n, EPI == EPI_GLU ? 16 : NT16 * 16), SEGS * 64, 0, stream>>>(
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, rope);
   AXK_LAUNCH_CHECK("gemm_stream");
@@ -863,9 +1056,8 @@ static int launch_stream_rows(const bf16_t* x, int x_stride, const bf16_t* w, co
     case 1: return launch_stream<NT16, MT16, 1, EPI>(ARGS);             \
     case 2: return launch_stream<NT16, MT16, 2, EPI>(ARGS);             \
     case 4: return launch_stream<NT16, MT16, 4, EPI>(ARGS);             \
-    case 8: return launch_stream<NT16, MT16, 8, EPI>(ARGS);             \
   }
-  if (m <= 16) { BY_SEGS(1) } else { BY_SEGS(2) }
+  BY_SEGS(1)
 #undef BY_SEGS
 #undef ARGS
   axk_set_error("gemm_stream: %d segments", segs);
@@ -934,10 +1126,10 @@ int gemm_segments(int tiles32, int k) {
 
 static int tiles32_of(int n, int mode) { return mode == MODE_SWIGLU ? n / 16 : (n + 31) / 32; }
 
-// The most rows the streaming kernel takes: beyond, every block would read more of X than of W.
-#ifndef AXON_STREAM_MAX_M
-#define AXON_STREAM_MAX_M 32
-#endif
+// The most rows the streaming kernel takes: with more, its waves, which fetch X each for itself,
+// ask the caches for as much of X as of W, and the kernel that shares X within a block is faster
+// (measured on the products of a 7B layer: from 17 rows on, by 10 to 30 %).
+#define AXON_STREAM_MAX_M 16
 
 // More rows than the streaming kernel takes, S > 1 segments: a block a segment (the blocks' sums
 // go through a workspace and are added in segment order by a second kernel; measured faster for
@@ -1002,14 +1194,15 @@ static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, co
   float* ws = (float*)workspace;
   const bool glu = mode == MODE_SWIGLU;
   if (m <= 64) {
-    // one tile of 64 rows; the segments in registers only where the sums cannot go through the workspace
+    // the segments in registers only where the sums cannot go through the workspace (one tile of 64 rows)
     if (segs > 1 && !across) {
       if (glu) return launch_tile<64, 256, 1, 4, true, true>(ARGS, segs);
       return launch_tile<64, 128, 1, 4, false, true, 64, 3>(ARGS, segs);
     }
-    if (glu) return launch_tile<64, 256, 1, 4, true>(ARGS, segs, ws);
-    if (n >= 8192) return launch_tile<64, 256, 1, 4, false>(ARGS, segs, ws, norm, rope_after);
-    return launch_tile<64, 128, 1, 4, false, false, 64, 3>(ARGS, segs, ws, norm, rope_after);
+    // W streamed, X shared through LDS; a block a segment.  Two row tiles a wave where the matrix is large.
+    if (glu) return launch_rows<2, EPI_GLU>(ARGS, segs, ws, nullptr, nullptr);
+    if (n >= 32 * 512) return launch_rows<2, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
+    return launch_rows<1, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
   }
   if (segs > 1 && !across) {
     // the segments in registers: 128 x 256 tiles (8 waves) where they occupy the chip, else 128 x 128
