@@ -450,19 +450,20 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
 }
 
 // ============================================================================ decoding tokens
-// grid (work items x kv heads): a block of four waves per (token, kv head, chunk of 256
-// positions); a wave takes one block of 64 of them, on its own: it brings the block's K into a
-// stage of LDS of its own and its V^T straight into registers as MFMA operands (every load
+// A wave takes one block of 64 positions of a (token, kv head): the range of a token is cut into
+// chunks of 256 positions, four such blocks each (grid: work items x kv heads, in blocks of four
+// waves or of one).  A wave is on its own from start to end: it brings the block's K into a stage of LDS (16 KB at head
+// size 128: ten waves fit a CU) and its V^T straight into registers as MFMA operands (every load
 // issued at once, 32 KB in flight per wave), runs attention_scores and the chains of
 // attention_values with the query heads of the group as the columns (a group of up to 32 heads)
 // and leaves (o_b, m_b, l_b) of every head in `partial`.  The work list names the chunks that
 // exist, token by token (item = token slot * CMB_MAX_CHUNKS + chunk, -1: nothing), so that a
-// batch of short and long contexts launches no block without work.  How a token's range is cut
+// batch of short and long contexts launches few blocks without work.  How a token's range is cut
 // depends on its own position and the window alone, never on the rest of the batch.
 // partial [token slot][head][block][HD + 2]: o_b, then m_b and l_b; blocks counted from the
 // chunk that holds the window's first position (or 0).
-template <int HD>
-__global__ void __launch_bounds__(256, 2)
+template <int HD, int BW>
+__global__ void __launch_bounds__(BW * 64, BW == 1 ? 3 : 2)      // waves a SIMD: three leave each 168 registers
 attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                         const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
                         const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
@@ -472,13 +473,16 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
   using S = AttStage<HD>;
   constexpr int KS = HD / 16, DT = HD / 32;
   extern __shared__ __align__(16) unsigned char smem[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int item = work[blockIdx.x / n_kv_heads];    // the kv heads of a chunk side by side: they share its pages
+  static_assert(DC_CHUNK / ATT_BLOCK == 4 && (BW == 1 || BW == 4), "four blocks of positions a chunk");
+  const int lane = threadIdx.x & 63;
+  const int wave = BW == 1 ? blockIdx.x & 3 : threadIdx.x >> 6;       // which 64 positions of the chunk
+  const int unit = BW == 1 ? blockIdx.x >> 2 : blockIdx.x;
+  const int item = work[unit / n_kv_heads];          // the kv heads of a chunk side by side: they share its pages
   if (item < 0) return;                              // padding of the list
   const int slot = item / CMB_MAX_CHUNKS, chunk = item % CMB_MAX_CHUNKS;
   if (slot >= n_tokens || chunk >= max_chunks) return;   // no item of this launch
   const int t = token_index ? token_index[slot] : slot;
-  const int kvh = blockIdx.x % n_kv_heads;
+  const int kvh = unit % n_kv_heads;
   const int group = n_heads / n_kv_heads;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
@@ -491,7 +495,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
   const size_t page_stride = (size_t)n_kv_heads * HD * page_size;
   const bf16_t* k_head = k_cache + (size_t)kvh * HD * page_size;
   const bf16_t* v_head = v_cache + (size_t)kvh * HD * page_size;
-  unsigned char* stage = smem + wave * S::K_BYTES;   // keys only
+  unsigned char* stage = smem + (BW == 1 ? 0 : wave) * S::K_BYTES;   // keys only
 
   // every page first, then every load: nothing waits behind a table entry.  V^T: k step s2 takes
   // the lane's positions p0 + 8 c .. + 7, c = 4 (s2 / 2) + 2 (s2 % 2) + half, of dim 32 dt + l32:
@@ -698,16 +702,19 @@ extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_c
               "attention_decode: bad arguments (tokens %d, chunks %d, window %d, q stride %d)", n_tokens, max_chunks,
               window, q_stride);
   AXK_REQUIRE(partial != nullptr && ((uintptr_t)partial & 7) == 0, "attention_decode: needs its workspace, 8-byte aligned");
-  AXK_REQUIRE(n_work >= 0 && (n_work == 0 || work != nullptr) && (long)n_work * n_kv_heads < (1l << 31),
+  AXK_REQUIRE(n_work >= 0 && (n_work == 0 || work != nullptr) && (long)n_work * n_kv_heads * 4 < (1l << 31),
               "attention_decode: a work list of %d items", n_work);
   if (n_tokens == 0 || n_work == 0) return 0;
-  dim3 grid((unsigned)n_work * n_kv_heads), cgrid(n_tokens, n_heads);
-#define LAUNCH(HD)                                                                                                   \
+  // A wave a block where every wave finds a place on the chip at once (ten a CU): an even spread
+  // over the CUs; blocks of four waves where there are more, which are launched faster.
+  const bool single = (long)n_work * n_kv_heads * 4 <= 2560;
+  dim3 cgrid(n_tokens, n_heads);
+#define LAUNCH(HD, BW)                                                                                               \
   {                                                                                                                  \
     static bool configured = false;                                                                                  \
-    constexpr int lds = 4 * ATT_BLOCK * HD * 2;                              /* a wave its block's keys */        \
+    constexpr int lds = BW * ATT_BLOCK * HD * 2;                             /* a wave its block's keys */        \
     if (!configured) {                                                                                               \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_kernel<HD>),                \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_kernel<HD, BW>),            \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);                           \
       if (e != hipSuccess) {                                                                                         \
         axk_set_error("attention_decode: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));            \
@@ -715,14 +722,15 @@ extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_c
       }                                                                                                              \
       configured = true;                                                                                             \
     }                                                                                                                \
-    attention_decode_kernel<HD><<<grid, 256, lds, (hipStream_t)stream>>>(                                            \
+    attention_decode_kernel<HD, BW><<<(unsigned)n_work * n_kv_heads * (4 / BW), BW * 64, lds, (hipStream_t)stream>>>( \
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,       \
         positions, seq_rows, token_index, n_tokens, work, partial, max_chunks, n_heads, n_kv_heads, page_size,       \
         window, scale);                                                                                              \
     attention_combine_kernel<HD><<<cgrid, HD, 0, (hipStream_t)stream>>>(partial, positions, token_index,            \
                                                                        (bf16_t*)out, max_chunks, n_heads, window);   \
   }
-  if (head_dim == 64) LAUNCH(64) else LAUNCH(128)
+  if (head_dim == 64) { if (single) LAUNCH(64, 1) else LAUNCH(64, 4) }
+  else { if (single) LAUNCH(128, 1) else LAUNCH(128, 4) }
 #undef LAUNCH
   AXK_LAUNCH_CHECK("attention_decode");
   return 0;

@@ -82,7 +82,8 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
                  int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode, int m_blocks,
                  int n_blocks, float* __restrict__ partial, int segs) {
   extern __shared__ __align__(16) unsigned char smem[];
-  static_assert(BK == 64, "segments of K are counted in steps of 64");
+  static_assert(BK == 64 || BK == 32, "segments of K are counted in steps of 64: whole K tiles");
+  constexpr int PER64 = 64 / BK;                       // K tiles in a step of 64
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // a wave's tile
   constexpr int TM = WM / 32, TN = WN / 32;            // in 32 x 32 MFMA tiles
@@ -146,8 +147,8 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
 
   // Split K (gridDim.y > 1): this block multiplies the K tiles kt_begin .. kt_begin + nk - 1 and
   // leaves its sums in `partial`; gemm_split_reduce_kernel adds the blocks' sums in block order.
-  const int kt_begin = (int)((long)blockIdx.y * (K / BK) / gridDim.y);
-  const int nk = (int)((long)(blockIdx.y + 1) * (K / BK) / gridDim.y) - kt_begin;
+  const int kt_begin = (int)((long)blockIdx.y * (K / 64) / gridDim.y) * PER64;
+  const int nk = (int)((long)(blockIdx.y + 1) * (K / 64) / gridDim.y) * PER64 - kt_begin;
   auto issue = [&](int kt) {     // kt counts from kt_begin
     unsigned char* stage = smem + (kt % STAGES) * STAGE;
     const int koff = (kt_begin + kt) * BK;
@@ -172,7 +173,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
         acc[i][j][e] = 0.0f;
         if (SEG) total[i][j][e] = 0.0f;
       }
-  int seg_at = 0, seg_end = SEG ? (int)((long)nk / segs) : 0;   // SEG: the segment under way ends before K tile seg_end
+  int seg_at = 0, seg_end = SEG ? (int)((long)(nk / PER64) / segs) * PER64 : 0;   // SEG: the segment under way ends before K tile seg_end
 
   // fragment addresses: row = tile row + lane % 32, k chunk = 2 ks + lane / 32, slot = chunk ^ SWZ(row)
   const int frow = lane & 31, fhalf = lane >> 5, fsw = SWZ(frow);
@@ -250,7 +251,7 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
             acc[i][j][e] = 0.0f;
           }
       ++seg_at;
-      seg_end = (int)((long)(seg_at + 1) * nk / segs);
+      seg_end = (int)((long)(seg_at + 1) * (nk / PER64) / segs) * PER64;
     }
   }
 #undef SWZ
@@ -603,6 +604,50 @@ static int launch_split_reduce_rope(const float* partial, int splits, int m, int
   return 0;
 }
 
+// What the rotary epilogue reads besides the sums (a token's position, the page it is stored in,
+// its sines and cosines): a chain of dependent loads that can start before the product does.
+template <int MT16>
+struct RopeAhead {
+  int pos[MT16], page[MT16];
+  float4 t0[MT16], t1[MT16];
+};
+
+// First the loads that depend on nothing (issued before the product's own first loads), then,
+// once those are under way, the page, which needs the position.
+template <int MT16, int SHARE>
+__device__ inline RopeAhead<MT16> rope_look_ahead(const RopeStore& rope, int share, int unit, int lane, int M) {
+  RopeAhead<MT16> ahead;
+  const int half = rope.head_dim / 2, per_head = half / 16;
+  const int slot = unit / per_head, d = (unit % per_head) * 16 + (lane >> 4) * 4;
+#pragma unroll
+  for (int j = 0; j < MT16; ++j) {
+    ahead.pos[j] = ahead.page[j] = 0;
+    ahead.t0[j] = ahead.t1[j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    const int m = j * 16 + (lane & 15);
+    if (j % SHARE != share || m >= M) continue;
+    if (slot >= rope.n_heads) {
+      ahead.pos[j] = rope.positions[m];
+      ahead.page[j] = rope.seq_rows[m];                 // the row of the block table, until rope_look_ahead_page
+    }
+    if (slot < rope.n_heads + rope.n_kv_heads) {
+      const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * half + d) * 2);
+      ahead.t0[j] = tab[0];
+      ahead.t1[j] = tab[1];
+    }
+  }
+  return ahead;
+}
+
+template <int MT16, int SHARE>
+__device__ inline void rope_look_ahead_page(RopeAhead<MT16>& ahead, const RopeStore& rope, int share, int unit, int lane, int M) {
+  const int slot = unit / (rope.head_dim / 32);
+#pragma unroll
+  for (int j = 0; j < MT16; ++j) {
+    if (j % SHARE != share || j * 16 + (lane & 15) >= M || slot < rope.n_heads) continue;
+    ahead.page[j] = rope.block_table[(size_t)ahead.page[j] * rope.table_stride + ahead.pos[j] / rope.page_size];
+  }
+}
+
 // What a wave does with finished sums (`summed(t, e)`: tile t = i * MT16 + j, element e; a lane
 // holds X row 16 j + lane % 16 and W rows 4 (lane / 16) .. + 3 of tile i): the epilogue of the
 // product.  `unit` names the tiles: for PLAIN the columns from unit * NT16 * 16, for GLU gate and
@@ -611,7 +656,7 @@ static int launch_split_reduce_rope(const float* partial, int splits, int m, int
 template <int NT16, int MT16, int EPI, int SHARE, class Summed>
 __device__ inline void rows_epilogue(Summed summed, int share, int unit, int lane, const void* __restrict__ bias,
                                      int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int mode,
-                                     const RopeStore& rope) {
+                                     const RopeStore& rope, const RopeAhead<MT16>& ahead) {
   constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE;
   const int r16 = lane & 15;
   const int n0 = unit * (GLU ? 16 : NT16 * 16);
@@ -640,8 +685,7 @@ __device__ inline void rows_epilogue(Summed summed, int share, int unit, int lan
       if (slot < rope.n_heads) {
         dst = reinterpret_cast<bf16_t*>(out) + (size_t)m * out_stride + (size_t)slot * hd;
       } else {
-        const int pos = rope.positions[m];
-        const int page = rope.block_table[(size_t)rope.seq_rows[m] * rope.table_stride + pos / rope.page_size];
+        const int pos = ahead.pos[j], page = ahead.page[j];
         const int in_page = pos % rope.page_size;
         if (slot >= rope.n_heads + rope.n_kv_heads) {
           const int kvh = slot - rope.n_heads - rope.n_kv_heads;
@@ -656,8 +700,7 @@ __device__ inline void rows_epilogue(Summed summed, int share, int unit, int lan
         const int kvh = slot - rope.n_heads;
         dst = rope.k_cache + (((size_t)page * rope.n_kv_heads + kvh) * rope.page_size + in_page) * hd;
       }
-      const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * half + d) * 2);
-      const float4 t0 = tab[0], t1 = tab[1];
+      const float4 t0 = ahead.t0[j], t1 = ahead.t1[j];
       const float sn[4] = {t0.x, t0.z, t1.x, t1.z}, cs[4] = {t0.y, t0.w, t1.y, t1.w};
       float lo[4], hi[4];
 #pragma unroll
@@ -815,9 +858,12 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[slot][i][h]), as_frag(xf[slot][j][h]), acc[i][j],
                                                               0, 0, 0);
   };
+  RopeAhead<MT16> ahead;
+  if (ROPE) ahead = rope_look_ahead<MT16, SEGS>(rope, seg, blockIdx.x, lane, M);
   if (mine > 0) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) load(d, min(d, mine - 1));   // beyond this wave's steps: a valid step again
+    if (ROPE) rope_look_ahead_page<MT16, SEGS>(ahead, rope, seg, blockIdx.x, lane, M);
     int base = 0;  // the ring holds local steps base .. base + DEPTH - 1
     for (; base + 2 * DEPTH <= mine; base += DEPTH) {
 #pragma unroll
@@ -855,7 +901,8 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
     return sum;
   };
 
-  rows_epilogue<NT16, MT16, EPI, SEGS>(summed, seg, blockIdx.x, lane, bias, bias_is_f32, out, out_stride, M, N, mode, rope);
+  rows_epilogue<NT16, MT16, EPI, SEGS>(summed, seg, blockIdx.x, lane, bias, bias_is_f32, out, out_stride, M, N, mode, rope,
+                                       ahead);
 }
 
 // ---------------------------------------------------------------------------- gemm_rows
@@ -873,7 +920,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
 // product.  The chain of an output element is the same as in every other kernel: 16x16x32
 // MFMAs in ascending k from zero over its segment.
 template <int NT16, int WAVES, int NS, int EPI>
-__global__ void __launch_bounds__(WAVES * 64, WAVES > 4 ? 1 : 8 / WAVES)      // up to two waves a SIMD: 256 registers each
+__global__ void __launch_bounds__(WAVES * 64, 2)      // two waves a SIMD: 256 registers each
 gemm_rows_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const void* __restrict__ bias,
                  int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode,
                  float* __restrict__ partial, int n_units) {
@@ -930,7 +977,11 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
     for (int q = 0; q < XI; ++q) {
       const bf16_t* src = xsrc[q] + k0;
       const unsigned dst = __builtin_amdgcn_readfirstlane(ring0 + slot * XB * 1024 + xdst[q]);
-      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(dst) : "memory", "m0");
+      unsigned kept;                                      // M0 goes back as it was: the compiler counts on it
+      asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                   : "=&s"(kept)
+                   : "v"(src), "s"(dst)
+                   : "memory");
     }
 #pragma unroll
     for (int i = 0; i < NT16; ++i) {
@@ -995,7 +1046,8 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
     return;
   }
   auto summed = [&](int t, int e) { return acc[t / MT16][t % MT16][e]; };
-  rows_epilogue<NT16, MT16, EPI, 1>(summed, 0, unit, lane, bias, bias_is_f32, out, out_stride, M, N, mode, RopeStore());
+  rows_epilogue<NT16, MT16, EPI, 1>(summed, 0, unit, lane, bias, bias_is_f32, out, out_stride, M, N, mode, RopeStore(),
+                                    RopeAhead<MT16>());
 }
 
 #define ROWS_NS 8
