@@ -95,7 +95,7 @@ int axk_pack_matrix(const void* src, void* dst, int rows, int k, void* stream);
 // float32 [M, N] (the residual stream); 2: store float32 [M, N] (logits); 3: W holds 2 N rows,
 // gate rows then up rows, and out elem [M, N] = silu(X . gate^T) * (X . up^T) (no bias).
 // x_stride / out_stride: elements between rows.  workspace: axk_gemm_workspace(m, n, k, mode) bytes
-// (0 for most shapes: then it may be null), 16-byte aligned; products of more than 64 rows with a
+// (0 for most shapes: then it may be null), 16-byte aligned; products of more than 16 rows with a
 // narrow output give each segment of K blocks of their own and add the segments' sums through it.
 //
 // With a packed W every output element is the sum, in ascending order, of axk_gemm_segments(n, k,
@@ -126,7 +126,7 @@ int axk_gemm_then_norm(const void* x, int x_stride, const void* w, const void* b
 // The attention's [q; k; v] product (W packed, [(n_heads + 2 n_kv_heads) head_dim, K], or the q rows alone
 // if write_kv is 0) with what follows it in the same launches: bias, the rotary encoding of q and k
 // heads over their whole width (table [M, head_dim / 2, 2]: sin, cos), q into qkv [M, >= n_heads
-// head_dim], k and v into the request's pages (as axk_rope_kv_write stores them).  Up to 64 rows it
+// head_dim], k and v into the request's pages (as axk_rope_kv_write stores them).  Up to 16 rows it
 // is the product's epilogue; with more rows, where the product runs with a block per segment of K
 // (axk_gemm_qkv_rope_ok says so; n = the rows of W), the kernel that adds the segments' sums rotates
 // and stores; workspace: axk_gemm_workspace(m, n, k, 0) bytes.  Bit-identical to axk_gemm followed

@@ -18,12 +18,17 @@
 // get it from exact block sums, src/cuda/decode.cu:352-369).  The kernels are chosen by M, for
 // speed alone:
 //
-// * gemm_stream (M <= 64): bound by reading W once.  A wave owns 32 rows of W and one segment of
-//   K and streams its share from memory straight into MFMA operands, keeping a ring of steps
-//   in flight; W is the A operand, up to 64 rows of X the B operand.  The waves of a block are
-//   the segments of one tile of rows (or several tiles where S is small); their sums are added
-//   in segment order through LDS.  Epilogues: bias / residual add / SwiGLU, and the attention's
-//   qkv product with the rotary encoding and the store into the paged cache.
+// * gemm_stream (M <= 16): bound by reading W once.  A wave owns one or two tiles of 16 rows of W
+//   and one segment of K and streams its share from memory straight into 16x16x32 MFMA operands
+//   (one such MFMA gives the bits of two chained 32x32x16 ones over the same k), keeping a ring
+//   of steps in flight; W is the A operand, the rows of X the B operand.  The waves of a block
+//   are the segments of its tiles; their sums are added in segment order through LDS.
+//   Epilogues: bias / residual add / SwiGLU, and the attention's qkv product with the rotary
+//   encoding and the store into the paged cache.
+//
+// * gemm_rows (17 <= M <= 64): W still streams into registers, but the waves of a block walk the
+//   same segment of K and share X through LDS; a block a segment, the sums of several segments
+//   through a workspace.
 //
 // * gemm_tile (M > 64): a block of 4 or 8 waves owns a BM x BN tile of the output, walks K in
 //   steps of 64 through LDS stages filled by direct global -> LDS loads (the next step's loads
@@ -519,11 +524,11 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
 }
 
 // ---------------------------------------------------------------------------- gemm_stream
-// Up to 64 rows of X: the product is bound by reading W once.  A block owns NT16 row tiles (of
+// Up to 16 rows of X: the product is bound by reading W once.  A block owns NT16 row tiles (of
 // 16) of W; its waves are the S segments of K, each streaming its share of the tiles from memory
 // straight into 16x16x32 MFMA operands (a packed block as it lies in memory, 1 KB an
 // instruction), keeping a ring of steps in flight so that the memory pipe never drains, and
-// multiplying with up to 64 rows of X (the B operand: lane l holds row l % 16, 8 consecutive k
+// multiplying with the rows of X (the B operand: lane l holds row l % 16, 8 consecutive k
 // from (l / 16) * 8).  C[n][m] tiles of 16 x 16: a lane ends with 4 consecutive n of one m, one
 // vector store.  The segments' sums meet in LDS and are added in segment order.  A 16x16x32 MFMA
 // gives the bits of two chained 32x32x16 MFMAs over the same 32 k (measured over wide ranges of
@@ -553,24 +558,38 @@ enum { EPI_PLAIN = 0, EPI_GLU = 1, EPI_ROPE = 2 };
 
 // The sums of a split [q; k; v] product with the bias, the rotary encoding and the store into the
 // pages: what gemm_split_reduce_kernel (storing bfloat16) and the rotary kernel do one after the
-// other, bit for bit.  One wave per (token, head slot), four waves a block; q heads go rotated to
-// `out`, k heads rotated into the request's page of keys, v heads as they are into its page of
-// values.  Every head is rotated over its whole width.
+// other, bit for bit.  A block per token and group of head slots; a thread takes 4 consecutive dims
+// of a head's lower half and their partners in the upper half (every load a float4, all of a
+// thread's loads independent of each other); q heads go rotated to `out`, k heads rotated into the
+// request's page of keys, v heads as they are into its page of values.  Every head is rotated
+// over its whole width.
 __global__ void __launch_bounds__(256)
 gemm_split_reduce_rope_kernel(const float* __restrict__ partial, int splits, int M, int N, const void* __restrict__ bias,
                               int bias_is_f32, bf16_t* __restrict__ out, int out_stride, RopeStore rope) {
-  const int m = blockIdx.x, slot = blockIdx.y * 4 + threadIdx.x / AXON_WAVE, lane = threadIdx.x % AXON_WAVE;
-  const int hd = rope.head_dim, half = hd / 2;
-  if (slot * hd >= N) return;
+  const int hd = rope.head_dim, half = hd / 2, per_head = half / 4;     // threads a head
+  const int heads_a_block = 256 / per_head;
+  const int m = blockIdx.x, within = threadIdx.x / per_head, slot = blockIdx.y * heads_a_block + within;
+  const int d = (threadIdx.x % per_head) * 4;
+  if (within >= heads_a_block || slot * hd >= N) return;
   const size_t plane = (size_t)M * N;
-  // a column's sum, rounded as the product's own store rounds it
-  auto value = [&](int col) {
+  // four columns' sums, rounded as the product's own store rounds them
+  auto values = [&](int col, float (&v)[4]) {
     const float* src = partial + (size_t)m * N + col;
-    float g = src[0];
-    for (int z = 1; z < splits; ++z) g += src[(size_t)z * plane];
-    if (bias) g += load_vec(bias, bias_is_f32, col);
-    return bf16_to_float(float_to_bf16(g));
+    float4 g = *reinterpret_cast<const float4*>(src);
+    for (int z = 1; z < splits; ++z) {
+      const float4 a = *reinterpret_cast<const float4*>(src + (size_t)z * plane);
+      g.x += a.x; g.y += a.y; g.z += a.z; g.w += a.w;
+    }
+    v[0] = g.x; v[1] = g.y; v[2] = g.z; v[3] = g.w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (bias) v[e] += load_vec(bias, bias_is_f32, col + e);
+      v[e] = bf16_to_float(float_to_bf16(v[e]));
+    }
   };
+  float a[4], b[4];
+  values(slot * hd + d, a);
+  values(slot * hd + half + d, b);
   bf16_t* dst;
   if (slot < rope.n_heads) {
     dst = out + (size_t)m * out_stride + (size_t)slot * hd;
@@ -581,23 +600,37 @@ gemm_split_reduce_rope_kernel(const float* __restrict__ partial, int splits, int
     if (slot >= rope.n_heads + rope.n_kv_heads) {
       const int kvh = slot - rope.n_heads - rope.n_kv_heads;
       bf16_t* vdst = rope.v_cache + ((size_t)page * rope.n_kv_heads + kvh) * hd * rope.page_size + in_page;
-      for (int i = lane; i < hd; i += AXON_WAVE) vdst[(size_t)i * rope.page_size] = float_to_bf16(value(slot * hd + i));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        vdst[(size_t)(d + e) * rope.page_size] = float_to_bf16(a[e]);
+        vdst[(size_t)(half + d + e) * rope.page_size] = float_to_bf16(b[e]);
+      }
       return;
     }
     dst = rope.k_cache + (((size_t)page * rope.n_kv_heads + (slot - rope.n_heads)) * rope.page_size + in_page) * hd;
   }
-  const float* tab = rope.table + (size_t)m * half * 2;
-  for (int i = lane; i < half; i += AXON_WAVE) {
-    const float sn = tab[2 * i], cs = tab[2 * i + 1];
-    const float a = value(slot * hd + i), b = value(slot * hd + i + half);
-    dst[i] = float_to_bf16(__fsub_rn(__fmul_rn(a, cs), __fmul_rn(b, sn)));
-    dst[i + half] = float_to_bf16(__fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, cs)));
+  const float4* tab = reinterpret_cast<const float4*>(rope.table + ((size_t)m * half + d) * 2);
+  const float4 t0 = tab[0], t1 = tab[1];
+  const float sn[4] = {t0.x, t0.z, t1.x, t1.z}, cs[4] = {t0.y, t0.w, t1.y, t1.w};
+  float lo[4], hi[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    lo[e] = __fsub_rn(__fmul_rn(a[e], cs[e]), __fmul_rn(b[e], sn[e]));
+    hi[e] = __fadd_rn(__fmul_rn(a[e], sn[e]), __fmul_rn(b[e], cs[e]));
   }
+  uint2 pk;
+  pk.x = pack2_bf16(lo[0], lo[1]);
+  pk.y = pack2_bf16(lo[2], lo[3]);
+  *reinterpret_cast<uint2*>(dst + d) = pk;
+  pk.x = pack2_bf16(hi[0], hi[1]);
+  pk.y = pack2_bf16(hi[2], hi[3]);
+  *reinterpret_cast<uint2*>(dst + half + d) = pk;
 }
 
 static int launch_split_reduce_rope(const float* partial, int splits, int m, int n, const void* bias, int bias_is_f32,
                                     void* out, int out_stride, const RopeStore& rope, hipStream_t stream) {
-  const dim3 grid(m, ceil_div(n / rope.head_dim, 4));
+  const int heads_a_block = 256 / (rope.head_dim / 8);
+  const dim3 grid(m, ceil_div(n / rope.head_dim, heads_a_block));
   gemm_split_reduce_rope_kernel<<<grid, 256, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, (bf16_t*)out, out_stride,
                                                           rope);
   AXK_LAUNCH_CHECK("gemm_split_reduce_rope");
@@ -1302,7 +1335,7 @@ int launch_gemm_mfma(const bf16_t* x, int x_stride, const bf16_t* w, const void*
                             then_norm ? &after : nullptr, workspace, workspace_bytes, nullptr);
 }
 
-// The [q; k; v] product with rotary encoding and cache store (see RopeStore): up to 64 rows in
+// The [q; k; v] product with rotary encoding and cache store (see RopeStore): up to 16 rows in
 // the epilogue of gemm_stream, more rows where the product runs with a block a segment (then the
 // kernel that adds the segments' sums rotates and stores); every head rotated over its whole
 // width, halves of a head a multiple of 16 wide.

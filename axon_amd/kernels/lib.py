@@ -246,7 +246,7 @@ class Kernels:
     def gemm_qkv_rope(self, x, w, bias, qkv, table, positions, seq_rows, block_table, k_cache, v_cache, n_heads,
                       n_kv_heads, head_dim, page_size, write_kv=True) -> None:
         """The [q; k; v] product, the rotary encoding and the store into the pages in one launch
-        (up to 64 tokens) or with the kernel that adds a product's segments doing the rest:
+        (up to 16 tokens) or with the kernel that adds a product's segments doing the rest:
         the same bits as `gemm` into qkv followed by `rope_kv_write`.  q lands in qkv[:, :n_heads *
         head_dim]; the k and v columns of qkv are not written.  Without write_kv, w holds the q
         rows only."""
