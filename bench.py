@@ -212,7 +212,7 @@ def main() -> int:
         # tokens, which the host draws and so cannot run ahead
         ps = [prompt(prompt_len) for _ in range(args.batch)]
         n_new = min(steps, 64)
-        llm.generate(ps, max_new_tokens=3)                            # graphs of this batch are captured here
+        llm.generate(ps, max_new_tokens=n_new)                        # the graphs of these steps are captured here
         for label, kw in (("greedy", {}), ("stop_token", dict(stop=[V - 1])),
                           ("sampled", dict(temperature=0.8, top_k=40, seed=1))):
             llm.generate(ps, max_new_tokens=n_new, **kw)
