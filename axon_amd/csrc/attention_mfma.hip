@@ -58,6 +58,8 @@ __device__ inline uint32_t pack_bf16(float a, float b) { return pack2_bf16(a, b)
 // loads of 16 bytes a lane (an instruction fills 1 KB: 1024 / (2 HD) rows of K, or 8 rows of
 // V^T).  16-byte slots of a row are permuted (slot ^ row & 7) so that fragment reads of
 // neighbouring rows fall into different banks.
+#define ATT_ZERO16 (f32x16{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f})
+
 template <int HD>
 struct AttStage {
   static constexpr int K_BYTES = ATT_BLOCK * HD * 2;
@@ -70,19 +72,24 @@ struct AttStage {
   static constexpr int V_INSTR = HD / 8;                         // and of its V^T
 };
 
+// Pages hold a power of two of positions (axk_attention_fast_ok): the page of a position and its
+// place in it by a shift and a mask, not by a division (which costs some twenty instructions).
+__device__ __forceinline__ int page_index(int p, int page_size) { return p >> (31 - __builtin_clz(page_size)); }
+__device__ __forceinline__ int page_offset(int p, int page_size) { return p & (page_size - 1); }
+
 // The page a lane's piece of load instruction `instr` lies in (looked up ahead of the load that
 // uses it).  Positions past `hi` (never written for this request): any valid row.
 template <int HD>
 __device__ __forceinline__ int att_k_page(int instr, int lane, int p0, int hi, const int32_t* table_row, int page_size) {
   const int row = instr * AttStage<HD>::K_ROWS_PER_INSTR + lane / AttStage<HD>::KCH;
-  return table_row[min(p0 + row, hi) / page_size];
+  return table_row[page_index(min(p0 + row, hi), page_size)];
 }
 
 template <int HD>
 __device__ __forceinline__ int att_v_page(int instr, int lane, int p0, int hi, const int32_t* table_row, int page_size) {
   const int d = instr * 8 + (lane >> 3);
   const int chunk = (lane & 7) ^ (d & 7);
-  return table_row[min(p0 + chunk * 8, hi) / page_size];
+  return table_row[page_index(min(p0 + chunk * 8, hi), page_size)];
 }
 
 // K: lane i of instruction `instr` brings row i / KCH of the instruction's rows, into slot i % KCH,
@@ -94,7 +101,7 @@ __device__ __forceinline__ void att_issue_k(unsigned char* stage, int instr, int
   const int row = instr * S::K_ROWS_PER_INSTR + lane / S::KCH;
   const int chunk = (lane % S::KCH) ^ (row & 7);
   const int p = min(p0 + row, hi);
-  const bf16_t* src = k_head + (size_t)page * page_stride + (size_t)(p % page_size) * HD + chunk * 8;
+  const bf16_t* src = k_head + (size_t)page * page_stride + (size_t)page_offset(p, page_size) * HD + chunk * 8;
   __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + instr * 1024), 16, 0, 0);
 }
 
@@ -107,7 +114,7 @@ __device__ __forceinline__ void att_issue_v(unsigned char* stage, int instr, int
   const int d = instr * 8 + (lane >> 3);
   const int chunk = (lane & 7) ^ (d & 7);
   const int p = min(p0 + chunk * 8, hi);
-  const bf16_t* src = v_head + (size_t)page * page_stride + (size_t)d * page_size + ((p % page_size) & ~7);
+  const bf16_t* src = v_head + (size_t)page * page_stride + (size_t)d * page_size + (page_offset(p, page_size) & ~7);
   __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + S::K_BYTES + instr * 1024), 16, 0, 0);
 }
 
@@ -148,11 +155,7 @@ __device__ __forceinline__ void attention_scores(unsigned st, const bf16x8 (&qf)
   const unsigned k_at = st + k_row * S::KROW, k_swz = k_row & 7;
 
   // S^T [64 positions][32 queries] = K Q^T: two tiles of 32 positions, two k steps a group
-  f32x16 s_acc[2];
-#pragma unroll
-  for (int pt = 0; pt < 2; ++pt)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) s_acc[pt][e] = 0.0f;
+  f32x16 s_acc[2];                    // each chain starts from the constant zero
   u32x4 kf[2][4];
   auto read_k = [&](u32x4 (&dst)[4], int ks0) {
 #pragma unroll
@@ -177,7 +180,7 @@ __device__ __forceinline__ void attention_scores(unsigned st, const bf16x8 (&qf)
 #pragma unroll
       for (int pt = 0; pt < 2; ++pt)
         s_acc[pt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[g & 1][kk * 2 + pt]),
-                                                            qf[2 * g + kk], s_acc[pt], 0, 0, 0);
+                                                            qf[2 * g + kk], g + kk == 0 ? ATT_ZERO16 : s_acc[pt], 0, 0, 0);
   }
 
   // the largest raw score first (the scale is positive), then exp2(score * c - max * c) in one
@@ -252,11 +255,10 @@ __device__ __forceinline__ void attention_values(unsigned st, const bf16x8 (&pf)
       wait_lgkmcnt<0>();
     }
     use_frags<4>(vf[dt & 1]);
-    f32x16 tile;
+    // the chain starts from the constant zero (an operand of the instruction, not sixteen registers to clear)
+    f32x16 tile = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[dt & 1][0]), pf[0], ATT_ZERO16, 0, 0, 0);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) tile[e] = 0.0f;
-#pragma unroll
-    for (int s2 = 0; s2 < 4; ++s2)
+    for (int s2 = 1; s2 < 4; ++s2)
       tile = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[dt & 1][s2]), pf[s2], tile, 0, 0, 0);
     consume(dt, tile);
   }
@@ -269,11 +271,9 @@ __device__ __forceinline__ void attention_values_of(const uint4 (&vf)[HD / 32][4
   constexpr int DT = HD / 32;
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
-    f32x16 tile;
+    f32x16 tile = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_of(vf[dt][0]), pf[0], ATT_ZERO16, 0, 0, 0);
 #pragma unroll
-    for (int e = 0; e < 16; ++e) tile[e] = 0.0f;
-#pragma unroll
-    for (int s2 = 0; s2 < 4; ++s2)
+    for (int s2 = 1; s2 < 4; ++s2)
       tile = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_of(vf[dt][s2]), pf[s2], tile, 0, 0, 0);
     consume(dt, tile);
   }
@@ -509,8 +509,8 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
     const int pa = p0 + 8 * (4 * (s2 >> 1) + 2 * (s2 & 1) + half);
     keep[s2] = max(0, min(pos - pa + 1, 8));          // positions past the token were never written
     const int pa_c = min(pa, pos);
-    v_page[s2] = table_row[pa_c / page_size];
-    v_at[s2] = (pa_c % page_size) & ~7;
+    v_page[s2] = table_row[page_index(pa_c, page_size)];
+    v_at[s2] = page_offset(pa_c, page_size) & ~7;
   }
 #pragma unroll
   for (int n = 0; n < S::K_INSTR; ++n) att_issue_k<HD>(stage, n, lane, k_page[n], p0, pos, k_head, page_stride, page_size);

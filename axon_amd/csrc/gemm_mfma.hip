@@ -1218,12 +1218,12 @@ static int tiles32_of(int n, int mode) { return mode == MODE_SWIGLU ? n / 16 : (
 
 // More rows than the streaming kernel takes, S > 1 segments: a block a segment (the blocks' sums
 // go through a workspace and are added in segment order by a second kernel; measured faster for
-// every product of the 7B and 14B layers up to 2,048 rows, and the only way to occupy the chip
-// when the output is small), unless the workspace would pass 256 MB: then blocks walk all of K
+// every product of the 7B and 14B layers up to 8,192 rows, and the only way to occupy the chip
+// when the output is small), unless the workspace would pass 2 GB: then blocks walk all of K
 // and keep the segments apart in registers.  Decided by the sizes alone.
 static bool segments_across_blocks(int m, int n, int k, int mode, int segs) {
   if (segs <= 1 || n % 4 != 0) return false;
-  return (size_t)segs * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float) <= ((size_t)256 << 20);
+  return (size_t)segs * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float) <= ((size_t)2048 << 20);
 }
 
 size_t gemm_workspace_bytes(int m, int n, int k, int mode) {

@@ -116,7 +116,8 @@ def main() -> int:
 
     prefill_point = prefill(PREFILL_TOKENS, args.steps if args.phase == "prefill" and args.steps else 4)
     if args.phase == "prefill":
-        print(json.dumps({"phase": "prefill", "prefill": prefill_point, "layers": L}))
+        print(json.dumps({"phase": "prefill", "prefill": prefill_point, "prefill_8192": prefill(min(8192, ctx_len), 2),
+                          "layers": L}))
         return 0
 
     # ---- decode at a batch size: prefill every request, then time K steps
