@@ -216,7 +216,9 @@ def test_gemm_rows_do_not_depend_on_the_batch(dtype):
     number of rows (src/lm.rs:272-278): every kernel a product may meet adds in the one order its
     matrix fixes."""
     k = kernels(dtype)
-    for N, K in [(96, 80), (256, 512), (130, 1000), (512, 1024), (300, 4096), (200, 8192), (4100, 256)]:
+    # the last three: blocks of 3, 6 and 8 waves in the kernel for 17 to 64 rows
+    for N, K in [(96, 80), (256, 512), (130, 1000), (512, 1024), (300, 4096), (200, 8192), (4100, 256), (9600, 256),
+                 (6144, 2048), (8192, 2048)]:
         x, _ = as_dtype(rnd(2100, K, seed=14), dtype)
         w, _ = as_dtype(rnd(N, K, seed=15, scale=0.2), dtype)
         w = packed(k, w)
