@@ -573,42 +573,77 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
   }
 }
 
-// The fold of a token's blocks, in ascending order, with the prompt kernel's own instructions.
-// grid (tokens, heads), HD threads: thread d folds dim d; every thread folds (m, l) for itself.
+// The fold of a token's blocks, in ascending order, with the prompt kernel's own arithmetic
+// (attention_fold: the factors a = 2^(m - m'), b = 2^(m_b - m') of the old state and of the
+// block, m' the new maximum; l' = fma(l, a, l_b b), o' = fma(o, a, o_b b)).
+// grid (tokens, heads), HD threads.  The factors depend on the blocks' maxima alone, so they are
+// worked out for HD blocks at once, thread i those of block i (the running maximum before a block
+// is the largest of the maxima before it: no rounding, any order), and only the two multiply-adds
+// a block remain a chain: thread d folds dim d, every thread folds l for itself.
 template <int HD>
 __global__ void __launch_bounds__(HD)
 attention_combine_kernel(const float* __restrict__ partial, const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ token_index, bf16_t* __restrict__ out, int max_chunks, int n_heads,
                          int window) {
+  __shared__ float block_max[HD], block_sum[HD], old_factor[HD], new_factor[HD], wave_max[HD / 64];
   const int t = token_index ? token_index[blockIdx.x] : blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
   const int first = (lo / DC_CHUNK) * DC_CHUNK;
   const int b0 = (lo - first) / ATT_BLOCK, b1 = (pos - first) / ATT_BLOCK;     // the blocks that hold seen positions
   const float* src = partial + ((size_t)blockIdx.x * n_heads + head) * (max_chunks * (DC_CHUNK / ATT_BLOCK)) * (HD + 2);
-  float m = -INFINITY, l = 0.0f, o = 0.0f;
-  int b = b0;
-  for (; b + 3 <= b1; b += 4) {       // four blocks' loads under way at a time; folded one after the other
-    float ob[4], mb[4], lb[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float* p = src + (size_t)(b + i) * (HD + 2);
-      ob[i] = p[d];
-      mb[i] = p[HD];
-      lb[i] = p[HD + 1];
+  float m = -INFINITY, l = 0.0f, o = 0.0f;     // m: the maximum of all blocks before this group
+  for (int g0 = b0; g0 <= b1; g0 += HD) {
+    const int n = min(HD, b1 - g0 + 1);        // blocks of this group
+    if (g0 > b0) __syncthreads();              // everyone has read the group before
+    if (d < n) {
+      const float* p = src + (size_t)(g0 + d) * (HD + 2);
+      block_max[d] = p[HD];
+      block_sum[d] = p[HD + 1];
     }
+    __syncthreads();
+    {
+      // the running maximum before block d: a scan over the lanes of each wave, then the waves before
+      const int lane = d & 63, wave = d >> 6;
+      const float mine = d < n ? block_max[d] : -INFINITY;
+      float upto = mine;                       // the largest of this wave's blocks up to d
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float fa, fb;
-      attention_fold(m, l, mb[i], lb[i], fa, fb);
-      o = attention_fold_value(o, fa, ob[i], fb);
+      for (int off = 1; off < 64; off <<= 1) {
+        const float other = __shfl_up(upto, off, AXON_WAVE);
+        if (lane >= off) upto = fmaxf(upto, other);
+      }
+      float before = __shfl_up(upto, 1, AXON_WAVE);
+      if (lane == 0) before = -INFINITY;
+      if (lane == 63) wave_max[wave] = upto;
+      __syncthreads();
+      before = fmaxf(before, m);
+      for (int w = 0; w < wave; ++w) before = fmaxf(before, wave_max[w]);
+      if (d < n) {
+        float fa, fb, unused = 0.0f;
+        attention_fold(before, unused, mine, 0.0f, fa, fb);
+        old_factor[d] = fa;
+        new_factor[d] = fb;
+      }
     }
-  }
-  for (; b <= b1; ++b) {
-    const float* p = src + (size_t)b * (HD + 2);
-    float fa, fb;
-    attention_fold(m, l, p[HD], p[HD + 1], fa, fb);
-    o = attention_fold_value(o, fa, p[d], fb);
+    __syncthreads();
+    int i = 0;
+    for (; i + 15 < n; i += 16) {              // sixteen blocks' values under way at a time
+      float ob[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) ob[j] = src[(size_t)(g0 + i + j) * (HD + 2) + d];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const float fa = old_factor[i + j], fb = new_factor[i + j];
+        l = __builtin_fmaf(l, fa, __fmul_rn(block_sum[i + j], fb));
+        o = attention_fold_value(o, fa, ob[j], fb);
+      }
+    }
+    for (; i < n; ++i) {
+      const float fa = old_factor[i], fb = new_factor[i];
+      l = __builtin_fmaf(l, fa, __fmul_rn(block_sum[i], fb));
+      o = attention_fold_value(o, fa, src[(size_t)(g0 + i) * (HD + 2) + d], fb);
+    }
+    for (int w = 0; w < HD / 64; ++w) m = fmaxf(m, wave_max[w]);     // blocks past n count as -inf
   }
   out[(size_t)t * n_heads * HD + (size_t)head * HD + d] = float_to_bf16(__fmul_rn(o, attention_inverse(l)));
 }
