@@ -534,20 +534,19 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
     }
   }
   wait_vmcnt<0>();                    // the stage is this wave's alone: what it loaded is what it reads
-  // weights of unwritten positions are zero, and zero times whatever a page holds must stay zero
+  // weights of unwritten positions are zero, and zero times whatever a page holds must stay zero:
+  // only the block that holds the token's own position has any (one branch for the wave), and
+  // there a word of two positions keeps both, the first or none of them
+  if (p0 + ATT_BLOCK - 1 > pos) {
 #pragma unroll
-  for (int s2 = 0; s2 < 4; ++s2) {
-    if (keep[s2] < 8) {
+    for (int s2 = 0; s2 < 4; ++s2)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        uint32_t* w = reinterpret_cast<uint32_t*>(&vf[dt][s2]);
+      for (int i = 0; i < 4; ++i) {
+        const int kept = keep[s2] - 2 * i;                          // positions of word i that were written
+        const uint32_t mask = kept >= 2 ? 0xffffffffu : kept == 1 ? 0x0000ffffu : 0u;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (keep[s2] <= 2 * i) w[i] = 0;
-          else if (keep[s2] == 2 * i + 1) w[i] &= 0xffffu;
-        }
+        for (int dt = 0; dt < DT; ++dt) reinterpret_cast<uint32_t*>(&vf[dt][s2])[i] &= mask;
       }
-    }
   }
   const bool whole = p0 + ATT_BLOCK - 1 <= pos && p0 >= lo;
   float m_b, l_b;
