@@ -47,7 +47,7 @@ def parse_ids(text: str) -> List[int]:
 def _engine_flags(p: argparse.ArgumentParser) -> None:
     p.add_argument("--dtype", default="bfloat16", help="bfloat16 (default) or float32: true 32-bit everywhere")
     p.add_argument("--ctx", type=int, default=0, help="positions a request may reach (default: the model's)")
-    p.add_argument("--page-size", type=int, default=16, help="positions in one cache page (default 16)")
+    p.add_argument("--page-size", type=int, default=64, help="positions in one cache page (default 64: a block of the attention kernels)")
     p.add_argument("--num-pages", type=int, default=0, help="pages in the cache pool (default: what the request needs)")
     p.add_argument("--device", default="cuda:0", help="the GPU to run on (default cuda:0)")
     p.add_argument("--verbose", action="store_true", help="print what was loaded and the settings in use")

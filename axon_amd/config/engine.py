@@ -25,7 +25,7 @@ class EngineConfig:
     `max_seq_len`: positions a request may reach (0: the model's max_position_embeddings).
     `use_graphs`: replay pure decode steps from captured HIP graphs."""
     dtype: str = "bfloat16"
-    page_size: int = 16
+    page_size: int = 64
     num_pages: int = 0
     max_cache_tokens: int = 0
     memory_fraction: float = 0.85

@@ -101,7 +101,8 @@ __device__ __forceinline__ void att_issue_k(unsigned char* stage, int instr, int
   const int row = instr * S::K_ROWS_PER_INSTR + lane / S::KCH;
   const int chunk = (lane % S::KCH) ^ (row & 7);
   const int p = min(p0 + row, hi);
-  const bf16_t* src = k_head + (size_t)page * page_stride + (size_t)page_offset(p, page_size) * HD + chunk * 8;
+  const bf16_t* base = k_head + (size_t)page * page_stride;          // scalar arithmetic where the page is the wave's
+  const bf16_t* src = base + (unsigned)(page_offset(p, page_size) * HD + chunk * 8);
   __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + instr * 1024), 16, 0, 0);
 }
 
@@ -114,7 +115,8 @@ __device__ __forceinline__ void att_issue_v(unsigned char* stage, int instr, int
   const int d = instr * 8 + (lane >> 3);
   const int chunk = (lane & 7) ^ (d & 7);
   const int p = min(p0 + chunk * 8, hi);
-  const bf16_t* src = v_head + (size_t)page * page_stride + (size_t)d * page_size + (page_offset(p, page_size) & ~7);
+  const bf16_t* base = v_head + (size_t)page * page_stride;
+  const bf16_t* src = base + (unsigned)(d * page_size + (page_offset(p, page_size) & ~7));
   __builtin_amdgcn_global_load_lds((global_ptr_t)src, (lds_ptr_t)(stage + S::K_BYTES + instr * 1024), 16, 0, 0);
 }
 
@@ -185,24 +187,22 @@ __device__ __forceinline__ void attention_scores(unsigned st, const bf16x8 (&qf)
 
   // the largest raw score first (the scale is positive), then exp2(score * c - max * c) in one
   // multiply-add each
-  float mloc = -INFINITY;
-  if (whole) {
-#pragma unroll
-    for (int pt = 0; pt < 2; ++pt)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) mloc = fmaxf(mloc, s_acc[pt][e]);
-  } else {
+  if (!whole) {
+    asm volatile("" ::: "memory");      // a branch of its own: the blocks every column sees whole pay nothing for the mask
 #pragma unroll
     for (int pt = 0; pt < 2; ++pt)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int p = p0 + pt * 32 + (e >> 3) * 16 + half * 8 + (e & 7);
         const bool seen = p <= my_pos && p >= my_lo;
-        const float v = seen ? s_acc[pt][e] : -INFINITY;
-        s_acc[pt][e] = v;
-        mloc = fmaxf(mloc, v);
+        s_acc[pt][e] = seen ? s_acc[pt][e] : -INFINITY;
       }
   }
+  float mloc = -INFINITY;
+#pragma unroll
+  for (int pt = 0; pt < 2; ++pt)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) mloc = fmaxf(mloc, s_acc[pt][e]);
   mloc = fmaxf(mloc, __shfl_xor(mloc, 32, AXON_WAVE));
   m_b = __fmul_rn(mloc, c);
   const float mref = m_b == -INFINITY ? 0.0f : m_b;     // a column that sees nothing of this block
@@ -289,8 +289,14 @@ __device__ __forceinline__ void attention_fold(float& m, float& l, float m_b, fl
   m = mn;
 }
 
+// fma(o, a, o_b b), written as the three-address instruction: left to itself the compiler takes the
+// two-address form, whose result lands in the product's register, and moves every value back
+// into the loop's own register afterwards (64 moves a block of positions).
 __device__ __forceinline__ float attention_fold_value(float o, float a, float o_b, float b) {
-  return __builtin_fmaf(o, a, __fmul_rn(o_b, b));
+  const float t = __fmul_rn(o_b, b);
+  float r;
+  asm("v_fma_f32 %0, %1, %2, %3" : "=v"(r) : "v"(o), "v"(a), "v"(t));
+  return r;
 }
 
 __device__ __forceinline__ float attention_inverse(float l) { return __fdiv_rn(1.0f, l); }
@@ -303,7 +309,7 @@ __device__ __forceinline__ float attention_inverse(float l) { return __fdiv_rn(1
 // loads are in flight while this one is multiplied.
 #define PF_TOKENS 128
 
-template <int HD, int HPB>
+template <int HD, int HPB, bool ONE_PAGE>
 __device__ __forceinline__ void
 attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __restrict__ q, int q_stride,
                        const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -318,7 +324,8 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
   constexpr int DT = HD / 32;                     // output tiles (32 dims each)
   constexpr int KS = HD / 16;                     // k steps of S^T
 
-  const int tid = threadIdx.x, lane = tid & 63, block_wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int block_wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // a scalar: what depends on it alone branches, not masks
   const int wave = block_wave & 3;                 // which 32 query rows of the tile
   const int group = n_heads / n_kv_heads, sets = (group + HPB - 1) / HPB;   // sets of HPB query heads per kv head
   const int kvh = blockIdx.y / sets;
@@ -353,9 +360,15 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
   const bf16_t* v_head = v_cache + (size_t)kvh * HD * page_size;
   // The pages a block of positions lies in are looked up one block ahead of the loads that use
   // them, so that no load waits for a table entry behind the loads issued just before it.
+  // ONE_PAGE (pages of 64 positions or more): a block lies in one page, known to the whole wave,
+  // and the addresses are a scalar base plus a lane's 32-bit offset.
   int k_page[K_INSTR], v_page[V_INSTR];
   auto lookup = [&](int b) {
     const int p0 = first_block + b * ATT_BLOCK;
+    if (ONE_PAGE) {
+      k_page[0] = table_row[page_index(p0, page_size)];
+      return;
+    }
 #pragma unroll
     for (int n = 0; n < K_INSTR; ++n) k_page[n] = att_k_page<HD>(n * NW + block_wave, lane, p0, hi, table_row, page_size);
 #pragma unroll
@@ -366,10 +379,12 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
     const int p0 = first_block + b * ATT_BLOCK;
 #pragma unroll
     for (int n = 0; n < K_INSTR; ++n)
-      att_issue_k<HD>(stage, n * NW + block_wave, lane, k_page[n], p0, hi, k_head, page_stride, page_size);
+      att_issue_k<HD>(stage, n * NW + block_wave, lane, ONE_PAGE ? k_page[0] : k_page[n], p0, hi, k_head, page_stride,
+                      page_size);
 #pragma unroll
     for (int n = 0; n < V_INSTR; ++n)
-      att_issue_v<HD>(stage, n * NW + block_wave, lane, v_page[n], p0, hi, v_head, page_stride, page_size);
+      att_issue_v<HD>(stage, n * NW + block_wave, lane, ONE_PAGE ? k_page[0] : v_page[n], p0, hi, v_head, page_stride,
+                      page_size);
   };
 
   f32x16 o_acc[DT];
@@ -444,8 +459,12 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_
     const int t0 = mine[2 * part], count = mine[2 * part + 1];
     if (count <= 0) break;                        // the same for the whole block
     if (part) __syncthreads();                    // everyone has read the first tile's last stage
-    attention_prefill_tile<HD, HPB>(smem, t0, count, q, q_stride, k_cache, v_cache, block_table, table_stride, positions,
-                                    seq_rows, out, n_heads, n_kv_heads, page_size, window, scale);
+    if (page_size >= ATT_BLOCK)
+      attention_prefill_tile<HD, HPB, true>(smem, t0, count, q, q_stride, k_cache, v_cache, block_table, table_stride,
+                                            positions, seq_rows, out, n_heads, n_kv_heads, page_size, window, scale);
+    else
+      attention_prefill_tile<HD, HPB, false>(smem, t0, count, q, q_stride, k_cache, v_cache, block_table, table_stride,
+                                             positions, seq_rows, out, n_heads, n_kv_heads, page_size, window, scale);
   }
 }
 
@@ -475,7 +494,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
   extern __shared__ __align__(16) unsigned char smem[];
   static_assert(DC_CHUNK / ATT_BLOCK == 4 && (BW == 1 || BW == 4), "four blocks of positions a chunk");
   const int lane = threadIdx.x & 63;
-  const int wave = BW == 1 ? blockIdx.x & 3 : threadIdx.x >> 6;       // which 64 positions of the chunk
+  const int wave = BW == 1 ? blockIdx.x & 3 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // which 64 positions of the chunk (a scalar)
   const int unit = BW == 1 ? blockIdx.x >> 2 : blockIdx.x;
   const int item = work[unit / n_kv_heads];          // the kv heads of a chunk side by side: they share its pages
   if (item < 0) return;                              // padding of the list
@@ -501,25 +520,42 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t
   // the lane's positions p0 + 8 c .. + 7, c = 4 (s2 / 2) + 2 (s2 % 2) + half, of dim 32 dt + l32:
   // 16 bytes of one page (a page holds a multiple of 8 positions); the two halves of a wave read
   // neighbouring chunks, so an instruction reads whole rows of a page of 16 positions.
-  int k_page[S::K_INSTR], v_page[4], v_at[4], keep[4];
-#pragma unroll
-  for (int n = 0; n < S::K_INSTR; ++n) k_page[n] = att_k_page<HD>(n, lane, p0, pos, table_row, page_size);
-#pragma unroll
-  for (int s2 = 0; s2 < 4; ++s2) {
-    const int pa = p0 + 8 * (4 * (s2 >> 1) + 2 * (s2 & 1) + half);
-    keep[s2] = max(0, min(pos - pa + 1, 8));          // positions past the token were never written
-    const int pa_c = min(pa, pos);
-    v_page[s2] = table_row[page_index(pa_c, page_size)];
-    v_at[s2] = page_offset(pa_c, page_size) & ~7;
-  }
-#pragma unroll
-  for (int n = 0; n < S::K_INSTR; ++n) att_issue_k<HD>(stage, n, lane, k_page[n], p0, pos, k_head, page_stride, page_size);
+  int keep[4];
   uint4 vf[DT][4];
 #pragma unroll
-  for (int s2 = 0; s2 < 4; ++s2) {
-    const bf16_t* va = v_head + (size_t)v_page[s2] * page_stride + v_at[s2];
+  for (int s2 = 0; s2 < 4; ++s2) keep[s2] = max(0, min(pos - (p0 + 8 * (4 * (s2 >> 1) + 2 * (s2 & 1) + half)) + 1, 8));
+  if (page_size >= ATT_BLOCK) {
+    // the block lies in one page, known to the whole wave: a scalar base and 32-bit offsets
+    const int page = table_row[page_index(p0, page_size)];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) vf[dt][s2] = *reinterpret_cast<const uint4*>(va + (size_t)(dt * 32 + l32) * page_size);
+    for (int n = 0; n < S::K_INSTR; ++n) att_issue_k<HD>(stage, n, lane, page, p0, pos, k_head, page_stride, page_size);
+    const bf16_t* base = v_head + (size_t)page * page_stride;
+#pragma unroll
+    for (int s2 = 0; s2 < 4; ++s2) {
+      const int pa_c = min(p0 + 8 * (4 * (s2 >> 1) + 2 * (s2 & 1) + half), pos);
+      const unsigned at = page_offset(pa_c, page_size) & ~7;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        vf[dt][s2] = *reinterpret_cast<const uint4*>(base + (unsigned)((dt * 32 + l32) * page_size + at));
+    }
+  } else {
+    int k_page[S::K_INSTR], v_page[4], v_at[4];
+#pragma unroll
+    for (int n = 0; n < S::K_INSTR; ++n) k_page[n] = att_k_page<HD>(n, lane, p0, pos, table_row, page_size);
+#pragma unroll
+    for (int s2 = 0; s2 < 4; ++s2) {
+      const int pa_c = min(p0 + 8 * (4 * (s2 >> 1) + 2 * (s2 & 1) + half), pos);   // positions past the token were never written
+      v_page[s2] = table_row[page_index(pa_c, page_size)];
+      v_at[s2] = page_offset(pa_c, page_size) & ~7;
+    }
+#pragma unroll
+    for (int n = 0; n < S::K_INSTR; ++n) att_issue_k<HD>(stage, n, lane, k_page[n], p0, pos, k_head, page_stride, page_size);
+#pragma unroll
+    for (int s2 = 0; s2 < 4; ++s2) {
+      const bf16_t* va = v_head + (size_t)v_page[s2] * page_stride + v_at[s2];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vf[dt][s2] = *reinterpret_cast<const uint4*>(va + (size_t)(dt * 32 + l32) * page_size);
+    }
   }
 
   // Q^T (B operand): column = head of the group (zero beyond it), 8 consecutive dims from 16 ks + 8 half
@@ -654,7 +690,7 @@ attention_combine_kernel(const float* __restrict__ partial, const int32_t* __res
 extern "C" int axk_attention_fast_ok(int head_dim, int page_size, int n_heads, int n_kv_heads) {
 #if AXON_BF16
   const bool hd_ok = head_dim == 64 || head_dim == 128;
-  const bool page_ok = page_size >= 8 && page_size <= 64 && (page_size & (page_size - 1)) == 0;
+  const bool page_ok = page_size >= 8 && page_size <= 1024 && (page_size & (page_size - 1)) == 0;
   return hd_ok && page_ok && n_kv_heads > 0 && n_heads % n_kv_heads == 0 && n_heads / n_kv_heads <= 32;
 #else
   return 0;

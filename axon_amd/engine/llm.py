@@ -273,7 +273,7 @@ class LLM:
 
 
 def load(model: Union[str, dict, ModelConfig], dtype: str = "bfloat16", *, random_seed: Optional[int] = None,
-         init_std: float = 0.02, device: str = "cuda:0", page_size: int = 16, num_pages: int = 0,
+         init_std: float = 0.02, device: str = "cuda:0", page_size: int = 64, num_pages: int = 0,
          max_cache_tokens: int = 0, memory_fraction: float = 0.85, max_seqs: int = 64, max_batch_tokens: int = 2048,
          max_seq_len: int = 0, use_graphs: bool = True) -> LLM:
     """A model folder (config.json + safetensors), or a configuration (a dict of config.json

@@ -81,7 +81,7 @@ def main() -> int:
         cfg["num_hidden_layers"] = args.layers
     L, dim, ffn, V = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
-    ctx_len, page = cfg["max_position_embeddings"], 16
+    ctx_len, page = cfg["max_position_embeddings"], 64
     elem = 2 if args.dtype == "bfloat16" else 4
     points_on = not args.no_points and args.phase == "all"
     most_batch = max(args.batch, 64) if points_on else max(args.batch, 36 if args.phase == "mixed" else 1)

@@ -36,7 +36,7 @@ TINY = {
                           intermediate_size=320, num_attention_heads=6, num_key_value_heads=2, head_dim=64,
                           vocab_size=300, max_position_embeddings=1024, rope_theta=10000.0, rms_norm_eps=1e-6,
                           tie_word_embeddings=True),
-              std=0.05, page_size=16, seed=7),
+              std=0.05, page_size=64, seed=7),
     "E": dict(config=dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=2, hidden_size=256,
                           intermediate_size=384, num_attention_heads=7, num_key_value_heads=1, head_dim=128,
                           vocab_size=401, max_position_embeddings=2048, rope_theta=1000000.0, rms_norm_eps=1e-5,

@@ -424,7 +424,8 @@ def _mfma_case(nh, nkv, hd, page, T, window, seed=0, scale_q=1.0):
 
 @pytest.mark.parametrize("nh,nkv,hd,page,T,window", [
     (4, 2, 64, 16, 300, 0), (7, 1, 128, 16, 257, 0), (6, 2, 128, 8, 130, 0), (2, 2, 64, 64, 200, 0),
-    (8, 2, 128, 32, 333, 0), (4, 1, 64, 16, 400, 100), (14, 2, 128, 16, 129, 37), (16, 1, 64, 8, 70, 0)])
+    (8, 2, 128, 32, 333, 0), (4, 1, 64, 16, 400, 100), (14, 2, 128, 16, 129, 37), (16, 1, 64, 8, 70, 0),
+    (7, 1, 128, 64, 300, 0), (4, 2, 128, 128, 333, 90), (6, 3, 64, 256, 290, 0)])
 def test_prompt_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
     k = kernels("bfloat16")
     assert k.attention_fast_ok(hd, page, nh, nkv)
@@ -464,7 +465,8 @@ def test_prompt_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
 
 @pytest.mark.parametrize("nh,nkv,hd,page,T,window", [
     (4, 2, 64, 16, 300, 0), (7, 1, 128, 16, 1030, 0), (28, 4, 128, 16, 600, 0), (6, 2, 128, 8, 255, 0),
-    (2, 2, 64, 64, 257, 0), (16, 1, 64, 32, 513, 0), (4, 1, 64, 16, 900, 300), (5, 5, 128, 16, 64, 0), (3, 1, 128, 16, 700, 70), (4, 1, 128, 16, 4100, 0), (2, 1, 64, 32, 3000, 1000)])
+    (2, 2, 64, 64, 257, 0), (16, 1, 64, 32, 513, 0), (4, 1, 64, 16, 900, 300), (5, 5, 128, 16, 64, 0), (3, 1, 128, 16, 700, 70), (4, 1, 128, 16, 4100, 0), (2, 1, 64, 32, 3000, 1000),
+    (28, 4, 128, 64, 600, 0), (4, 1, 128, 128, 700, 200), (6, 2, 64, 256, 1000, 0)])
 def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
     k = kernels("bfloat16")
     q, kc, vc, table, ref = _mfma_case(nh, nkv, hd, page, T, window, seed=5)
@@ -511,7 +513,7 @@ def test_decoding_attention_on_the_matrix_cores(nh, nkv, hd, page, T, window):
 
 @pytest.mark.parametrize("nh,nkv,hd,page,T,window", [
     (28, 4, 128, 16, 700, 0), (40, 8, 128, 16, 300, 0), (4, 2, 64, 8, 333, 0), (6, 1, 128, 64, 600, 150),
-    (32, 1, 64, 16, 200, 0), (3, 3, 128, 32, 1100, 0)])
+    (32, 1, 64, 16, 200, 0), (3, 3, 128, 32, 1100, 0), (7, 1, 128, 128, 500, 0), (4, 2, 64, 64, 330, 100)])
 def test_a_position_gets_the_same_bits_from_the_prompt_kernel_and_the_decoding_kernel(nh, nkv, hd, page, T, window):
     """Every position of a sequence once as a row of a prompt portion (tiles cut at several places)
     and once as a single decoding token: bit for bit the same result, whatever the cut, because
@@ -537,6 +539,31 @@ def test_a_position_gets_the_same_bits_from_the_prompt_kernel_and_the_decoding_k
         k.attention_prefill(q, nh * hd, kc, vc, table, pos, rows, prompt, torch.tensor(tiles, dtype=torch.int32).cuda(),
                             nh, nkv, hd, page, window, scale)
         assert torch.equal(prompt, decoded), cuts
+
+
+@pytest.mark.parametrize("nh,nkv,hd,T,window", [(7, 1, 128, 450, 0), (4, 2, 64, 300, 0), (6, 2, 128, 333, 120)])
+def test_the_page_size_does_not_change_a_bit_of_the_attention(nh, nkv, hd, T, window):
+    """Pages of 64 positions or more hold a whole block of the kernels, which then take the page
+    from one table entry for the wave; smaller pages are looked up lane by lane.  Both read the
+    same keys and values, so the results are the same bits, from both kernels."""
+    k = kernels("bfloat16")
+    scale = 1.0 / math.sqrt(hd)
+    pos = torch.arange(T, dtype=torch.int32).cuda()
+    rows = torch.zeros(T, dtype=torch.int32).cuda()
+    ch = k.attention_decode_chunk
+    chunks = max((p - ((max(0, p + 1 - window) if window else 0) // ch * ch)) // ch + 1 for p in range(T))
+    tiles = torch.tensor([(a, min(128, T - a)) for a in range(0, T, 128)], dtype=torch.int32).cuda()
+    results = []
+    for page in (8, 16, 64, 128):
+        q, kc, vc, table, ref = _mfma_case(nh, nkv, hd, page, T, window, seed=21)
+        prompt = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+        k.attention_prefill(q, nh * hd, kc, vc, table, pos, rows, prompt, tiles, nh, nkv, hd, page, window, scale)
+        partial = torch.empty(k.attention_decode_workspace(T, nh, hd, chunks), dtype=torch.float32, device="cuda")
+        decoded = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
+        k.attention_decode(q, nh * hd, kc, vc, table, pos, rows, decoded, T, partial, chunks, nh, nkv, hd, page, window, scale)
+        assert not torch.isnan(prompt).any() and torch.equal(prompt, decoded), page
+        results.append(prompt)
+    assert all(torch.equal(results[0], r) for r in results[1:])
 
 
 def test_matrix_core_attention_finds_a_far_key_and_respects_the_windows_edge():
