@@ -138,6 +138,20 @@ int axk_gemm_qkv_rope(const void* x, int x_stride, const void* w, const void* bi
                       void* v_cache, int n_heads, int n_kv_heads, int head_dim, int page_size, int write_kv,
                       void* workspace, long workspace_bytes, void* stream);
 
+// Few rows (a decoding step), bfloat16 build: the gated product (out = silu(X Wg^T) * (X Wu^T), W
+// the packed [gate; up] matrix) and the [q; k; v] product (as axk_gemm_qkv_rope) with the RMS norm
+// of their operand inside: X = axk_rmsnorm(rows, gain, eps) is worked out in the kernel's own LDS
+// and never stored.  Bit-identical to axk_rmsnorm followed by axk_gemm / axk_gemm_qkv_rope.
+// axk_gemm_normed_ok(m, n, k, gated): whether these sizes are taken (up to 8 rows, X within LDS).
+int axk_gemm_normed_ok(int m, int n, int k, int gated);
+int axk_gemm_normed_glu(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps, const void* w,
+                        void* out, int out_stride, int m, int n, int k, void* stream);
+int axk_gemm_normed_qkv_rope(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps,
+                             const void* w, const void* bias, int bias_is_f32, void* qkv, int qkv_stride, int m, int k,
+                             const float* table, const int32_t* positions, const int32_t* seq_rows,
+                             const int32_t* block_table, int table_stride, void* k_cache, void* v_cache, int n_heads,
+                             int n_kv_heads, int head_dim, int page_size, int write_kv, void* stream);
+
 // out[t, f] = silu(gu[t, f]) * gu[t, F + f]: gate in the first F columns, up in the last.
 int axk_swiglu(const void* gate_up, void* out, int n_tokens, int n_ffn, void* stream);
 

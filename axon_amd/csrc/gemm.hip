@@ -157,6 +157,14 @@ int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const v
                          const int32_t* seq_rows, const int32_t* block_table, int table_stride, bf16_t* k_cache,
                          bf16_t* v_cache, int n_heads, int n_kv_heads, int head_dim, int page_size, void* workspace,
                          size_t workspace_bytes, hipStream_t stream);
+int gemm_normed_ok(int m, int k);
+int launch_gemm_normed_glu(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps, const bf16_t* w,
+                           bf16_t* out, int out_stride, int m, int n, int k, hipStream_t stream);
+int launch_gemm_normed_qkv_rope(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps,
+                                const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out, int out_stride, int m, int n,
+                                int k, const float* table, const int32_t* positions, const int32_t* seq_rows,
+                                const int32_t* block_table, int table_stride, bf16_t* k_cache, bf16_t* v_cache, int n_heads,
+                                int n_kv_heads, int head_dim, int page_size, hipStream_t stream);
 #endif
 
 static int gemm_checked(const void* x, int x_stride, const void* w, int w_packed, const void* bias, int bias_is_f32,
@@ -284,6 +292,64 @@ extern "C" int axk_gemm_qkv_rope(const void* x, int x_stride, const void* w, con
                               workspace_bytes > 0 ? (size_t)workspace_bytes : 0, (hipStream_t)stream);
 #else
   axk_set_error("gemm_qkv_rope: only in the bfloat16 build");
+  return -1;
+#endif
+}
+
+// ---------------------------------------------------------------------------- the norm inside the product
+// Few rows (a decoding step): the gated product and the [q; k; v] product read the float32 rows
+// themselves and apply the RMS norm on the way (the norm kernel's arithmetic, the same bits), so
+// the norm is no launch of its own.  `ok` depends on the sizes alone.
+extern "C" int axk_gemm_normed_ok(int m, int n, int k, int gated) {
+#if AXON_BF16
+  if (m <= 0 || n <= 0 || k <= 0 || !gemm_pack_ok(gated ? 2 * n : n, k, gated)) return 0;
+  return gemm_normed_ok(m, k);
+#else
+  return 0;   // the 32-bit build keeps the norm a pass of its own
+#endif
+}
+
+extern "C" int axk_gemm_normed_glu(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps,
+                                   const void* w, void* out, int out_stride, int m, int n, int k, void* stream) {
+#if AXON_BF16
+  AXK_REQUIRE(axk_gemm_normed_ok(m, n, k, 1), "gemm_normed_glu: M=%d N=%d K=%d are not taken", m, n, k);
+  AXK_REQUIRE(rows && gain && w && out, "gemm_normed_glu: an operand is missing");
+  AXK_REQUIRE(rows_stride >= k && rows_stride % 4 == 0 && out_stride >= n && ((uintptr_t)rows & 15) == 0 &&
+                  ((uintptr_t)gain & 15) == 0 && ((uintptr_t)w & 15) == 0,
+              "gemm_normed_glu: strides rows=%d out=%d or the alignment of an operand are not taken", rows_stride, out_stride);
+  return launch_gemm_normed_glu(rows, rows_stride, gain, gain_is_f32, eps, (const bf16_t*)w, (bf16_t*)out, out_stride, m, n, k,
+                                (hipStream_t)stream);
+#else
+  axk_set_error("gemm_normed_glu: only in the bfloat16 build");
+  return -1;
+#endif
+}
+
+extern "C" int axk_gemm_normed_qkv_rope(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps,
+                                        const void* w, const void* bias, int bias_is_f32, void* qkv, int qkv_stride, int m,
+                                        int k, const float* table, const int32_t* positions, const int32_t* seq_rows,
+                                        const int32_t* block_table, int table_stride, void* k_cache, void* v_cache,
+                                        int n_heads, int n_kv_heads, int head_dim, int page_size, int write_kv, void* stream) {
+#if AXON_BF16
+  AXK_REQUIRE(n_heads > 0 && n_kv_heads > 0 && page_size > 0 && head_dim > 0,
+              "gemm_normed_qkv_rope: heads %d/%d of %d, page %d", n_heads, n_kv_heads, head_dim, page_size);
+  const int n = (n_heads + (write_kv ? 2 * n_kv_heads : 0)) * head_dim;
+  AXK_REQUIRE(axk_gemm_normed_ok(m, n, k, 0) && axk_gemm_qkv_rope_ok(m, n, k, head_dim, head_dim),
+              "gemm_normed_qkv_rope: M=%d N=%d K=%d head_dim=%d are not taken", m, n, k, head_dim);
+  AXK_REQUIRE(rows && gain && w && qkv, "gemm_normed_qkv_rope: an operand is missing");
+  AXK_REQUIRE(rows_stride >= k && rows_stride % 4 == 0 && qkv_stride >= n_heads * head_dim && qkv_stride % 4 == 0 &&
+                  ((uintptr_t)rows & 15) == 0 && ((uintptr_t)gain & 15) == 0 && ((uintptr_t)w & 15) == 0 &&
+                  ((uintptr_t)qkv & 7) == 0 && ((uintptr_t)table & 15) == 0,
+              "gemm_normed_qkv_rope: strides rows=%d qkv=%d or the alignment of an operand are not taken", rows_stride,
+              qkv_stride);
+  AXK_REQUIRE(table && positions && (!write_kv || (seq_rows && block_table && k_cache && v_cache)),
+              "gemm_normed_qkv_rope: a table, the positions or the cache is missing");
+  return launch_gemm_normed_qkv_rope(rows, rows_stride, gain, gain_is_f32, eps, (const bf16_t*)w, bias, bias_is_f32,
+                                     (bf16_t*)qkv, qkv_stride, m, n, k, table, positions, seq_rows, block_table, table_stride,
+                                     (bf16_t*)k_cache, (bf16_t*)v_cache, n_heads, n_kv_heads, head_dim, page_size,
+                                     (hipStream_t)stream);
+#else
+  axk_set_error("gemm_normed_qkv_rope: only in the bfloat16 build");
   return -1;
 #endif
 }

@@ -938,6 +938,331 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
                                        ahead);
 }
 
+// ---------------------------------------------------------------------------- gemm_normed
+// The product of few rows with the RMS norm before it inside: X never exists in memory.  A block
+// has waves of two kinds.  NORMED_NORM_WAVES waves read the float32 rows, norm them and leave
+// X = bf16((row * inv) * gain) in LDS, in the blocks of MPAD rows x 32 k that one LDS read of a
+// wave takes as an MFMA operand.  The others stream W as gemm_stream does (G groups of tiles times
+// the S segments of K, a wave each; every block needs all of X, so G is such that each CU has
+// about one block): their ring of loads is filled while the rows are normed (as soon as the
+// rows themselves have arrived), and they start to multiply when X is there.  The norm is the norm kernel's, bit for bit: a wave takes a row, lane
+// l stands for that kernel's threads l, 64 + l, 128 + l and 192 + l (four chains over the float4
+// l + 64 j, j = v, v + 4, ...), the four butterflies are added in order.  Takes the norm's launch
+// out of a decoding step.
+struct NormedRows {
+  const float* rows;       // [M, K], rows_stride apart
+  int rows_stride;
+  const void* gain;        // [K]
+  int gain_is_f32;
+  float eps;
+};
+
+#define NORMED_MAX_LDS (152 * 1024)
+#define NORMED_STREAM_WAVES 4   // at most
+#define NORMED_NORM_WAVES 4
+#define NORMED_KC 16            // float4 of a row a lane holds: K <= 256 * 16
+
+// UNITS: pairs of row tiles a streaming wave
+#define NORMED_MAX_M 8          // with more rows the norm takes longer than it saves (measured)
+
+template <int UNITS, int SEGS, int DEPTH, int EPI>
+__global__ void __launch_bounds__((NORMED_STREAM_WAVES + NORMED_NORM_WAVES) * 64, 1)
+gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __restrict__ bias, int bias_is_f32,
+                   void* __restrict__ out, int out_stride, int M, int N, int K, int mode, RopeStore rope, int n_units) {
+  constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE;
+  constexpr int MPAD = NORMED_MAX_M;
+  constexpr int NT = 2 * UNITS, XBLOCK = MPAD * 64, KC = NORMED_KC;   // XBLOCK: bytes of MPAD rows x 32 k of X
+  static_assert(GLU || ROPE, "the paired epilogues");
+  static_assert(!ROPE || UNITS == 1, "one head half-pair a wave");
+  static_assert(MPAD == 8, "rows of X in LDS: half a tile of 16, lanes of rows 8 .. 15 read rows 0 .. 7 again");
+  extern __shared__ __align__(16) unsigned char x_lds[];        // X, then the segments' sums [wave][tile][lane][4]
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nw = (blockDim.x >> 6) - NORMED_NORM_WAVES;         // streaming waves
+  const int KB = K / 32;
+
+  if (wave >= nw) {
+    // ------------------------------------------------------------------ a norming wave: rows w, w + 4, ..., two at a time
+    // A row is n4 float4: `full` rounds of the 64 lanes and `tail` lanes more; lane l holds the
+    // float4 l + 64 j.  In LDS that is block (l >> 3) + 8 j of X, chunk (l & 7) >> 1, half l & 1:
+    // one address a lane and row, 8 blocks further for every j.
+    const int n4 = K / 4, full = n4 >> 6, tail = n4 & 63, first_row = wave - nw;
+    int ln = lane;
+    asm volatile("" : "+v"(ln));        // what follows from the lane is worked out here, not kept in registers from the start
+    const bool in_tail = ln < tail;
+    uint2 gain_bf[KC];                                          // a bfloat16 gain: the lane's share, asked for with the rows
+    if (!in.gain_is_f32 && first_row < M) {
+#pragma unroll
+      for (int j = 0; j < KC; ++j)
+        if (j < full || (j == full && in_tail))
+          gain_bf[j] = *reinterpret_cast<const uint2*>((const bf16_t*)in.gain + 4 * (ln + 64 * j));
+    }
+    const int q = (ln & 7) >> 1;
+    const unsigned swz = (q + 4 * ((ln >> 3) & 1)) & 7;           // slots of 16 bytes (a row's 8 k) are permuted within
+    unsigned char* at0 = x_lds + (ln >> 3) * XBLOCK + (ln & 1) * 8;   // eights, by chunk and block parity: these stores,
+                                                                  // which walk along a row, spread over the banks
+    if (first_row >= M) __syncthreads();                        // a wave without rows: the barrier of those with
+    for (int m0 = first_row; m0 < M; m0 += 2 * NORMED_NORM_WAVES) {
+      const int m1 = m0 + NORMED_NORM_WAVES;
+      float4 kept[2][KC];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int m = min(r ? m1 : m0, M - 1);                   // no second row: the first again, not stored
+        const float4* row = reinterpret_cast<const float4*>(in.rows + (size_t)m * in.rows_stride) + ln;
+#pragma unroll
+        for (int j = 0; j < KC; ++j) {
+          if (j < full) kept[r][j] = row[64 * j];                // the same for every lane: a branch, no mask
+          else {
+            kept[r][j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (j == full && in_tail) kept[r][j] = row[64 * j];
+          }
+        }
+      }
+      // four chains a row as the norm kernel's four waves have them, then their butterflies, all
+      // eight side by side (a step of a butterfly is a round trip through the LDS crossbar)
+      float ss[2][4];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) ss[r][v] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < KC; ++j) {
+          const float4 x = kept[r][j];
+          ss[r][j & 3] = fmaf(x.x, x.x, ss[r][j & 3]);
+          ss[r][j & 3] = fmaf(x.y, x.y, ss[r][j & 3]);
+          ss[r][j & 3] = fmaf(x.z, x.z, ss[r][j & 3]);
+          ss[r][j & 3] = fmaf(x.w, x.w, ss[r][j & 3]);
+        }
+      }
+      if (m0 == first_row) {
+        asm volatile("" :: "v"(ss[0][0]), "v"(ss[1][0]), "v"(ss[0][3]), "v"(ss[1][3]));   // the sums, so the rows, are here
+        __syncthreads();                 // ... and only now do the streaming waves ask for all their W
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        float other[2][4];
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) other[r][v] = __shfl_xor(ss[r][v], off, AXON_WAVE);
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) ss[r][v] += other[r][v];
+      }
+      float inv[2];
+      unsigned char* at[2];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const float total = ((ss[r][0] + ss[r][1]) + ss[r][2]) + ss[r][3];
+        inv[r] = 1.0f / sqrtf(total / (float)K + in.eps);
+        at[r] = at0 + (((unsigned)(r ? m1 : m0) + MPAD * q) ^ swz) * 16;
+      }
+      const bool second = m1 < M;
+      // a chunk of the gain at a time, for both rows
+#pragma unroll
+      for (int j = 0; j < KC; ++j) {
+        if (!(j < full || (j == full && in_tail))) continue;     // (for j != full the same for every lane)
+        float4 gn;
+        if (in.gain_is_f32) gn = *reinterpret_cast<const float4*>((const float*)in.gain + 4 * (ln + 64 * j));
+        else {
+          const uint2 gb = gain_bf[j];
+          gn = make_float4(__uint_as_float(gb.x << 16), __uint_as_float(gb.x & 0xffff0000u), __uint_as_float(gb.y << 16),
+                           __uint_as_float(gb.y & 0xffff0000u));
+        }
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          if (r && !second) continue;
+          const float4 x = kept[r][j];
+          uint2 pk;
+          pk.x = pack2_bf16((x.x * inv[r]) * gn.x, (x.y * inv[r]) * gn.y);
+          pk.y = pack2_bf16((x.z * inv[r]) * gn.z, (x.w * inv[r]) * gn.w);
+          *reinterpret_cast<uint2*>(at[r] + j * 8 * XBLOCK) = pk;
+        }
+      }
+    }
+    __syncthreads();                     // X is there
+    if (SEGS > 1) __syncthreads();       // (the streaming waves exchange their sums)
+    return;
+  }
+
+  // -------------------------------------------------------------------- a streaming wave
+  const int seg = wave % SEGS, g = wave / SEGS, groups = nw / SEGS;
+  const int r16 = lane & 15;
+  float* partial = reinterpret_cast<float*>(x_lds + (size_t)KB * XBLOCK);
+  int unit[UNITS];
+  bool live[UNITS];
+  const bf16_t* wtile[NT];
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u) {
+    const int at = ((int)blockIdx.x * groups + g) * UNITS + u;
+    live[u] = at < n_units;
+    unit[u] = min(at, n_units - 1);                             // past the last: the last again, nothing stored
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      int tile;
+      if (GLU) tile = i * (N / 16) + unit[u];                    // gate rows, then the up rows of the same columns
+      else {
+        const int half = rope.head_dim / 2, per_head = half / 16;
+        tile = ((unit[u] / per_head) * rope.head_dim + i * half) / 16 + unit[u] % per_head;
+      }
+      wtile[u * 2 + i] = w + (size_t)tile * KB * 512 + lane * 8;
+    }
+  }
+  f32x4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  const int nk = K / 64;
+  const int first = (int)((long)seg * nk / SEGS);
+  const int mine = (int)((long)(seg + 1) * nk / SEGS) - first;
+  uint4 wf[DEPTH][NT][2];
+  auto load = [&](int slot, int local) {
+    const int k0 = (first + local) * 64;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      wf[slot][t][0] = *reinterpret_cast<const uint4*>(wtile[t] + k0 * 16);
+      wf[slot][t][1] = *reinterpret_cast<const uint4*>(wtile[t] + k0 * 16 + 512);
+    }
+  };
+  // X of a step: lane (row r16, chunk q of 8 k) reads the slot of (row, chunk) in the step's two blocks
+  const int q4 = lane >> 4;
+  const unsigned xslot = (r16 % MPAD) + MPAD * q4;
+  const unsigned xoff0 = (xslot ^ (q4 & 7)) * 16, xoff1 = (xslot ^ ((q4 + 4) & 7)) * 16;
+  auto multiply = [&](int slot, int local) {
+    const unsigned char* xs = x_lds + (size_t)(first + local) * 2 * XBLOCK;
+    const uint4 x0 = *reinterpret_cast<const uint4*>(xs + xoff0);
+    const uint4 x1 = *reinterpret_cast<const uint4*>(xs + XBLOCK + xoff1);
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[slot][t][0]), as_frag(x0), acc[t], 0, 0, 0);
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[slot][t][1]), as_frag(x1), acc[t], 0, 0, 0);
+  };
+  RopeAhead<1> ahead;
+  if (ROPE) ahead = rope_look_ahead<1, SEGS>(rope, seg, unit[0], lane, M);
+  // The ring is filled once the norming waves have their rows: the rings of every wave of the chip
+  // at once are tens of megabytes, and the rows would queue behind them.
+  if (ROPE) rope_look_ahead_page<1, SEGS>(ahead, rope, seg, unit[0], lane, M);
+  __syncthreads();
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load(d, min(d, mine - 1));     // beyond this wave's steps: a valid step again
+  __syncthreads();                                               // X is there
+
+  {
+    int base = 0;  // the ring holds local steps base .. base + DEPTH - 1
+    for (; base + 2 * DEPTH <= mine; base += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        multiply(d, base + d);
+        load(d, base + DEPTH + d);
+      }
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (base + d < mine) multiply(d, base + d);
+      if (base + DEPTH + d < mine) load(d, base + DEPTH + d);
+    }
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+      if (base + DEPTH + d < mine) multiply(d, base + DEPTH + d);
+  }
+
+  if (SEGS > 1) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      *reinterpret_cast<f32x4*>(partial + (((size_t)wave * NT + t) * 64 + lane) * 4) = acc[t];
+    __syncthreads();
+  }
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u) {
+    if (!live[u]) continue;
+    // the segments' sums in segment order; lane: X row r16, W rows 4 (lane / 16) .. + 3 of tile t
+    auto summed = [&](int t, int e) {
+      if (SEGS == 1) return acc[u * 2 + t][e];
+      float sum = partial[(((size_t)(g * SEGS) * NT + u * 2 + t) * 64 + lane) * 4 + e];
+#pragma unroll
+      for (int q = 1; q < SEGS; ++q) sum += partial[(((size_t)(g * SEGS + q) * NT + u * 2 + t) * 64 + lane) * 4 + e];
+      return sum;
+    };
+    rows_epilogue<2, 1, EPI, SEGS>(summed, seg, unit[u], lane, bias, bias_is_f32, out, out_stride, M, N, mode, rope, ahead);
+  }
+}
+
+// How a product with n / 16 (gated) or n / 32 pairs of row tiles is laid over blocks: streaming
+// waves = groups x segs <= 4, a wave `per_wave` pairs, about one block a CU.  0 groups: not taken.
+struct NormedShape {
+  int groups, per_wave, blocks;
+};
+
+static NormedShape normed_shape(int units, int segs, bool gated) {
+  const int most = NORMED_STREAM_WAVES / segs;                   // groups a block can hold
+  const int per_block = ceil_div(units, 256);
+  int per_wave = gated ? ceil_div(per_block, most) : 1;          // the rotary epilogue: one pair a wave
+  if (per_wave > 3) per_wave = 3;
+  int groups = ceil_div(per_block, per_wave);
+  groups = groups < 1 ? 1 : groups > most ? most : groups;
+  return NormedShape{groups, per_wave, ceil_div(units, groups * per_wave)};
+}
+
+// Whether a product of m rows of width k takes the norm inside: X (and the segments' sums) fit LDS,
+// a lane holds a row's share in registers.
+int gemm_normed_ok(int m, int k) {
+  if (m < 1 || m > NORMED_MAX_M || k % 64 != 0 || k > 256 * NORMED_KC) return 0;
+  return (size_t)(k / 32) * NORMED_MAX_M * 64 + NORMED_STREAM_WAVES * 6 * 1024 <= NORMED_MAX_LDS;
+}
+
+template <int UNITS, int SEGS, int EPI>
+static int launch_normed_of(const NormedRows& in, const bf16_t* w, const void* bias, int bias_is_f32, void* out, int out_stride,
+                            int m, int n, int k, int mode, hipStream_t stream, const RopeStore& rope, int units,
+                            const NormedShape& shape) {
+  const int nw = shape.groups * SEGS;
+  const size_t lds = (size_t)(k / 32) * NORMED_MAX_M * 64 + (SEGS > 1 ? (size_t)nw * 2 * UNITS * 1024 : 0);
+#define NORMED_LAUNCH()                                                                                               \
+  {                                                                                                                   \
+    auto kernel = &gemm_normed_kernel<UNITS, SEGS, UNITS == 1 ? 8 : UNITS == 2 ? 4 : 3, EPI>;                         \
+    static bool configured = false;                                                                                   \
+    if (!configured) {                                                                                                \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                         NORMED_MAX_LDS);                                                             \
+      if (e != hipSuccess) {                                                                                          \
+        axk_set_error("gemm_normed: cannot reserve %d bytes of LDS: %s", NORMED_MAX_LDS, hipGetErrorString(e));       \
+        return -2;                                                                                                    \
+      }                                                                                                               \
+      configured = true;                                                                                              \
+    }                                                                                                                 \
+    kernel<<<shape.blocks, (nw + NORMED_NORM_WAVES) * 64, lds, stream>>>(in, w, bias, bias_is_f32, out, out_stride, m, n, k, \
+                                                                         mode, rope, units);                          \
+  }
+  NORMED_LAUNCH()
+#undef NORMED_LAUNCH
+  AXK_LAUNCH_CHECK("gemm_normed");
+  return 0;
+}
+
+template <int EPI>
+static int launch_normed(const NormedRows& in, const bf16_t* w, const void* bias, int bias_is_f32, void* out, int out_stride,
+                         int m, int n, int k, int mode, hipStream_t stream, int segs, const RopeStore& rope) {
+  const int units = EPI == EPI_GLU ? n / 16 : n / 32;
+  const NormedShape shape = normed_shape(units, segs, EPI == EPI_GLU);
+#define ARGS_NORMED in, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, rope, units, shape
+#define BY_SEGS(U)                                                    \
+  switch (segs) {                                                     \
+    case 1: return launch_normed_of<U, 1, EPI>(ARGS_NORMED);          \
+    case 2: return launch_normed_of<U, 2, EPI>(ARGS_NORMED);          \
+    case 4: return launch_normed_of<U, 4, EPI>(ARGS_NORMED);          \
+  }
+  if (shape.per_wave == 1) BY_SEGS(1)
+  if constexpr (EPI == EPI_GLU) {
+    if (shape.per_wave == 2) BY_SEGS(2)
+    if (shape.per_wave == 3) BY_SEGS(3)
+  }
+#undef BY_SEGS
+#undef ARGS_NORMED
+  axk_set_error("gemm_normed: %d segments, %d pairs of tiles a wave", segs, shape.per_wave);
+  return -1;
+}
+
 // ---------------------------------------------------------------------------- gemm_rows
 // 17 to 64 rows of X: still bound by reading W once, but X is now as large as a tile of W, and a
 // wave that fetched its own X for every step (as gemm_stream does) would ask the caches for as
@@ -1358,6 +1683,27 @@ int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const v
                               workspace, workspace_bytes, &rope);
   return launch_stream_any<EPI_ROPE>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream,
                                      gemm_segments(n / 32, k), rope);
+}
+
+// The gated product and the [q; k; v] product of few rows with the RMS norm of their operand
+// inside (gemm_normed_kernel): rows are the float32 rows the norm would read.
+int launch_gemm_normed_glu(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps, const bf16_t* w,
+                           bf16_t* out, int out_stride, int m, int n, int k, hipStream_t stream) {
+  const NormedRows in = {rows, rows_stride, gain, gain_is_f32, eps};
+  return launch_normed<EPI_GLU>(in, w, nullptr, 0, out, out_stride, m, n, k, MODE_SWIGLU, stream,
+                                gemm_segments(tiles32_of(n, MODE_SWIGLU), k), RopeStore());
+}
+
+int launch_gemm_normed_qkv_rope(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps,
+                                const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out, int out_stride, int m, int n,
+                                int k, const float* table, const int32_t* positions, const int32_t* seq_rows,
+                                const int32_t* block_table, int table_stride, bf16_t* k_cache, bf16_t* v_cache, int n_heads,
+                                int n_kv_heads, int head_dim, int page_size, hipStream_t stream) {
+  const NormedRows in = {rows, rows_stride, gain, gain_is_f32, eps};
+  const RopeStore rope = {table, positions, seq_rows, block_table, table_stride, k_cache, v_cache,
+                          n_heads, n_kv_heads, head_dim, page_size};
+  return launch_normed<EPI_ROPE>(in, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream,
+                                 gemm_segments(n / 32, k), rope);
 }
 
 #endif  // AXON_BF16

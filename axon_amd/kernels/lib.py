@@ -40,6 +40,12 @@ _SIGNATURES = {
     "axk_gemm_qkv_rope": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                           c_int, c_void_p, ctypes.c_long, c_void_p],
+    "axk_gemm_normed_ok": [c_int, c_int, c_int, c_int],
+    "axk_gemm_normed_glu": [c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                            c_void_p],
+    "axk_gemm_normed_qkv_rope": [c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                 c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                                 c_int, c_int, c_int, c_int, c_void_p],
     "axk_attention": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
                       c_int, c_int, c_int, c_int, c_float, c_void_p],
     "axk_attention_prefill": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
@@ -273,6 +279,60 @@ class Kernels:
             _ptr(table), _ptr(positions), _ptr(seq_rows), _ptr(block_table),
             block_table.shape[-1], _ptr(k_cache if write_kv else None), _ptr(v_cache if write_kv else None), n_heads,
             n_kv_heads, head_dim, page_size, 1 if write_kv else 0, _ptr(work), need, _stream()))
+
+    def gemm_normed_ok(self, m: int, n: int, k: int, gated: bool = False) -> bool:
+        """Whether the product of m rows with a packed [n, k] matrix (gated: [gate; up] of 2 n rows)
+        takes the RMS norm of its operand inside (`gemm_normed_glu`, `gemm_normed_qkv_rope`)."""
+        return bool(self.lib.axk_gemm_normed_ok(m, n, k, 1 if gated else 0))
+
+    def _normed_rows(self, rows, gain, K, what):
+        if rows.dtype != torch.float32 or not rows.is_cuda:
+            raise KernelError(f"{what}: the rows must be float32 on the device, got {rows.dtype} on {rows.device}")
+        if rows.dim() != 2 or rows.shape[1] != K or rows.stride(1) != 1 or gain.numel() != K or not gain.is_contiguous():
+            raise KernelError(f"{what}: rows {tuple(rows.shape)} or a gain of {gain.numel()} do not fit K={K}")
+
+    def gemm_normed_glu(self, rows, gain, eps, w, out) -> torch.Tensor:
+        """out = silu(X Wg^T) * (X Wu^T) with X = rmsnorm(rows, gain, eps) worked out inside the
+        kernel (few rows; `gemm_normed_ok`): the same bits as `rmsnorm` followed by `gemm` in the
+        gated mode."""
+        if not isinstance(w, PackedMatrix):
+            raise KernelError("gemm_normed_glu: needs a packed matrix")
+        M, K = rows.shape
+        N = w.shape[0] // 2
+        self._normed_rows(rows, gain, K, "gemm_normed_glu")
+        self._elem(w.data, "gate|up w"); self._elem(out, "gate|up out")
+        if w.shape != (2 * N, K) or out.shape != (M, N) or out.stride(1) != 1:
+            raise KernelError(f"gemm_normed_glu: w {tuple(w.shape)} out {tuple(out.shape)} for rows {tuple(rows.shape)}")
+        self._check(self.lib.axk_gemm_normed_glu(_ptr(rows), rows.stride(0), _ptr(gain), self._vec_flag(gain, "norm gain"),
+                                                 float(eps), _ptr(w), _ptr(out), out.stride(0), M, N, K, _stream()))
+        return out
+
+    def gemm_normed_qkv_rope(self, rows, gain, eps, w, bias, qkv, table, positions, seq_rows, block_table, k_cache, v_cache,
+                             n_heads, n_kv_heads, head_dim, page_size, write_kv=True) -> None:
+        """`gemm_qkv_rope` of X = rmsnorm(rows, gain, eps), X worked out inside the kernel (few
+        rows; `gemm_normed_ok`): the same bits as `rmsnorm` followed by `gemm_qkv_rope`."""
+        if not isinstance(w, PackedMatrix):
+            raise KernelError("gemm_normed_qkv_rope: needs a packed matrix")
+        M, K = rows.shape
+        self._normed_rows(rows, gain, K, "gemm_normed_qkv_rope")
+        self._elem(w.data, "qkv w"); self._elem(qkv, "qkv out"); self._f32(table, "rope table")
+        self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
+        n = (n_heads + (2 * n_kv_heads if write_kv else 0)) * head_dim
+        if w.shape != (n, K):
+            raise KernelError(f"gemm_normed_qkv_rope: w {tuple(w.shape)}, expected [{n}, {K}]")
+        if qkv.shape[0] != M or qkv.shape[1] < n_heads * head_dim or qkv.stride(1) != 1:
+            raise KernelError(f"gemm_normed_qkv_rope: qkv {tuple(qkv.shape)} does not hold [{M}, {n_heads * head_dim}]")
+        if table.shape != (M, head_dim // 2, 2) or positions.numel() != M or seq_rows.numel() != M:
+            raise KernelError(f"gemm_normed_qkv_rope: table {tuple(table.shape)} or positions do not fit {M} tokens")
+        if bias is not None and bias.numel() != n:
+            raise KernelError(f"gemm_normed_qkv_rope: bias of {bias.numel()} for {n} rows")
+        if write_kv:
+            self._check_caches(k_cache, v_cache, n_kv_heads, page_size, head_dim)
+        self._check(self.lib.axk_gemm_normed_qkv_rope(
+            _ptr(rows), rows.stride(0), _ptr(gain), self._vec_flag(gain, "norm gain"), float(eps), _ptr(w), _ptr(bias),
+            self._vec_flag(bias, "qkv bias"), _ptr(qkv), qkv.stride(0), M, K, _ptr(table), _ptr(positions), _ptr(seq_rows),
+            _ptr(block_table), block_table.shape[-1], _ptr(k_cache if write_kv else None),
+            _ptr(v_cache if write_kv else None), n_heads, n_kv_heads, head_dim, page_size, 1 if write_kv else 0, _stream()))
 
     def attention(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, n_heads, n_kv_heads,
                   head_dim, page_size, window, scale) -> torch.Tensor:

@@ -21,7 +21,7 @@ import torch
 
 from ..config.base import ConfigError
 from ..kernels import MODE_ADD_F32, MODE_STORE, PackedMatrix
-from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, build_part, register_mixer
+from .base import CacheBinding, CacheSpec, Mixer, PrecedingNorm, TensorDecl, build_part, register_mixer
 
 
 PREFILL_TILE = 128     # tokens of one request per tile of the prompt kernel
@@ -194,6 +194,13 @@ class GQAttention(Mixer):
     def finishes_following_norm(self, ctx) -> bool:
         return isinstance(self.w_o, PackedMatrix) and ctx.rt.k.gemm_then_norm_ok(ctx.n_tokens, self.hidden, self.q_dim)
 
+    def applies_preceding_norm(self, ctx) -> bool:
+        k = ctx.rt.k
+        rows = self.q_dim + 2 * self.kv_dim
+        return (isinstance(self.w_qkv, PackedMatrix) and self.position is not None
+                and k.gemm_qkv_rope_ok(ctx.n_tokens, rows, self.hidden, self.hd, self.position.rotary_dim)
+                and k.gemm_normed_ok(ctx.n_tokens, rows, self.hidden))
+
     def forward(self, ctx, binding: CacheBinding, h, residual, following=None) -> None:
         k = ctx.rt.k
         T = h.shape[0]
@@ -211,15 +218,21 @@ class GQAttention(Mixer):
         else:
             # reading another run's cache: only the queries are needed
             w, bias = self.w_qkv[:self.q_dim], None if self.b_qkv is None else self.b_qkv[:self.q_dim]
-        if isinstance(w, PackedMatrix) and k.gemm_qkv_rope_ok(T, w.shape[0], self.hidden, self.hd, rotary):
+        in_one = isinstance(w, PackedMatrix) and k.gemm_qkv_rope_ok(T, w.shape[0], self.hidden, self.hd, rotary)
+        cache = (group.block_table, k_cache, v_cache, self.nh, self.nkv, self.hd)
+        if isinstance(h, PrecedingNorm) and not (in_one and k.gemm_normed_ok(T, w.shape[0], self.hidden)):
+            h = h.apply(ctx)
+        if isinstance(h, PrecedingNorm):
+            # few rows: the norm, the product, the rotation and the store into the pages in one launch
+            k.gemm_normed_qkv_rope(h.rows, h.gain, h.eps, w, bias, qkv, table, ctx.positions, ctx.seq_rows, *cache,
+                                   group.page_size, binding.writes)
+        elif in_one:
             # product, rotation and the store into the pages in one launch (a short step) or with the
             # rotation and the store done by the kernel that adds the sums of the product's segments
-            k.gemm_qkv_rope(h, w, bias, qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache,
-                            self.nh, self.nkv, self.hd, group.page_size, binding.writes)
+            k.gemm_qkv_rope(h, w, bias, qkv, table, ctx.positions, ctx.seq_rows, *cache, group.page_size, binding.writes)
         else:
             k.gemm(h, w, qkv[:, :w.shape[0]], bias, MODE_STORE)
-            k.rope_kv_write(qkv, table, ctx.positions, ctx.seq_rows, group.block_table, k_cache, v_cache, self.nh,
-                            self.nkv, self.hd, rotary, group.page_size, binding.writes)
+            k.rope_kv_write(qkv, table, ctx.positions, ctx.seq_rows, *cache, rotary, group.page_size, binding.writes)
         att = ctx.ws.take((T, self.q_dim), ctx.rt.dtype)
         if k.attention_fast_ok(self.hd, group.page_size, self.nh, self.nkv):
             plan = attention_plan(ctx, self.window, self.nh, self.hd)

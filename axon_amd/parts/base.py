@@ -105,9 +105,33 @@ class FollowingNorm:
         return (self.gain, self.values, self.eps)
 
 
+class PrecedingNorm:
+    """A norm handed to the part that runs after it (an option, never a duty: a part that does
+    not say `applies_preceding_norm` gets the normed rows as always).  Where the first product of a
+    part can norm its operand on the way, the norm is no pass of its own: the part gets this
+    object in place of the normed rows, with the float32 `rows` [T, size], the `gain` and `eps`,
+    and gives the same bits as the norm's own pass followed by its product.  `apply(ctx)` is that
+    pass, for a part that finds in the middle of a step that it cannot after all."""
+
+    def __init__(self, norm, rows):
+        self.norm, self.rows, self.gain, self.eps = norm, rows, norm.gain, norm.eps
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    def apply(self, ctx):
+        return self.norm.forward(ctx, self.rows)
+
+
 class Norm(Part):
     def forward(self, ctx, x, out=None):
         raise NotImplementedError
+
+    def preceding(self, ctx, x) -> Optional[PrecedingNorm]:
+        """This norm of the rows x as work for the first product of the part after it, or None if
+        it always runs on its own (the default)."""
+        return None
 
     def following(self, ctx, n_rows: int) -> Optional[FollowingNorm]:
         """This norm as work for the product before it (with a buffer for `n_rows` rows), or None
@@ -157,12 +181,21 @@ class Mixer(Part):
         product also writes the finished norm of the rows it has added into.  Optional."""
         return False
 
+    def applies_preceding_norm(self, ctx) -> bool:
+        """Whether `forward` takes `h` as a PrecedingNorm in this step: its first product norms
+        its operand itself.  Optional."""
+        return False
+
     def forward(self, ctx, binding: CacheBinding, h, residual) -> None:
         raise NotImplementedError
 
 
 class FeedForward(Part):
     def finishes_following_norm(self, ctx) -> bool:
+        """As for a mixer: optional."""
+        return False
+
+    def applies_preceding_norm(self, ctx) -> bool:
         """As for a mixer: optional."""
         return False
 
@@ -203,6 +236,14 @@ class Block(Part):
         if norm is None or part is None or not part.finishes_following_norm(ctx):
             return None
         return norm.following(ctx, n_rows)
+
+
+    @staticmethod
+    def preceding_of(ctx, norm: Optional[Norm], part, x) -> Optional[PrecedingNorm]:
+        """`norm` of the rows x as work for `part`'s first product in this step, or None."""
+        if norm is None or part is None or not part.applies_preceding_norm(ctx):
+            return None
+        return norm.preceding(ctx, x)
 
 
 # --------------------------------------------------------------------------- registries

@@ -11,7 +11,8 @@ from typing import List
 from .base import Block, CacheBinding, TensorDecl, register_block
 
 # A norm behind a product whose kernel holds the finished rows anyway can be written by that
-# kernel (the same bits as the norm's own pass): the block asks its parts, step by step.
+# kernel, and a norm before a product of few rows can be worked out inside that product (the same
+# bits as the norm's own pass, both): the block asks its parts, step by step.
 
 
 class PreNormBlock(Block):
@@ -38,14 +39,20 @@ class PreNormBlock(Block):
         return self.feed_forward
 
     def forward(self, ctx, binding: CacheBinding, x, normed=None, following=None) -> None:
-        h = normed if normed is not None else self.norm1.forward(ctx, x)
+        h = normed
+        if h is None:
+            h = self.preceding_of(ctx, self.norm1, self.mixer, x)
+        if h is None:
+            h = self.norm1.forward(ctx, x)
         second = self.following_of(ctx, self.mixer, self.norm2, x.shape[0])
         if second is not None:
             self.mixer.forward(ctx, binding, h, x, second)
             h = second.values
         else:
             self.mixer.forward(ctx, binding, h, x)
-            h = self.norm2.forward(ctx, x)
+            h = self.preceding_of(ctx, self.norm2, self.feed_forward, x)
+            if h is None:
+                h = self.norm2.forward(ctx, x)
         if following is not None:
             self.feed_forward.forward(ctx, h, x, following)
         else:

@@ -10,7 +10,7 @@ from __future__ import annotations
 from typing import List
 
 from ..kernels import MODE_ADD_F32, MODE_SWIGLU, PackedMatrix
-from .base import FeedForward, TensorDecl, register_feed_forward
+from .base import FeedForward, PrecedingNorm, TensorDecl, register_feed_forward
 
 
 class SwiGLUMLP(FeedForward):
@@ -36,10 +36,17 @@ class SwiGLUMLP(FeedForward):
     def finishes_following_norm(self, ctx) -> bool:
         return isinstance(self.w_down, PackedMatrix) and ctx.rt.k.gemm_then_norm_ok(ctx.n_tokens, self.hidden, self.ffn)
 
+    def applies_preceding_norm(self, ctx) -> bool:
+        return (isinstance(self.w_gate_up, PackedMatrix)
+                and ctx.rt.k.gemm_normed_ok(ctx.n_tokens, self.ffn, self.hidden, gated=True))
+
     def forward(self, ctx, h, residual, following=None) -> None:
         k = ctx.rt.k
         act = ctx.ws.take((h.shape[0], self.ffn), ctx.rt.dtype)
-        k.gemm(h, self.w_gate_up, act, None, MODE_SWIGLU)       # silu(gate h) * up h, in the product's epilogue
+        if isinstance(h, PrecedingNorm):                        # few rows: the norm inside the product
+            k.gemm_normed_glu(h.rows, h.gain, h.eps, self.w_gate_up, act)
+        else:
+            k.gemm(h, self.w_gate_up, act, None, MODE_SWIGLU)   # silu(gate h) * up h, in the product's epilogue
         k.gemm(act, self.w_down, residual, None, MODE_ADD_F32,
                following_norm=None if following is None else following.as_argument())
 

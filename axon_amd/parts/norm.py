@@ -9,7 +9,7 @@ from typing import List, Optional
 
 import torch
 
-from .base import FollowingNorm, Norm, TensorDecl, register_norm
+from .base import FollowingNorm, Norm, PrecedingNorm, TensorDecl, register_norm
 
 
 class RMSNorm(Norm):
@@ -37,6 +37,11 @@ class RMSNorm(Norm):
     def following(self, ctx, n_rows: int) -> Optional[FollowingNorm]:
         """The product before the norm writes the finished rows (where its kernel offers it)."""
         return FollowingNorm(self.gain, self.eps, ctx.ws.take((n_rows, self.size), ctx.rt.dtype))
+
+    def preceding(self, ctx, x) -> Optional[PrecedingNorm]:
+        """The product after the norm reads the float32 rows and norms them on the way (where its
+        kernel offers it)."""
+        return PrecedingNorm(self, x)
 
 
 register_norm("rmsnorm", RMSNorm)

@@ -54,6 +54,42 @@ def test_cache_rows_are_the_same_bits_however_the_tokens_were_fed(name, dtype, m
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("name", ["D", "E"])
+def test_a_norm_inside_the_product_after_it_changes_no_bit(name, model_dirs, monkeypatch):
+    """Steps of up to eight tokens hand their norms to the product after them (the [q; k; v] product
+    and the gated product norm their operand on the way; model E's width is taken by that kernel
+    whole, D's leaves lanes of a row's last round idle): logits and cache rows are those of the same steps
+    with every norm a pass of its own, and the kernel did run."""
+    from axon_amd.parts.attention import GQAttention
+    from axon_amd.parts.mlp import SwiGLUMLP
+    d = model_dirs(name, "bfloat16")
+    page = TINY[name]["page_size"]
+    a, b = prompts_for(name, [90, 60], seed=29)
+
+    def run(eng):
+        out = [eng.step([StepEntry("a", a[:70], [69]), StepEntry("b", b[:30], [])])]
+        out.append(eng.step([StepEntry("a", a[70:73], [0, 2]), StepEntry("b", b[30:35], [4])]))      # 8 tokens
+        for t in range(73, 84):                                                                 # 1 or 2 tokens
+            out.append(eng.step([StepEntry("a", a[t:t + 1], [0])] + ([StepEntry("b", b[t - 38:t - 37], [0])] if t % 3 else [])))
+        return torch.cat([o.clone() for o in out]), cache_rows(eng, "a")
+
+    calls = []
+    inside = engine_for(d, "bfloat16", page, 32)
+    k = inside.rt.k
+    glu, qkv = k.gemm_normed_glu, k.gemm_normed_qkv_rope
+    monkeypatch.setattr(k, "gemm_normed_glu", lambda *a_, **kw: (calls.append("glu"), glu(*a_, **kw))[1])
+    monkeypatch.setattr(k, "gemm_normed_qkv_rope", lambda *a_, **kw: (calls.append("qkv"), qkv(*a_, **kw))[1])
+    got, got_rows = run(inside)
+    assert calls.count("glu") >= 12 and calls.count("qkv") >= 12
+    monkeypatch.setattr(GQAttention, "applies_preceding_norm", lambda self, ctx: False)
+    monkeypatch.setattr(SwiGLUMLP, "applies_preceding_norm", lambda self, ctx: False)
+    calls.clear()
+    apart = engine_for(d, "bfloat16", page, 32)
+    want, want_rows = run(apart)
+    assert not calls
+    assert torch.equal(got, want) and torch.equal(got_rows, want_rows)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["D", "E"])
 def test_a_replayed_graph_gives_the_bits_of_the_step_launched_kernel_by_kernel(name, dtype, model_dirs):

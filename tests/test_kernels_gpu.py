@@ -342,6 +342,71 @@ def test_qkv_product_with_rotation_and_cache_store_in_one(M, nh, nkv, hd, hidden
         assert write_kv == bool((got[1] != 7.0).any())
 
 
+@pytest.mark.parametrize("M,hidden,ffn", [(1, 64, 32), (8, 3584, 4864), (3, 192, 320), (8, 256, 9600), (7, 1024, 8192),
+                                          (8, 4096, 256), (5, 896, 4864), (2, 3584, 2368), (6, 3584, 18944)])
+@pytest.mark.parametrize("gain_dt", [torch.bfloat16, torch.float32])
+def test_gated_product_with_the_norm_inside(M, hidden, ffn, gain_dt):
+    """The norm worked out inside the product against the norm kernel followed by the product: the
+    same bits (the norm is the norm kernel's arithmetic, the product's order of addition the same)."""
+    k = kernels("bfloat16")
+    assert k.gemm_normed_ok(M, ffn, hidden, gated=True)
+    assert not k.gemm_normed_ok(9, ffn, hidden, gated=True) and not k.gemm_normed_ok(M, ffn, 8192, gated=True)
+    assert not kernels("float32").gemm_normed_ok(M, ffn, hidden, gated=True)
+    rows = (rnd(M + 2, hidden + 8, seed=60) * 3.0).float().cuda()[1:M + 1, :hidden]      # strided rows
+    gain = (1.0 + rnd(hidden, seed=61)).to(gain_dt).cuda()
+    w, _ = as_dtype(rnd(2 * ffn, hidden, seed=62, scale=0.2), "bfloat16")
+    ww = k.pack_matrix(w)
+    x = torch.empty(M, hidden, dtype=torch.bfloat16, device="cuda")
+    k.rmsnorm(rows.contiguous(), gain, 1e-5, x)
+    want = torch.empty(M, ffn, dtype=torch.bfloat16, device="cuda")
+    k.gemm(x, ww, want, None, MODE_SWIGLU)
+    got = torch.full((M + 1, ffn + 8), 7.0, dtype=torch.bfloat16, device="cuda")
+    k.gemm_normed_glu(rows, gain, 1e-5, ww, got[:M, :ffn])
+    assert torch.equal(got[:M, :ffn], want)
+    assert (got[M] == 7.0).all() and (got[:, ffn:] == 7.0).all()
+
+
+@pytest.mark.parametrize("M,nh,nkv,hd,hidden,page", [(1, 4, 2, 32, 64, 8), (8, 28, 4, 128, 3584, 64), (6, 7, 1, 128, 256, 8),
+                                                      (7, 3, 3, 96, 128, 4), (5, 4, 1, 64, 320, 32), (3, 14, 2, 64, 896, 16)])
+def test_qkv_product_with_the_norm_inside(M, nh, nkv, hd, hidden, page):
+    """As above for the [q; k; v] product with rotation and cache store: the same bits in q and in
+    the pages as the norm kernel followed by `gemm_qkv_rope`."""
+    k = kernels("bfloat16")
+    width = (nh + 2 * nkv) * hd
+    assert k.gemm_normed_ok(M, width, hidden)
+    rows = (rnd(M, hidden, seed=70) * 2.0).float().cuda()
+    gain = (1.0 + rnd(hidden, seed=71)).to(torch.bfloat16).cuda()
+    w, _ = as_dtype(rnd(width, hidden, seed=72, scale=0.2), "bfloat16")
+    g = torch.Generator().manual_seed(73)
+    n_pages, max_pages = 40, 8
+    slots = torch.randperm(3 * max_pages * page, generator=g)[:M]
+    seq = (slots // (max_pages * page)).to(torch.int32)
+    pos = (slots % (max_pages * page)).to(torch.int32)
+    table_of_pages = torch.randperm(n_pages, generator=g)[:3 * max_pages].view(3, max_pages).to(torch.int32).cuda()
+    table = torch.empty(M, hd // 2, 2, dtype=torch.float32, device="cuda")
+    k.rope_table(pos.cuda(), P.rope_freqs(hd, 10000.0).cuda(), table)
+    x = torch.empty(M, hidden, dtype=torch.bfloat16, device="cuda")
+    k.rmsnorm(rows, gain, 1e-6, x)
+    for bias_dt, write_kv in ((None, True), (torch.float32, True), (torch.bfloat16, False)):
+        bias = None if bias_dt is None else rnd(width, seed=74).to(bias_dt).cuda()
+        n_rows = width if write_kv else nh * hd
+        ww, bb = k.pack_matrix(w[:n_rows].contiguous()), (None if bias is None else bias[:n_rows])
+        got, want = [], []
+        for inside in (True, False):
+            kc = torch.full((n_pages, nkv, page, hd), 7.0, dtype=torch.bfloat16, device="cuda")
+            vc = torch.full((n_pages, nkv, hd, page), 7.0, dtype=torch.bfloat16, device="cuda")
+            qkv = torch.zeros(M, width, dtype=torch.bfloat16, device="cuda")
+            if inside:
+                k.gemm_normed_qkv_rope(rows, gain, 1e-6, ww, bb, qkv, table, pos.cuda(), seq.cuda(), table_of_pages, kc, vc,
+                                       nh, nkv, hd, page, write_kv)
+            else:
+                k.gemm_qkv_rope(x, ww, bb, qkv, table, pos.cuda(), seq.cuda(), table_of_pages, kc, vc, nh, nkv, hd, page,
+                                write_kv)
+            (got if inside else want).extend([qkv[:, :nh * hd].clone(), kc, vc])
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_strided_rows(dtype):
     k = kernels(dtype)
