@@ -55,6 +55,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0: all)")
     ap.add_argument("--prompt", type=int, default=0, help="prompt tokens of every decoding request (default: the size's own)")
     ap.add_argument("--dtype", default="bfloat16")
+    ap.add_argument("--page-size", type=int, default=16, help="positions in a cache page (default: the 16 that the "
+                    "measured configurations name; the engine's own default is 64, a block of its attention kernels)")
     ap.add_argument("--sizes", default="7b", choices=sorted(SIZES), help="layer sizes of Qwen2.5-7B (the default), 14B or 32B")
     ap.add_argument("--no-points", action="store_true", help="only the headline batch and the prefill point")
     ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "mixed"],
@@ -81,7 +83,7 @@ def main() -> int:
         cfg["num_hidden_layers"] = args.layers
     L, dim, ffn, V = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     nh, nkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
-    ctx_len, page = cfg["max_position_embeddings"], 64
+    ctx_len, page = cfg["max_position_embeddings"], args.page_size
     elem = 2 if args.dtype == "bfloat16" else 4
     points_on = not args.no_points and args.phase == "all"
     most_batch = max(args.batch, 64) if points_on else max(args.batch, 36 if args.phase == "mixed" else 1)
