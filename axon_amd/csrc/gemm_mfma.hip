@@ -26,6 +26,10 @@
 //   Epilogues: bias / residual add / SwiGLU, and the attention's qkv product with the rotary
 //   encoding and the store into the paged cache.
 //
+// * gemm_normed (M <= 8, the operand an RMS norm of float32 rows): gemm_stream's product with the
+//   norm inside; waves of their own norm the rows into LDS while the streaming waves fill their
+//   rings, so the norm is no launch of its own in a decoding step.
+//
 // * gemm_rows (17 <= M <= 64): W still streams into registers, but the waves of a block walk the
 //   same segment of K and share X through LDS; a block a segment, the sums of several segments
 //   through a workspace.
