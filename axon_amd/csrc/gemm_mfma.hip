@@ -948,8 +948,8 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
 // X = bf16((row * inv) * gain) in LDS, in the blocks of MPAD rows x 32 k that one LDS read of a
 // wave takes as an MFMA operand.  The others stream W as gemm_stream does (G groups of tiles times
 // the S segments of K, a wave each; every block needs all of X, so G is such that each CU has
-// about one block): their ring of loads is filled while the rows are normed (as soon as the
-// rows themselves have arrived), and they start to multiply when X is there.  The norm is the norm kernel's, bit for bit: a wave takes a row, lane
+// about one block): their ring of loads is filled while the rows are normed (behind the loads
+// of the rows themselves), and they start to multiply when X is there.  The norm is the norm kernel's, bit for bit: a wave takes a row, lane
 // l stands for that kernel's threads l, 64 + l, 128 + l and 192 + l (four chains over the float4
 // l + 64 j, j = v, v + 4, ...), the four butterflies are added in order.  Takes the norm's launch
 // out of a decoding step.
@@ -1004,7 +1004,7 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
     const unsigned swz = (q + 4 * ((ln >> 3) & 1)) & 7;           // slots of 16 bytes (a row's 8 k) are permuted within
     unsigned char* at0 = x_lds + (ln >> 3) * XBLOCK + (ln & 1) * 8;   // eights, by chunk and block parity: these stores,
                                                                   // which walk along a row, spread over the banks
-    if (first_row >= M) __syncthreads();                        // a wave without rows: the barrier of those with
+    if (first_row >= M) __builtin_amdgcn_s_barrier();           // a wave without rows: the barrier of those with
     for (int m0 = first_row; m0 < M; m0 += 2 * NORMED_NORM_WAVES) {
       const int m1 = m0 + NORMED_NORM_WAVES;
       float4 kept[2][KC];
@@ -1021,6 +1021,13 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
           }
         }
       }
+      if (m0 == first_row) {
+        // the rows are asked for: only now do the streaming waves ask for their W (the barrier alone,
+        // which waits for no load; nothing moves across it)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+      }
       // four chains a row as the norm kernel's four waves have them, then their butterflies, all
       // eight side by side (a step of a butterfly is a round trip through the LDS crossbar)
       float ss[2][4];
@@ -1036,10 +1043,6 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
           ss[r][j & 3] = fmaf(x.z, x.z, ss[r][j & 3]);
           ss[r][j & 3] = fmaf(x.w, x.w, ss[r][j & 3]);
         }
-      }
-      if (m0 == first_row) {
-        asm volatile("" :: "v"(ss[0][0]), "v"(ss[1][0]), "v"(ss[0][3]), "v"(ss[1][3]));   // the sums, so the rows, are here
-        __syncthreads();                 // ... and only now do the streaming waves ask for all their W
       }
 #pragma unroll
       for (int off = 32; off > 0; off >>= 1) {
@@ -1145,10 +1148,12 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
   };
   RopeAhead<1> ahead;
   if (ROPE) ahead = rope_look_ahead<1, SEGS>(rope, seg, unit[0], lane, M);
-  // The ring is filled once the norming waves have their rows: the rings of every wave of the chip
-  // at once are tens of megabytes, and the rows would queue behind them.
+  // The ring is filled once the norming waves have asked for their rows: the rings of every wave of
+  // the chip at once are tens of megabytes, and rows asked for among them arrive last.
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
   if (ROPE) rope_look_ahead_page<1, SEGS>(ahead, rope, seg, unit[0], lane, M);
-  __syncthreads();
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) load(d, min(d, mine - 1));     // beyond this wave's steps: a valid step again
   __syncthreads();                                               // X is there
