@@ -158,9 +158,9 @@ int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const v
                          bf16_t* v_cache, int n_heads, int n_kv_heads, int head_dim, int page_size, void* workspace,
                          size_t workspace_bytes, hipStream_t stream);
 int gemm_normed_ok(int m, int k);
-int launch_gemm_normed_glu(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps, const bf16_t* w,
-                           bf16_t* out, int out_stride, int m, int n, int k, hipStream_t stream);
-int launch_gemm_normed_qkv_rope(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps,
+int launch_gemm_normed_glu(const float* rows, int rows_stride, const bf16_t* gain, float eps, const bf16_t* w, bf16_t* out,
+                           int out_stride, int m, int n, int k, hipStream_t stream);
+int launch_gemm_normed_qkv_rope(const float* rows, int rows_stride, const bf16_t* gain, float eps,
                                 const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out, int out_stride, int m, int n,
                                 int k, const float* table, const int32_t* positions, const int32_t* seq_rows,
                                 const int32_t* block_table, int table_stride, bf16_t* k_cache, bf16_t* v_cache, int n_heads,
@@ -313,12 +313,13 @@ extern "C" int axk_gemm_normed_glu(const float* rows, int rows_stride, const voi
                                    const void* w, void* out, int out_stride, int m, int n, int k, void* stream) {
 #if AXON_BF16
   AXK_REQUIRE(axk_gemm_normed_ok(m, n, k, 1), "gemm_normed_glu: M=%d N=%d K=%d are not taken", m, n, k);
+  AXK_REQUIRE(!gain_is_f32, "gemm_normed_glu: the gain must be bfloat16");
   AXK_REQUIRE(rows && gain && w && out, "gemm_normed_glu: an operand is missing");
   AXK_REQUIRE(rows_stride >= k && rows_stride % 4 == 0 && out_stride >= n && ((uintptr_t)rows & 15) == 0 &&
                   ((uintptr_t)gain & 15) == 0 && ((uintptr_t)w & 15) == 0,
               "gemm_normed_glu: strides rows=%d out=%d or the alignment of an operand are not taken", rows_stride, out_stride);
-  return launch_gemm_normed_glu(rows, rows_stride, gain, gain_is_f32, eps, (const bf16_t*)w, (bf16_t*)out, out_stride, m, n, k,
-                                (hipStream_t)stream);
+  return launch_gemm_normed_glu(rows, rows_stride, (const bf16_t*)gain, eps, (const bf16_t*)w, (bf16_t*)out, out_stride, m, n,
+                                k, (hipStream_t)stream);
 #else
   axk_set_error("gemm_normed_glu: only in the bfloat16 build");
   return -1;
@@ -337,6 +338,7 @@ extern "C" int axk_gemm_normed_qkv_rope(const float* rows, int rows_stride, cons
   AXK_REQUIRE(axk_gemm_normed_ok(m, n, k, 0) && axk_gemm_qkv_rope_ok(m, n, k, head_dim, head_dim),
               "gemm_normed_qkv_rope: M=%d N=%d K=%d head_dim=%d are not taken", m, n, k, head_dim);
   AXK_REQUIRE(rows && gain && w && qkv, "gemm_normed_qkv_rope: an operand is missing");
+  AXK_REQUIRE(!gain_is_f32, "gemm_normed_qkv_rope: the gain must be bfloat16");
   AXK_REQUIRE(rows_stride >= k && rows_stride % 4 == 0 && qkv_stride >= n_heads * head_dim && qkv_stride % 4 == 0 &&
                   ((uintptr_t)rows & 15) == 0 && ((uintptr_t)gain & 15) == 0 && ((uintptr_t)w & 15) == 0 &&
                   ((uintptr_t)qkv & 7) == 0 && ((uintptr_t)table & 15) == 0,
@@ -344,7 +346,7 @@ extern "C" int axk_gemm_normed_qkv_rope(const float* rows, int rows_stride, cons
               qkv_stride);
   AXK_REQUIRE(table && positions && (!write_kv || (seq_rows && block_table && k_cache && v_cache)),
               "gemm_normed_qkv_rope: a table, the positions or the cache is missing");
-  return launch_gemm_normed_qkv_rope(rows, rows_stride, gain, gain_is_f32, eps, (const bf16_t*)w, bias, bias_is_f32,
+  return launch_gemm_normed_qkv_rope(rows, rows_stride, (const bf16_t*)gain, eps, (const bf16_t*)w, bias, bias_is_f32,
                                      (bf16_t*)qkv, qkv_stride, m, n, k, table, positions, seq_rows, block_table, table_stride,
                                      (bf16_t*)k_cache, (bf16_t*)v_cache, n_heads, n_kv_heads, head_dim, page_size,
                                      (hipStream_t)stream);

@@ -949,15 +949,15 @@ gemm_stream_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __r
 // wave takes as an MFMA operand.  The others stream W as gemm_stream does (G groups of tiles times
 // the S segments of K, a wave each; every block needs all of X, so G is such that each CU has
 // about one block): their ring of loads is filled while the rows are normed (behind the loads
-// of the rows themselves), and they start to multiply when X is there.  The norm is the norm kernel's, bit for bit: a wave takes a row, lane
-// l stands for that kernel's threads l, 64 + l, 128 + l and 192 + l (four chains over the float4
+// of the rows themselves), and they start to multiply when X is there.  The gain is bfloat16 and
+// K a multiple of 256.  The norm is the norm kernel's, bit for bit: a wave takes a row, lane l
+// stands for that kernel's threads l, 64 + l, 128 + l and 192 + l (four chains over the float4
 // l + 64 j, j = v, v + 4, ...), the four butterflies are added in order.  Takes the norm's launch
 // out of a decoding step.
 struct NormedRows {
   const float* rows;       // [M, K], rows_stride apart
   int rows_stride;
-  const void* gain;        // [K]
-  int gain_is_f32;
+  const bf16_t* gain;      // [K]
   float eps;
 };
 
@@ -986,19 +986,17 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
 
   if (wave >= nw) {
     // ------------------------------------------------------------------ a norming wave: rows w, w + 4, ..., two at a time
-    // A row is n4 float4: `full` rounds of the 64 lanes and `tail` lanes more; lane l holds the
-    // float4 l + 64 j.  In LDS that is block (l >> 3) + 8 j of X, chunk (l & 7) >> 1, half l & 1:
-    // one address a lane and row, 8 blocks further for every j.
-    const int n4 = K / 4, full = n4 >> 6, tail = n4 & 63, first_row = wave - nw;
+    // A row is `full` rounds of 64 float4 (K a multiple of 256); lane l holds the float4 l + 64 j.
+    // In LDS that is block (l >> 3) + 8 j of X, chunk (l & 7) >> 1, half l & 1: one address a lane
+    // and row, 8 blocks further for every j.
+    const int full = K >> 8, first_row = wave - nw;
     int ln = lane;
     asm volatile("" : "+v"(ln));        // what follows from the lane is worked out here, not kept in registers from the start
-    const bool in_tail = ln < tail;
-    uint2 gain_bf[KC];                                          // a bfloat16 gain: the lane's share, asked for with the rows
-    if (!in.gain_is_f32 && first_row < M) {
+    uint2 gain_bf[KC];                                          // the gain (bfloat16): the lane's share, asked for with the rows
+    if (first_row < M) {
 #pragma unroll
       for (int j = 0; j < KC; ++j)
-        if (j < full || (j == full && in_tail))
-          gain_bf[j] = *reinterpret_cast<const uint2*>((const bf16_t*)in.gain + 4 * (ln + 64 * j));
+        if (j < full) gain_bf[j] = *reinterpret_cast<const uint2*>((const bf16_t*)in.gain + 4 * (ln + 64 * j));
     }
     const int q = (ln & 7) >> 1;
     const unsigned swz = (q + 4 * ((ln >> 3) & 1)) & 7;           // slots of 16 bytes (a row's 8 k) are permuted within
@@ -1013,13 +1011,8 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
         const int m = min(r ? m1 : m0, M - 1);                   // no second row: the first again, not stored
         const float4* row = reinterpret_cast<const float4*>(in.rows + (size_t)m * in.rows_stride) + ln;
 #pragma unroll
-        for (int j = 0; j < KC; ++j) {
-          if (j < full) kept[r][j] = row[64 * j];                // the same for every lane: a branch, no mask
-          else {
-            kept[r][j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            if (j == full && in_tail) kept[r][j] = row[64 * j];
-          }
-        }
+        for (int j = 0; j < KC; ++j)
+          kept[r][j] = j < full ? row[64 * j] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);     // (the same for every lane)
       }
       if (m0 == first_row) {
         // the rows are asked for: only now do the streaming waves ask for their W (the barrier alone,
@@ -1029,7 +1022,7 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
         asm volatile("" ::: "memory");
       }
       // four chains a row as the norm kernel's four waves have them, then their butterflies, all
-      // eight side by side (a step of a butterfly is a round trip through the LDS crossbar)
+      // eight side by side
       float ss[2][4];
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
@@ -1044,8 +1037,13 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
           ss[r][j & 3] = fmaf(x.w, x.w, ss[r][j & 3]);
         }
       }
+      // wave_sum's butterfly (lane l adds lane l ^ off, off = 32, 16, 8, 4, 2, 1): the same pairs, so
+      // the same bits.  The steps across rows of 16 lanes go through the LDS crossbar, those within a
+      // row through the adder's lane permutations, which cost an instruction and no round trip.
+#define NORMED_DPP(val, old, ctrl, banks) \
+  __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, val), ctrl, 0xf, banks, false))
 #pragma unroll
-      for (int off = 32; off > 0; off >>= 1) {
+      for (int off = 32; off >= 16; off >>= 1) {
         float other[2][4];
 #pragma unroll
         for (int r = 0; r < 2; ++r)
@@ -1056,6 +1054,19 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
 #pragma unroll
           for (int v = 0; v < 4; ++v) ss[r][v] += other[r][v];
       }
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float x = ss[r][v];
+          x += NORMED_DPP(x, 0.0f, 0x128, 0xf);                              // row_ror:8: lane l ^ 8
+          const float up = NORMED_DPP(x, 0.0f, 0x104, 0x5);                  // row_shl:4 in lanes 0-3, 8-11: lane l + 4
+          x += NORMED_DPP(x, up, 0x114, 0xa);                                // row_shr:4 in lanes 4-7, 12-15: lane l - 4
+          x += NORMED_DPP(x, 0.0f, 0x4e, 0xf);                               // quad_perm [2, 3, 0, 1]: lane l ^ 2
+          x += NORMED_DPP(x, 0.0f, 0xb1, 0xf);                               // quad_perm [1, 0, 3, 2]: lane l ^ 1
+          ss[r][v] = x;
+        }
+#undef NORMED_DPP
       float inv[2];
       unsigned char* at[2];
 #pragma unroll
@@ -1068,14 +1079,10 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
       // a chunk of the gain at a time, for both rows
 #pragma unroll
       for (int j = 0; j < KC; ++j) {
-        if (!(j < full || (j == full && in_tail))) continue;     // (for j != full the same for every lane)
-        float4 gn;
-        if (in.gain_is_f32) gn = *reinterpret_cast<const float4*>((const float*)in.gain + 4 * (ln + 64 * j));
-        else {
-          const uint2 gb = gain_bf[j];
-          gn = make_float4(__uint_as_float(gb.x << 16), __uint_as_float(gb.x & 0xffff0000u), __uint_as_float(gb.y << 16),
-                           __uint_as_float(gb.y & 0xffff0000u));
-        }
+        if (j >= full) continue;                                 // (the same for every lane)
+        const uint2 gb = gain_bf[j];
+        const float4 gn = make_float4(__uint_as_float(gb.x << 16), __uint_as_float(gb.x & 0xffff0000u),
+                                      __uint_as_float(gb.y << 16), __uint_as_float(gb.y & 0xffff0000u));
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
           if (r && !second) continue;
@@ -1217,7 +1224,7 @@ static NormedShape normed_shape(int units, int segs, bool gated) {
 // Whether a product of m rows of width k takes the norm inside: X (and the segments' sums) fit LDS,
 // a lane holds a row's share in registers.
 int gemm_normed_ok(int m, int k) {
-  if (m < 1 || m > NORMED_MAX_M || k % 64 != 0 || k > 256 * NORMED_KC) return 0;
+  if (m < 1 || m > NORMED_MAX_M || k % 256 != 0 || k > 256 * NORMED_KC) return 0;     // whole rounds of 64 float4 a row
   return (size_t)(k / 32) * NORMED_MAX_M * 64 + NORMED_STREAM_WAVES * 6 * 1024 <= NORMED_MAX_LDS;
 }
 
@@ -1696,19 +1703,19 @@ int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const v
 
 // The gated product and the [q; k; v] product of few rows with the RMS norm of their operand
 // inside (gemm_normed_kernel): rows are the float32 rows the norm would read.
-int launch_gemm_normed_glu(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps, const bf16_t* w,
-                           bf16_t* out, int out_stride, int m, int n, int k, hipStream_t stream) {
-  const NormedRows in = {rows, rows_stride, gain, gain_is_f32, eps};
+int launch_gemm_normed_glu(const float* rows, int rows_stride, const bf16_t* gain, float eps, const bf16_t* w, bf16_t* out,
+                           int out_stride, int m, int n, int k, hipStream_t stream) {
+  const NormedRows in = {rows, rows_stride, gain, eps};
   return launch_normed<EPI_GLU>(in, w, nullptr, 0, out, out_stride, m, n, k, MODE_SWIGLU, stream,
                                 gemm_segments(tiles32_of(n, MODE_SWIGLU), k), RopeStore());
 }
 
-int launch_gemm_normed_qkv_rope(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps,
+int launch_gemm_normed_qkv_rope(const float* rows, int rows_stride, const bf16_t* gain, float eps,
                                 const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out, int out_stride, int m, int n,
                                 int k, const float* table, const int32_t* positions, const int32_t* seq_rows,
                                 const int32_t* block_table, int table_stride, bf16_t* k_cache, bf16_t* v_cache, int n_heads,
                                 int n_kv_heads, int head_dim, int page_size, hipStream_t stream) {
-  const NormedRows in = {rows, rows_stride, gain, gain_is_f32, eps};
+  const NormedRows in = {rows, rows_stride, gain, eps};
   const RopeStore rope = {table, positions, seq_rows, block_table, table_stride, k_cache, v_cache,
                           n_heads, n_kv_heads, head_dim, page_size};
   return launch_normed<EPI_ROPE>(in, w, bias, bias_is_f32, out, out_stride, m, n, k, MODE_STORE, stream,

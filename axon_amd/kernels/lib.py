@@ -280,9 +280,12 @@ class Kernels:
             block_table.shape[-1], _ptr(k_cache if write_kv else None), _ptr(v_cache if write_kv else None), n_heads,
             n_kv_heads, head_dim, page_size, 1 if write_kv else 0, _ptr(work), need, _stream()))
 
-    def gemm_normed_ok(self, m: int, n: int, k: int, gated: bool = False) -> bool:
+    def gemm_normed_ok(self, m: int, n: int, k: int, gated: bool = False, gain=None) -> bool:
         """Whether the product of m rows with a packed [n, k] matrix (gated: [gate; up] of 2 n rows)
-        takes the RMS norm of its operand inside (`gemm_normed_glu`, `gemm_normed_qkv_rope`)."""
+        takes the RMS norm of its operand inside (`gemm_normed_glu`, `gemm_normed_qkv_rope`); with
+        `gain`, also whether that gain is one the kernels take (bfloat16)."""
+        if gain is not None and gain.dtype != torch.bfloat16:
+            return False
         return bool(self.lib.axk_gemm_normed_ok(m, n, k, 1 if gated else 0))
 
     def _normed_rows(self, rows, gain, K, what):

@@ -220,7 +220,7 @@ class GQAttention(Mixer):
             w, bias = self.w_qkv[:self.q_dim], None if self.b_qkv is None else self.b_qkv[:self.q_dim]
         in_one = isinstance(w, PackedMatrix) and k.gemm_qkv_rope_ok(T, w.shape[0], self.hidden, self.hd, rotary)
         cache = (group.block_table, k_cache, v_cache, self.nh, self.nkv, self.hd)
-        if isinstance(h, PrecedingNorm) and not (in_one and k.gemm_normed_ok(T, w.shape[0], self.hidden)):
+        if isinstance(h, PrecedingNorm) and not (in_one and k.gemm_normed_ok(T, w.shape[0], self.hidden, gain=h.gain)):
             h = h.apply(ctx)
         if isinstance(h, PrecedingNorm):
             # few rows: the norm, the product, the rotation and the store into the pages in one launch

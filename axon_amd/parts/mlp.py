@@ -43,6 +43,8 @@ class SwiGLUMLP(FeedForward):
     def forward(self, ctx, h, residual, following=None) -> None:
         k = ctx.rt.k
         act = ctx.ws.take((h.shape[0], self.ffn), ctx.rt.dtype)
+        if isinstance(h, PrecedingNorm) and not k.gemm_normed_ok(h.shape[0], self.ffn, self.hidden, gated=True, gain=h.gain):
+            h = h.apply(ctx)
         if isinstance(h, PrecedingNorm):                        # few rows: the norm inside the product
             k.gemm_normed_glu(h.rows, h.gain, h.eps, self.w_gate_up, act)
         else:

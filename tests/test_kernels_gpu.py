@@ -342,18 +342,19 @@ def test_qkv_product_with_rotation_and_cache_store_in_one(M, nh, nkv, hd, hidden
         assert write_kv == bool((got[1] != 7.0).any())
 
 
-@pytest.mark.parametrize("M,hidden,ffn", [(1, 64, 32), (8, 3584, 4864), (3, 192, 320), (8, 256, 9600), (7, 1024, 8192),
-                                          (8, 4096, 256), (5, 896, 4864), (2, 3584, 2368), (6, 3584, 18944)])
-@pytest.mark.parametrize("gain_dt", [torch.bfloat16, torch.float32])
-def test_gated_product_with_the_norm_inside(M, hidden, ffn, gain_dt):
+@pytest.mark.parametrize("M,hidden,ffn", [(1, 256, 32), (8, 3584, 4864), (3, 768, 320), (8, 256, 9600), (7, 1024, 8192),
+                                          (8, 4096, 256), (5, 512, 4864), (2, 3584, 2368), (6, 3584, 18944)])
+def test_gated_product_with_the_norm_inside(M, hidden, ffn):
     """The norm worked out inside the product against the norm kernel followed by the product: the
     same bits (the norm is the norm kernel's arithmetic, the product's order of addition the same)."""
     k = kernels("bfloat16")
     assert k.gemm_normed_ok(M, ffn, hidden, gated=True)
     assert not k.gemm_normed_ok(9, ffn, hidden, gated=True) and not k.gemm_normed_ok(M, ffn, 8192, gated=True)
+    assert not k.gemm_normed_ok(M, ffn, hidden + 64, gated=True)          # rows in whole rounds of 256 columns
     assert not kernels("float32").gemm_normed_ok(M, ffn, hidden, gated=True)
     rows = (rnd(M + 2, hidden + 8, seed=60) * 3.0).float().cuda()[1:M + 1, :hidden]      # strided rows
-    gain = (1.0 + rnd(hidden, seed=61)).to(gain_dt).cuda()
+    gain = (1.0 + rnd(hidden, seed=61)).to(torch.bfloat16).cuda()
+    assert not k.gemm_normed_ok(M, ffn, hidden, gated=True, gain=gain.float())          # the gain as it is stored: bfloat16
     w, _ = as_dtype(rnd(2 * ffn, hidden, seed=62, scale=0.2), "bfloat16")
     ww = k.pack_matrix(w)
     x = torch.empty(M, hidden, dtype=torch.bfloat16, device="cuda")
@@ -364,10 +365,12 @@ def test_gated_product_with_the_norm_inside(M, hidden, ffn, gain_dt):
     k.gemm_normed_glu(rows, gain, 1e-5, ww, got[:M, :ffn])
     assert torch.equal(got[:M, :ffn], want)
     assert (got[M] == 7.0).all() and (got[:, ffn:] == 7.0).all()
+    with pytest.raises(KernelError):
+        k.gemm_normed_glu(rows, gain.float(), 1e-5, ww, got[:M, :ffn])
 
 
-@pytest.mark.parametrize("M,nh,nkv,hd,hidden,page", [(1, 4, 2, 32, 64, 8), (8, 28, 4, 128, 3584, 64), (6, 7, 1, 128, 256, 8),
-                                                      (7, 3, 3, 96, 128, 4), (5, 4, 1, 64, 320, 32), (3, 14, 2, 64, 896, 16)])
+@pytest.mark.parametrize("M,nh,nkv,hd,hidden,page", [(1, 4, 2, 32, 256, 8), (8, 28, 4, 128, 3584, 64), (6, 7, 1, 128, 256, 8),
+                                                      (7, 3, 3, 96, 512, 4), (5, 4, 1, 64, 768, 32), (3, 14, 2, 64, 1024, 16)])
 def test_qkv_product_with_the_norm_inside(M, nh, nkv, hd, hidden, page):
     """As above for the [q; k; v] product with rotation and cache store: the same bits in q and in
     the pages as the norm kernel followed by `gemm_qkv_rope`."""
