@@ -980,16 +980,17 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
   static_assert(!ROPE || UNITS == 1, "one head half-pair a wave");
   static_assert(MPAD == 8, "rows of X in LDS: half a tile of 16, lanes of rows 8 .. 15 read rows 0 .. 7 again");
   extern __shared__ __align__(16) unsigned char x_lds[];        // X, then the segments' sums [wave][tile][lane][4]
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int nw = (blockDim.x >> 6) - NORMED_NORM_WAVES;         // streaming waves
+  // the norming waves are the block's first: they are at work before the others have started
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) - NORMED_NORM_WAVES;
+  const int nw = (blockDim.x >> 6) - NORMED_NORM_WAVES;         // streaming waves: 0 .. nw - 1
   const int KB = K / 32;
 
-  if (wave >= nw) {
+  if (wave < 0) {
     // ------------------------------------------------------------------ a norming wave: rows w, w + 4, ..., two at a time
     // A row is `full` rounds of 64 float4 (K a multiple of 256); lane l holds the float4 l + 64 j.
     // In LDS that is block (l >> 3) + 8 j of X, chunk (l & 7) >> 1, half l & 1: one address a lane
     // and row, 8 blocks further for every j.
-    const int full = K >> 8, first_row = wave - nw;
+    const int full = K >> 8, first_row = wave + NORMED_NORM_WAVES;
     int ln = lane;
     asm volatile("" : "+v"(ln));        // what follows from the lane is worked out here, not kept in registers from the start
     uint2 gain_bf[KC];                                          // the gain (bfloat16): the lane's share, asked for with the rows
