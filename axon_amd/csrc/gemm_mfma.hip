@@ -993,12 +993,7 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
     const int full = K >> 8, first_row = wave + NORMED_NORM_WAVES;
     int ln = lane;
     asm volatile("" : "+v"(ln));        // what follows from the lane is worked out here, not kept in registers from the start
-    uint2 gain_bf[KC];                                          // the gain (bfloat16): the lane's share, asked for with the rows
-    if (first_row < M) {
-#pragma unroll
-      for (int j = 0; j < KC; ++j)
-        if (j < full) gain_bf[j] = *reinterpret_cast<const uint2*>((const bf16_t*)in.gain + 4 * (ln + 64 * j));
-    }
+    uint2 gain_bf[KC];                                          // the gain (bfloat16): the lane's share, asked for behind the rows
     const int q = (ln & 7) >> 1;
     const unsigned swz = (q + 4 * ((ln >> 3) & 1)) & 7;           // slots of 16 bytes (a row's 8 k) are permuted within
     unsigned char* at0 = x_lds + (ln >> 3) * XBLOCK + (ln & 1) * 8;   // eights, by chunk and block parity: these stores,
@@ -1021,6 +1016,9 @@ gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __re
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+#pragma unroll
+        for (int j = 0; j < KC; ++j)
+          if (j < full) gain_bf[j] = *reinterpret_cast<const uint2*>((const bf16_t*)in.gain + 4 * (ln + 64 * j));
       }
       // four chains a row as the norm kernel's four waves have them, then their butterflies, all
       // eight side by side
