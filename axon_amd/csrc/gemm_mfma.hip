@@ -26,7 +26,7 @@
 //   Epilogues: bias / residual add / SwiGLU, and the attention's qkv product with the rotary
 //   encoding and the store into the paged cache.
 //
-// * gemm_normed (M <= 8, the operand an RMS norm of float32 rows): gemm_stream's product with the
+// * gemm_normed (M <= 16, the operand an RMS norm of float32 rows): gemm_stream's product with the
 //   norm inside; waves of their own norm the rows into LDS while the streaming waves fill their
 //   rings, so the norm is no launch of its own in a decoding step.
 //
@@ -967,18 +967,17 @@ struct NormedRows {
 #define NORMED_KC 16            // float4 of a row a lane holds: K <= 256 * 16
 
 // UNITS: pairs of row tiles a streaming wave
-#define NORMED_MAX_M 8          // with more rows the norm takes longer than it saves (measured)
+#define NORMED_MAX_M 16
 
-template <int UNITS, int SEGS, int DEPTH, int EPI>
+template <int UNITS, int SEGS, int DEPTH, int EPI, int MPAD>
 __global__ void __launch_bounds__((NORMED_STREAM_WAVES + NORMED_NORM_WAVES) * 64, 1)
 gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __restrict__ bias, int bias_is_f32,
                    void* __restrict__ out, int out_stride, int M, int N, int K, int mode, RopeStore rope, int n_units) {
   constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE;
-  constexpr int MPAD = NORMED_MAX_M;
   constexpr int NT = 2 * UNITS, XBLOCK = MPAD * 64, KC = NORMED_KC;   // XBLOCK: bytes of MPAD rows x 32 k of X
   static_assert(GLU || ROPE, "the paired epilogues");
   static_assert(!ROPE || UNITS == 1, "one head half-pair a wave");
-  static_assert(MPAD == 8, "rows of X in LDS: half a tile of 16, lanes of rows 8 .. 15 read rows 0 .. 7 again");
+  static_assert(MPAD == 8 || MPAD == 16, "rows of X in LDS: a tile of 16, or half of one (lanes of rows 8 .. 15 then read rows 0 .. 7 again)");
   extern __shared__ __align__(16) unsigned char x_lds[];        // X, then the segments' sums [wave][tile][lane][4]
   // the norming waves are the block's first: they are at work before the others have started
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) - NORMED_NORM_WAVES;
@@ -1224,7 +1223,7 @@ static NormedShape normed_shape(int units, int segs, bool gated) {
 // a lane holds a row's share in registers.
 int gemm_normed_ok(int m, int k) {
   if (m < 1 || m > NORMED_MAX_M || k % 256 != 0 || k > 256 * NORMED_KC) return 0;     // whole rounds of 64 float4 a row
-  return (size_t)(k / 32) * NORMED_MAX_M * 64 + NORMED_STREAM_WAVES * 6 * 1024 <= NORMED_MAX_LDS;
+  return (size_t)(k / 32) * (m <= 8 ? 8 : 16) * 64 + NORMED_STREAM_WAVES * 6 * 1024 <= NORMED_MAX_LDS;
 }
 
 template <int UNITS, int SEGS, int EPI>
@@ -1232,10 +1231,10 @@ static int launch_normed_of(const NormedRows& in, const bf16_t* w, const void* b
                             int m, int n, int k, int mode, hipStream_t stream, const RopeStore& rope, int units,
                             const NormedShape& shape) {
   const int nw = shape.groups * SEGS;
-  const size_t lds = (size_t)(k / 32) * NORMED_MAX_M * 64 + (SEGS > 1 ? (size_t)nw * 2 * UNITS * 1024 : 0);
-#define NORMED_LAUNCH()                                                                                               \
+  const size_t lds = (size_t)(k / 32) * (m <= 8 ? 8 : 16) * 64 + (SEGS > 1 ? (size_t)nw * 2 * UNITS * 1024 : 0);
+#define NORMED_LAUNCH(MPAD)                                                                                           \
   {                                                                                                                   \
-    auto kernel = &gemm_normed_kernel<UNITS, SEGS, UNITS == 1 ? 8 : UNITS == 2 ? 4 : 3, EPI>;                         \
+    auto kernel = &gemm_normed_kernel<UNITS, SEGS, UNITS == 1 ? 8 : UNITS == 2 ? 4 : 3, EPI, MPAD>;                   \
     static bool configured = false;                                                                                   \
     if (!configured) {                                                                                                \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
@@ -1249,7 +1248,7 @@ static int launch_normed_of(const NormedRows& in, const bf16_t* w, const void* b
     kernel<<<shape.blocks, (nw + NORMED_NORM_WAVES) * 64, lds, stream>>>(in, w, bias, bias_is_f32, out, out_stride, m, n, k, \
                                                                          mode, rope, units);                          \
   }
-  NORMED_LAUNCH()
+  if (m <= 8) NORMED_LAUNCH(8) else NORMED_LAUNCH(16)
 #undef NORMED_LAUNCH
   AXK_LAUNCH_CHECK("gemm_normed");
   return 0;
