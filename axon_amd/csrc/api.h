@@ -142,8 +142,8 @@ int axk_gemm_qkv_rope(const void* x, int x_stride, const void* w, const void* bi
 // the packed [gate; up] matrix) and the [q; k; v] product (as axk_gemm_qkv_rope) with the RMS norm
 // of their operand inside: X = axk_rmsnorm(rows, gain, eps) is worked out in the kernel's own LDS
 // and never stored.  Bit-identical to axk_rmsnorm followed by axk_gemm / axk_gemm_qkv_rope.
-// axk_gemm_normed_ok(m, n, k, gated): whether these sizes are taken (up to 16 rows, K a multiple of
-// 256 up to 4,096, X within LDS); the gain must be bfloat16 (gain_is_f32 = 0).
+// axk_gemm_normed_ok(m, n, k, gated): whether these sizes are taken (up to 16 rows of a multiple of 256
+// up to 4,096 columns, up to 8 rows of up to 5,120); the gain must be bfloat16 (gain_is_f32 = 0).
 int axk_gemm_normed_ok(int m, int n, int k, int gated);
 int axk_gemm_normed_glu(const float* rows, int rows_stride, const void* gain, int gain_is_f32, float eps, const void* w,
                         void* out, int out_stride, int m, int n, int k, void* stream);

@@ -964,17 +964,17 @@ struct NormedRows {
 #define NORMED_MAX_LDS (152 * 1024)
 #define NORMED_STREAM_WAVES 4   // at most
 #define NORMED_NORM_WAVES 4
-#define NORMED_KC 16            // float4 of a row a lane holds: K <= 256 * 16
+#define NORMED_MAX_KC 20        // float4 of a row a lane holds at most: K <= 256 * 20
 
 // UNITS: pairs of row tiles a streaming wave
 #define NORMED_MAX_M 16
 
-template <int UNITS, int SEGS, int DEPTH, int EPI, int MPAD>
+template <int UNITS, int SEGS, int DEPTH, int EPI, int MPAD, int KC>
 __global__ void __launch_bounds__((NORMED_STREAM_WAVES + NORMED_NORM_WAVES) * 64, 1)
 gemm_normed_kernel(NormedRows in, const bf16_t* __restrict__ w, const void* __restrict__ bias, int bias_is_f32,
                    void* __restrict__ out, int out_stride, int M, int N, int K, int mode, RopeStore rope, int n_units) {
   constexpr bool GLU = EPI == EPI_GLU, ROPE = EPI == EPI_ROPE;
-  constexpr int NT = 2 * UNITS, XBLOCK = MPAD * 64, KC = NORMED_KC;   // XBLOCK: bytes of MPAD rows x 32 k of X
+  constexpr int NT = 2 * UNITS, XBLOCK = MPAD * 64;             // XBLOCK: bytes of MPAD rows x 32 k of X
   static_assert(GLU || ROPE, "the paired epilogues");
   static_assert(!ROPE || UNITS == 1, "one head half-pair a wave");
   static_assert(MPAD == 8 || MPAD == 16, "rows of X in LDS: a tile of 16, or half of one (lanes of rows 8 .. 15 then read rows 0 .. 7 again)");
@@ -1222,7 +1222,8 @@ static NormedShape normed_shape(int units, int segs, bool gated) {
 // Whether a product of m rows of width k takes the norm inside: X (and the segments' sums) fit LDS,
 // a lane holds a row's share in registers.
 int gemm_normed_ok(int m, int k) {
-  if (m < 1 || m > NORMED_MAX_M || k % 256 != 0 || k > 256 * NORMED_KC) return 0;     // whole rounds of 64 float4 a row
+  if (m < 1 || m > NORMED_MAX_M || k % 256 != 0 || k > 256 * NORMED_MAX_KC) return 0;     // whole rounds of 64 float4 a row
+  if (k > 256 * 16 && m > 8) return 0;
   return (size_t)(k / 32) * (m <= 8 ? 8 : 16) * 64 + NORMED_STREAM_WAVES * 6 * 1024 <= NORMED_MAX_LDS;
 }
 
@@ -1232,9 +1233,9 @@ static int launch_normed_of(const NormedRows& in, const bf16_t* w, const void* b
                             const NormedShape& shape) {
   const int nw = shape.groups * SEGS;
   const size_t lds = (size_t)(k / 32) * (m <= 8 ? 8 : 16) * 64 + (SEGS > 1 ? (size_t)nw * 2 * UNITS * 1024 : 0);
-#define NORMED_LAUNCH(MPAD)                                                                                           \
+#define NORMED_LAUNCH(MPAD, KCV)                                                                                         \
   {                                                                                                                   \
-    auto kernel = &gemm_normed_kernel<UNITS, SEGS, UNITS == 1 ? 8 : UNITS == 2 ? 4 : 3, EPI, MPAD>;                   \
+    auto kernel = &gemm_normed_kernel<UNITS, SEGS, UNITS == 1 ? 8 : UNITS == 2 ? 4 : 3, EPI, MPAD, KCV>;              \
     static bool configured = false;                                                                                   \
     if (!configured) {                                                                                                \
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
@@ -1248,7 +1249,7 @@ static int launch_normed_of(const NormedRows& in, const bf16_t* w, const void* b
     kernel<<<shape.blocks, (nw + NORMED_NORM_WAVES) * 64, lds, stream>>>(in, w, bias, bias_is_f32, out, out_stride, m, n, k, \
                                                                          mode, rope, units);                          \
   }
-  if (m <= 8) NORMED_LAUNCH(8) else NORMED_LAUNCH(16)
+  if (k > 256 * 16) NORMED_LAUNCH(8, NORMED_MAX_KC) else if (m <= 8) NORMED_LAUNCH(8, 16) else NORMED_LAUNCH(16, 16)
 #undef NORMED_LAUNCH
   AXK_LAUNCH_CHECK("gemm_normed");
   return 0;

@@ -344,13 +344,14 @@ def test_qkv_product_with_rotation_and_cache_store_in_one(M, nh, nkv, hd, hidden
 
 @pytest.mark.parametrize("M,hidden,ffn", [(1, 256, 32), (8, 3584, 4864), (3, 768, 320), (8, 256, 9600), (7, 1024, 8192),
                                           (8, 4096, 256), (5, 512, 4864), (2, 3584, 2368), (6, 3584, 18944), (9, 3584, 4864), (13, 768, 1280),
-                                          (16, 3584, 2368), (16, 256, 9600), (15, 4096, 640)])
+                                          (16, 3584, 2368), (16, 256, 9600), (15, 4096, 640), (8, 5120, 1728), (3, 4352, 320)])
 def test_gated_product_with_the_norm_inside(M, hidden, ffn):
     """The norm worked out inside the product against the norm kernel followed by the product: the
     same bits (the norm is the norm kernel's arithmetic, the product's order of addition the same)."""
     k = kernels("bfloat16")
     assert k.gemm_normed_ok(M, ffn, hidden, gated=True)
     assert not k.gemm_normed_ok(17, ffn, hidden, gated=True) and not k.gemm_normed_ok(M, ffn, 8192, gated=True)
+    assert k.gemm_normed_ok(8, ffn, 5120, gated=True) and not k.gemm_normed_ok(9, ffn, 5120, gated=True)   # wide rows: up to 8 of them
     assert not k.gemm_normed_ok(M, ffn, hidden + 64, gated=True)          # rows in whole rounds of 256 columns
     assert not kernels("float32").gemm_normed_ok(M, ffn, hidden, gated=True)
     rows = (rnd(M + 2, hidden + 8, seed=60) * 3.0).float().cuda()[1:M + 1, :hidden]      # strided rows
@@ -372,7 +373,7 @@ def test_gated_product_with_the_norm_inside(M, hidden, ffn):
 
 @pytest.mark.parametrize("M,nh,nkv,hd,hidden,page", [(1, 4, 2, 32, 256, 8), (8, 28, 4, 128, 3584, 64), (6, 7, 1, 128, 256, 8),
                                                       (7, 3, 3, 96, 512, 4), (5, 4, 1, 64, 768, 32), (3, 14, 2, 64, 1024, 16),
-                                                      (12, 28, 4, 128, 3584, 64), (16, 6, 2, 64, 512, 16)])
+                                                      (12, 28, 4, 128, 3584, 64), (16, 6, 2, 64, 512, 16), (8, 40, 8, 128, 5120, 64)])
 def test_qkv_product_with_the_norm_inside(M, nh, nkv, hd, hidden, page):
     """As above for the [q; k; v] product with rotation and cache store: the same bits in q and in
     the pages as the norm kernel followed by `gemm_qkv_rope`."""
