@@ -56,7 +56,7 @@ def test_cache_rows_are_the_same_bits_however_the_tokens_were_fed(name, dtype, m
 
 @pytest.mark.parametrize("name", ["E"])
 def test_a_norm_inside_the_product_after_it_changes_no_bit(name, model_dirs, monkeypatch):
-    """Steps of up to eight tokens hand their norms to the product after them (the [q; k; v] product
+    """Steps of up to sixteen tokens hand their norms to the product after them (the [q; k; v] product
     and the gated product norm their operand on the way; model E's width, a multiple of 256, is one
     that kernel takes): logits and cache rows are those of the same steps with every norm a pass of
     its own, and the kernel did run."""
@@ -71,6 +71,7 @@ def test_a_norm_inside_the_product_after_it_changes_no_bit(name, model_dirs, mon
         out.append(eng.step([StepEntry("a", a[70:73], [0, 2]), StepEntry("b", b[30:35], [4])]))      # 8 tokens
         for t in range(73, 84):                                                                 # 1 or 2 tokens
             out.append(eng.step([StepEntry("a", a[t:t + 1], [0])] + ([StepEntry("b", b[t - 38:t - 37], [0])] if t % 3 else [])))
+        out.append(eng.step([StepEntry("a", a[84:90], [5]), StepEntry("b", b[46:53], [0, 6])]))     # 13 tokens
         return torch.cat([o.clone() for o in out]), cache_rows(eng, "a")
 
     calls = []
@@ -80,7 +81,7 @@ def test_a_norm_inside_the_product_after_it_changes_no_bit(name, model_dirs, mon
     monkeypatch.setattr(k, "gemm_normed_glu", lambda *a_, **kw: (calls.append("glu"), glu(*a_, **kw))[1])
     monkeypatch.setattr(k, "gemm_normed_qkv_rope", lambda *a_, **kw: (calls.append("qkv"), qkv(*a_, **kw))[1])
     got, got_rows = run(inside)
-    assert calls.count("glu") >= 12 and calls.count("qkv") >= 12
+    assert calls.count("glu") >= 13 and calls.count("qkv") >= 13
     monkeypatch.setattr(GQAttention, "applies_preceding_norm", lambda self, ctx: False)
     monkeypatch.setattr(SwiGLUMLP, "applies_preceding_norm", lambda self, ctx: False)
     calls.clear()
