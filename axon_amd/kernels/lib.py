@@ -131,7 +131,9 @@ class Kernels:
 
     # what launches kernels: wrapped while a step is profiled
     _LAUNCHING = ("embed", "rmsnorm", "rope_table", "rope_kv_write", "gemm_qkv_rope", "attention", "attention_prefill",
-                  "attention_decode", "gemm", "swiglu", "argmax", "topk", "fill_i32", "fill_f32")
+                  "attention_decode", "gemm", "gemm_normed_glu", "gemm_normed_qkv_rope", "swiglu", "argmax", "topk",
+                  "fill_i32", "fill_f32")
+    _MATRIX_AT = {"gemm": 1, "gemm_qkv_rope": 1, "gemm_normed_glu": 3, "gemm_normed_qkv_rope": 3}   # which argument is W
 
     def set_launch_hook(self, hook) -> None:
         """`hook(name, matrix_bytes)` is told of every call that has launched kernels, with the
@@ -147,8 +149,8 @@ class Kernels:
             def told(*a, _plain=plain, _name=name, **kw):
                 out = _plain(self, *a, **kw)
                 label, nbytes = _name, 0
-                if _name in ("gemm", "gemm_qkv_rope"):
-                    w = a[1]
+                if _name in self._MATRIX_AT:
+                    w = a[self._MATRIX_AT[_name]]
                     data = w.data if isinstance(w, PackedMatrix) else w
                     nbytes = data.numel() * data.element_size()
                     label = f"{_name} {w.shape[0]}x{w.shape[1]}"
