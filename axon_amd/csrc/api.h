@@ -174,11 +174,14 @@ int axk_argmax_static_max_n(void);
 int axk_argmax_static(const float* logits, int logits_stride, int32_t* picks, int n_rows, int n, void* stream);
 
 // Repeat penalty on `recent` ids, then the k best as 64-bit keys (order key of the logit <<
-// 32 | id), unsorted, into cands[r, 0..k); the penalty is applied to `logits` in place.  recent is [n_rows, recent_stride] with
-// n_recent[r] valid ids each; penalty 1 or n_recent 0: off.  k <= 1024.
+// 32 | id), unsorted, into cands[r, 0..k); the penalty is applied to `logits` in place.  recent is
+// [n_rows, recent_stride] with n_recent[r] valid ids each; penalty 1 or n_recent 0: off.
+// k <= cands_stride.  workspace: axk_topk_workspace(n_rows, n, cands_stride) bytes, 8-byte aligned
+// (the k best of every slice of a row, of which a second launch takes the k best).
+long axk_topk_workspace(int n_rows, int n, int cands_stride);
 int axk_topk(float* logits, int logits_stride, const int32_t* recent, int recent_stride,
              const int32_t* n_recent, const float* penalty, const int32_t* k_of_row, uint64_t* cands,
-             int cands_stride, int n_rows, int n, void* stream);
+             int cands_stride, int n_rows, int n, void* workspace, void* stream);
 
 // dst[i] = value for i < n (a fill that may be captured into a graph).
 int axk_fill_i32(int32_t* dst, int32_t value, int n, void* stream);

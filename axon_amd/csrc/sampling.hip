@@ -106,90 +106,174 @@ extern "C" int axk_argmax(const float* logits, int logits_stride, int32_t* picks
 }
 
 // ---------------------------------------------------------------------------- candidates
-// One block per row.  (1) llama.cpp's repeat penalty on the distinct ids of the row's recent
-// window, in place: a positive logit is divided by p, any other multiplied
-// (src/sample.rs:307-326).  (2) An 8-pass radix select on the 64-bit keys finds the k-th
-// largest key exactly.  (3) Every key at or above it is appended to the row's candidates:
-// exactly k of them, in no particular order (the host sorts k pairs).
-__global__ void __launch_bounds__(PICK_THREADS)
-topk_kernel(float* __restrict__ logits, int stride, const int32_t* __restrict__ recent, int recent_stride,
-            const int32_t* __restrict__ n_recent, const float* __restrict__ penalty,
-            const int32_t* __restrict__ k_of_row, uint64_t* __restrict__ cands, int cands_stride, int n) {
-  __shared__ int hist[256];
-  __shared__ int s_digit, s_remaining, s_count;
-  const int r = blockIdx.x;
-  float* row = logits + (size_t)r * stride;
-  int k = k_of_row[r];
-  if (k <= 0) return;
-  if (k > n) k = n;
+// (1) llama.cpp's repeat penalty on the distinct ids of the row's recent window, in place: a
+// positive logit is divided by p, any other multiplied (src/sample.rs:307-326).  (2) The k
+// largest of the row's 64-bit keys, exactly, in no particular order (the host sorts k pairs).
+// Two launches: blocks of 256 threads each take a slice of TOPK_SLICE logits of one row into LDS,
+// apply the penalty to the ids that lie in it and leave the slice's own k largest keys (the k
+// largest of the row are among them); then one block per row takes the k largest of those.  A
+// selection is an 8-pass radix select on the keys: integer histograms only, no step that depends
+// on an order.
+#define TOPK_SLICE 4096
+#define TOPK_THREADS 256
+#define TOPK_MERGE_THREADS 1024
 
+// The k-th largest (k >= 1) of the distinct keys key_at(i), i < count, of which at least k are
+// valid (key_at returns false for a place without a key).  Every thread of the block calls it
+// and gets the same value.  hist: 256 ints of LDS, vars: 2 ints of LDS; blocks of at least 256 threads.
+template <class KeyAt>
+__device__ inline uint64_t kth_largest_key(KeyAt key_at, int count, int k, int* hist, int* vars) {
+  __shared__ int wave_total[256 / AXON_WAVE];
+  uint64_t prefix = 0, mask = 0;
+  if (threadIdx.x == 0) vars[0] = k;                   // keys still wanted among those that match the prefix
+  for (int pass = 7; pass >= 0; --pass) {
+    const int shift = pass * 8;
+    for (int b = threadIdx.x; b < 256; b += blockDim.x) hist[b] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < count; i += blockDim.x) {
+      uint64_t key;
+      if (key_at(i, key) && (key & mask) == prefix) atomicAdd(&hist[(int)((key >> shift) & 255u)], 1);
+    }
+    __syncthreads();
+    // the digit whose bin holds the k-th largest: thread t owns bin 255 - t, counts the keys in the
+    // bins above its own (a scan over the threads: within each wave, then the waves before it) and
+    // the one thread whose bin the count crosses in says so
+    const int remaining = vars[0];
+    int mine = 0, upto = 0;
+    if (threadIdx.x < 256) {
+      mine = hist[255 - threadIdx.x];
+      upto = mine;
+      const int lane = threadIdx.x & (AXON_WAVE - 1);
+#pragma unroll
+      for (int off = 1; off < AXON_WAVE; off <<= 1) {
+        const int other = __shfl_up(upto, off, AXON_WAVE);
+        if (lane >= off) upto += other;
+      }
+      if (lane == AXON_WAVE - 1) wave_total[threadIdx.x / AXON_WAVE] = upto;
+    }
+    __syncthreads();
+    if (threadIdx.x < 256) {
+      for (int w = 0; w < (int)threadIdx.x / AXON_WAVE; ++w) upto += wave_total[w];
+      const int above = upto - mine;
+      if (above < remaining && upto >= remaining) {
+        vars[1] = 255 - threadIdx.x;
+        vars[0] = remaining - above;
+      }
+    }
+    __syncthreads();
+    prefix |= (uint64_t)vars[1] << shift;
+    mask |= (uint64_t)255u << shift;
+  }
+  __syncthreads();
+  return prefix;
+}
+
+// grid (slices, rows).  slice_keys [rows][slices][k_stride], slice_count [rows][slices].
+__global__ void __launch_bounds__(TOPK_THREADS)
+topk_slice_kernel(float* __restrict__ logits, int stride, const int32_t* __restrict__ recent, int recent_stride,
+                  const int32_t* __restrict__ n_recent, const float* __restrict__ penalty,
+                  const int32_t* __restrict__ k_of_row, uint64_t* __restrict__ slice_keys,
+                  int32_t* __restrict__ slice_count, int k_stride, int n) {
+  __shared__ float vals[TOPK_SLICE];
+  __shared__ int hist[256];
+  __shared__ int vars[2], s_count;
+  const int r = blockIdx.y, s = blockIdx.x, slices = gridDim.x;
+  const int lo = s * TOPK_SLICE, count = min(n - lo, TOPK_SLICE);
+  float* row = logits + (size_t)r * stride;
+  int k = min(k_of_row[r], n);
+  if (k <= 0) return;
+  for (int i = threadIdx.x; i < count; i += TOPK_THREADS) vals[i] = row[lo + i];
+  __syncthreads();
   const float p = penalty[r];
   const int nr = n_recent[r];
   if (p != 1.0f && nr > 0) {
     const int32_t* rec = recent + (size_t)r * recent_stride;
-    for (int j = threadIdx.x; j < nr; j += PICK_THREADS) {
+    for (int j = threadIdx.x; j < nr; j += TOPK_THREADS) {
       const int id = rec[j];
-      bool first = id >= 0 && id < n;
+      bool first = id >= lo && id < lo + count;         // the ids of this slice, each once
       for (int e = 0; e < j && first; ++e) first = rec[e] != id;
       if (first) {
-        const float v = row[id];
-        row[id] = v > 0.0f ? v / p : v * p;
+        const float v = vals[id - lo];
+        const float w = v > 0.0f ? v / p : v * p;
+        vals[id - lo] = w;
+        row[id] = w;
       }
     }
     __syncthreads();
   }
-
-  uint64_t prefix = 0, mask = 0;
-  if (threadIdx.x == 0) s_remaining = k;
-  for (int pass = 7; pass >= 0; --pass) {
-    const int shift = pass * 8;
-    if (threadIdx.x < 256) hist[threadIdx.x] = 0;
-    __syncthreads();
-    for (int i = threadIdx.x; i < n; i += PICK_THREADS) {
-      const uint64_t key = key64(row[i], i);
-      if ((key & mask) == prefix) atomicAdd(&hist[(int)((key >> shift) & 255u)], 1);
+  k = min(k, count);
+  auto key_at = [&](int i, uint64_t& key) {
+    key = key64(vals[i], lo + i);
+    return true;
+  };
+  const uint64_t least = k == count ? 0 : kth_largest_key(key_at, count, k, hist, vars);
+  if (threadIdx.x == 0) s_count = 0;
+  __syncthreads();
+  uint64_t* dst = slice_keys + ((size_t)r * slices + s) * k_stride;
+  for (int i = threadIdx.x; i < count; i += TOPK_THREADS) {
+    const uint64_t key = key64(vals[i], lo + i);
+    if (key >= least) {
+      const int at = atomicAdd(&s_count, 1);
+      if (at < k) dst[at] = key;
     }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      int acc = 0, digit = 0;
-      const int remaining = s_remaining;
-      for (int b = 255; b >= 0; --b) {
-        if (acc + hist[b] >= remaining) {
-          digit = b;
-          break;
-        }
-        acc += hist[b];
-      }
-      s_digit = digit;
-      s_remaining = remaining - acc;
-    }
-    __syncthreads();
-    prefix |= (uint64_t)s_digit << shift;
-    mask |= (uint64_t)255u << shift;
   }
+  if (threadIdx.x == 0) slice_count[r * slices + s] = k;
+}
 
+// One block per row: the k largest of the slices' keys.
+__global__ void __launch_bounds__(TOPK_MERGE_THREADS)
+topk_merge_kernel(const uint64_t* __restrict__ slice_keys, const int32_t* __restrict__ slice_count, int slices, int k_stride,
+                  const int32_t* __restrict__ k_of_row, uint64_t* __restrict__ cands, int cands_stride, int n) {
+  __shared__ int hist[256];
+  __shared__ int vars[2], s_count;
+  const int r = blockIdx.x;
+  const int k = min(k_of_row[r], n);
+  if (k <= 0) return;
+  const uint64_t* keys = slice_keys + (size_t)r * slices * k_stride;
+  const int32_t* counts = slice_count + r * slices;
+  const int places = slices * k_stride;
+  auto key_at = [&](int i, uint64_t& key) {
+    if (i % k_stride >= counts[i / k_stride]) return false;
+    key = keys[i];
+    return true;
+  };
+  const uint64_t least = kth_largest_key(key_at, places, k, hist, vars);
   if (threadIdx.x == 0) s_count = 0;
   __syncthreads();
   uint64_t* dst = cands + (size_t)r * cands_stride;
-  for (int i = threadIdx.x; i < n; i += PICK_THREADS) {
-    const uint64_t key = key64(row[i], i);
-    if (key >= prefix) {
+  for (int i = threadIdx.x; i < places; i += TOPK_MERGE_THREADS) {
+    uint64_t key;
+    if (key_at(i, key) && key >= least) {
       const int at = atomicAdd(&s_count, 1);
       if (at < k) dst[at] = key;
     }
   }
 }
 
+extern "C" long axk_topk_workspace(int n_rows, int n, int k_stride) {
+  if (n_rows <= 0 || n <= 0 || k_stride <= 0) return 0;
+  const long slices = ceil_div(n, TOPK_SLICE);
+  return (long)n_rows * slices * ((long)k_stride * 8 + 8);       // the slices' keys, then their counts (8-byte places)
+}
+
 extern "C" int axk_topk(float* logits, int logits_stride, const int32_t* recent, int recent_stride,
                         const int32_t* n_recent, const float* penalty, const int32_t* k_of_row, uint64_t* cands,
-                        int cands_stride, int n_rows, int n, void* stream) {
+                        int cands_stride, int n_rows, int n, void* workspace, void* stream) {
   AXK_REQUIRE(n_rows >= 0 && n > 0 && logits_stride >= n, "topk: bad sizes rows=%d n=%d stride=%d", n_rows, n,
               logits_stride);
   AXK_REQUIRE(cands_stride >= 1, "topk: candidate stride %d", cands_stride);
+  AXK_REQUIRE(n_rows <= 65535, "topk: %d rows are more than one launch takes", n_rows);
+  AXK_REQUIRE(workspace != nullptr && ((uintptr_t)workspace & 7) == 0, "topk: needs its workspace, 8-byte aligned");
   if (n_rows == 0) return 0;
-  topk_kernel<<<n_rows, PICK_THREADS, 0, (hipStream_t)stream>>>(logits, logits_stride, recent, recent_stride,
-                                                               n_recent, penalty, k_of_row, cands, cands_stride, n);
-  AXK_LAUNCH_CHECK("topk");
+  const int slices = ceil_div(n, TOPK_SLICE);
+  uint64_t* slice_keys = (uint64_t*)workspace;
+  int32_t* slice_count = (int32_t*)(slice_keys + (size_t)n_rows * slices * cands_stride);
+  topk_slice_kernel<<<dim3(slices, n_rows), TOPK_THREADS, 0, (hipStream_t)stream>>>(
+      logits, logits_stride, recent, recent_stride, n_recent, penalty, k_of_row, slice_keys, slice_count, cands_stride, n);
+  AXK_LAUNCH_CHECK("topk_slice");
+  topk_merge_kernel<<<n_rows, TOPK_MERGE_THREADS, 0, (hipStream_t)stream>>>(slice_keys, slice_count, slices, cands_stride,
+                                                                           k_of_row, cands, cands_stride, n);
+  AXK_LAUNCH_CHECK("topk_merge");
   return 0;
 }
 

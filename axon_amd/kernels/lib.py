@@ -65,7 +65,8 @@ _SIGNATURES = {
     "axk_swiglu": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_argmax": [c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p],
     "axk_topk": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                 c_void_p],
+                 c_void_p, c_void_p],
+    "axk_topk_workspace": [c_int, c_int, c_int],
     "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
     "axk_fill_f32": [c_void_p, c_float, c_int, c_void_p],
 }
@@ -119,6 +120,7 @@ class Kernels:
         self.lib.axk_packed_elems.restype = ctypes.c_long
         self.lib.axk_gemm_workspace.argtypes = [c_int, c_int, c_int, c_int]
         self.lib.axk_gemm_workspace.restype = ctypes.c_long
+        self.lib.axk_topk_workspace.restype = ctypes.c_long
         self.lib.axk_argmax_workspace.argtypes = [c_int, c_int]
         self.lib.axk_argmax_workspace.restype = ctypes.c_long
         if bool(self.lib.axk_is_bf16()) != (dtype_name == "bfloat16"):
@@ -535,17 +537,24 @@ class Kernels:
         self._check(self.lib.axk_argmax(_ptr(logits), logits.stride(0), _ptr(out), rows, n, _ptr(work), _stream()))
         return out
 
-    def topk(self, logits, recent, n_recent, penalty, k_of_row, cands) -> torch.Tensor:
+    def topk(self, logits, recent, n_recent, penalty, k_of_row, cands, k_max: Optional[int] = None) -> torch.Tensor:
+        """`k_max`: the largest of k_of_row, where the caller knows it (else it is read back from
+        the device, which waits for it)."""
         self._i32(recent, "topk recent"); self._i32(n_recent, "topk n_recent"); self._i32(k_of_row, "topk k")
         self._f32(penalty, "topk penalty")
         rows, n = logits.shape
         if (logits.dtype != torch.float32 or not logits.is_cuda or logits.stride(1) != 1 or cands.dtype != torch.int64
                 or cands.shape[0] != rows or not cands.is_contiguous() or recent.shape[0] != rows):
             raise KernelError(f"topk: logits {tuple(logits.shape)} cands {tuple(cands.shape)} {cands.dtype}")
-        if int(k_of_row.max()) > cands.shape[1]:
-            raise KernelError(f"topk: k up to {int(k_of_row.max())} for {cands.shape[1]} candidate places")
+        if k_max is None:
+            k_max = int(k_of_row.max())
+        if k_max > cands.shape[1]:
+            raise KernelError(f"topk: k up to {k_max} for {cands.shape[1]} candidate places")
+        need = self.lib.axk_topk_workspace(rows, n, cands.shape[1])
+        work = torch.empty(max(need, 8) // 8, dtype=torch.int64, device=logits.device)
         self._check(self.lib.axk_topk(_ptr(logits), logits.stride(0), _ptr(recent), recent.shape[1], _ptr(n_recent),
-                                      _ptr(penalty), _ptr(k_of_row), _ptr(cands), cands.shape[1], rows, n, _stream()))
+                                      _ptr(penalty), _ptr(k_of_row), _ptr(cands), cands.shape[1], rows, n, _ptr(work),
+                                      _stream()))
         return cands
 
     def fill_i32(self, dst: torch.Tensor, value: int) -> None:

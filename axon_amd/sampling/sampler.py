@@ -149,7 +149,7 @@ def pick_rows(rt, logits: torch.Tensor, samplers: Sequence[Optional[Sampler]],
         sel = logits if n == rows else logits[torch.tensor(device_rows, device=dev)].contiguous()
         cands = torch.zeros((n, max(ks)), dtype=torch.int64, device=dev)
         rt.k.topk(sel, on[:n * width].view(n, width), on[n * width:n * width + n], on[n * width + 2 * n:].view(torch.float32),
-                  on[n * width + n:n * width + 2 * n], cands)
+                  on[n * width + n:n * width + 2 * n], cands, k_max=max(ks))
         host = cands.cpu()
         for i, r in enumerate(device_rows):
             picks[r] = samplers[r].pick_keys(host[i, :ks[i]].contiguous())

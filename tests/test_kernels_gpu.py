@@ -458,19 +458,22 @@ def test_argmax_rules_on_the_device():
         assert out.tolist() == [P.argmax_last(r) for r in view.cpu().tolist()]
 
 
-def test_topk_with_penalty_on_the_device():
+@pytest.mark.parametrize("V,width", [(5003, 256), (40961, 1024), (300, 64)])
+def test_topk_with_penalty_on_the_device(V, width):
+    """Slices of 4,096 logits leave their own k best, of which the k best are taken: vocabularies of
+    one slice, of two with a short last one (shorter than k), and of eleven."""
     k = kernels("float32")
-    V = 5003
     logits = rnd(4, V, seed=20, scale=2.0)
-    logits[1, 10] = logits[1, 4000] = logits[1].max() + 1                      # ties at the top
+    far = V - 3                                                                 # an id in the last slice
+    logits[1, 10] = logits[1, far] = logits[1].max() + 1                        # ties at the top
     logits[2, 5] = float("nan")
-    recent = torch.tensor([[3, 5, 1, 1, 2, 1, 0, 0], [10, 10, 4000, 7, 0, 0, 0, 0], [0] * 8, [9] * 8], dtype=torch.int32)
+    recent = torch.tensor([[3, 5, 1, 1, 2, 1, 0, 0], [10, 10, far, 7, 0, 0, 0, 0], [0] * 8, [9] * 8], dtype=torch.int32)
     n_recent = torch.tensor([6, 4, 0, 8], dtype=torch.int32)
     penalty = torch.tensor([2.0, 1.3, 1.0, 1.1])
-    ks = torch.tensor([40, 7, 256, 1], dtype=torch.int32)
+    ks = torch.tensor([40, 7, min(width, V), 1], dtype=torch.int32)
     dev = logits.clone().cuda()
-    cands = torch.zeros(4, 256, dtype=torch.int64, device="cuda")
-    k.topk(dev, recent.cuda(), n_recent.cuda(), penalty.cuda(), ks.cuda(), cands)
+    cands = torch.zeros(4, width, dtype=torch.int64, device="cuda")
+    k.topk(dev, recent.cuda(), n_recent.cuda(), penalty.cuda(), ks.cuda(), cands, k_max=int(ks.max()))
     for r in range(4):
         pen = P.penalize(logits[r].tolist(), recent[r, :n_recent[r]].tolist(), 10 ** 6, float(penalty[r]))
         pen = torch.tensor(pen, dtype=torch.float32)
