@@ -18,6 +18,7 @@ import time
 from dataclasses import dataclass
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache.manager import host_lib
@@ -137,17 +138,16 @@ def pick_rows(rt, logits: torch.Tensor, samplers: Sequence[Optional[Sampler]],
         width = max(1, max(len(x) for x in recents))
         ks = [min(samplers[r].params.top_k, vocab) for r in device_rows]
         # one copy to the device: the recent tokens, how many, k, and the penalties' bits
-        flat = torch.zeros(n * width + 3 * n, dtype=torch.int32)
-        rec = flat[:n * width].view(n, width)
+        flat = np.zeros(n * width + 3 * n, dtype=np.int32)
+        rec = flat[:n * width].reshape(n, width)
         for i, x in enumerate(recents):
-            rec[i, :len(x)] = torch.tensor(x, dtype=torch.int32)
-        flat[n * width:n * width + n] = torch.tensor([len(x) for x in recents], dtype=torch.int32)
-        flat[n * width + n:n * width + 2 * n] = torch.tensor(ks, dtype=torch.int32)
-        flat[n * width + 2 * n:].view(torch.float32)[:] = torch.tensor(
-            [samplers[r].params.repeat_penalty for r in device_rows], dtype=torch.float32)
-        on = flat.to(dev)
+            rec[i, :len(x)] = x
+        flat[n * width:n * width + n] = [len(x) for x in recents]
+        flat[n * width + n:n * width + 2 * n] = ks
+        flat[n * width + 2 * n:].view(np.float32)[:] = [samplers[r].params.repeat_penalty for r in device_rows]
+        on = torch.from_numpy(flat).to(dev)
         sel = logits if n == rows else logits[torch.tensor(device_rows, device=dev)].contiguous()
-        cands = torch.zeros((n, max(ks)), dtype=torch.int64, device=dev)
+        cands = torch.empty((n, max(ks)), dtype=torch.int64, device=dev)      # a row's first k places are written
         rt.k.topk(sel, on[:n * width].view(n, width), on[n * width:n * width + n], on[n * width + 2 * n:].view(torch.float32),
                   on[n * width + n:n * width + 2 * n], cands, k_max=max(ks))
         host = cands.cpu()
