@@ -14,6 +14,11 @@ extern "C" {
 #endif
 
 const char* axk_last_error(void);
+// The kernel instances compiled into the library (only_hit 0) or launched since the last reset
+// (only_hit 1), a name a line, into buf; returns the bytes the whole list needs.  A test asserts
+// that every instance is launched, and checked, by some test.
+long axk_instances(char* buf, long size, int only_hit);
+void axk_instances_reset(void);
 // 1 for the bfloat16 build, 0 for float32; bytes of one element.
 int axk_is_bf16(void);
 int axk_elem_size(void);
@@ -96,7 +101,8 @@ int axk_pack_matrix(const void* src, void* dst, int rows, int k, void* stream);
 // gate rows then up rows, and out elem [M, N] = silu(X . gate^T) * (X . up^T) (no bias).
 // x_stride / out_stride: elements between rows.  workspace: axk_gemm_workspace(m, n, k, mode) bytes
 // (0 for most shapes: then it may be null), 16-byte aligned; products of more than 16 rows with a
-// narrow output give each segment of K blocks of their own and add the segments' sums through it.
+// matrix of several segments give each segment of K blocks of their own and add the segments' sums
+// through it (at most 2 GB: a product of more rows than that holds runs in passes).
 //
 // With a packed W every output element is the sum, in ascending order, of axk_gemm_segments(n, k,
 // gated) chains of 32x32x16 MFMAs over contiguous segments of K: the bits of a row do not depend on

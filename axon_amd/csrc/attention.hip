@@ -16,6 +16,7 @@
 
 #include "api.h"
 #include "common.h"
+#include "instances.h"
 
 #define ATT_BLOCK 64
 #define ATT_MAX_HD 256
@@ -111,6 +112,7 @@ extern "C" int axk_attention(const void* q, int q_stride, const void* k_cache, c
   AXK_REQUIRE(window >= 0, "attention: window %d is negative", window);
   if (n_tokens == 0) return 0;
   dim3 grid(n_tokens, n_heads);
+  AXK_INSTANCE(INST_ATTENTION_ROWS, AXON_BF16);
   attention_rows_kernel<<<grid, AXON_WAVE, 0, (hipStream_t)stream>>>(
       (const elem_t*)q, q_stride, (const elem_t*)k_cache, (const elem_t*)v_cache, block_table, table_stride, positions,
       seq_rows, (elem_t*)out, n_heads, n_kv_heads, head_dim, page_size, window, scale);

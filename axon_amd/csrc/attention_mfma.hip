@@ -30,6 +30,7 @@
 
 #include "api.h"
 #include "common.h"
+#include "instances.h"
 
 #define ATT_BLOCK 64          // positions of a block: the unit of the fold
 #define DC_CHUNK 256          // positions of one work item of the decoding kernel: four blocks, a wave each
@@ -724,6 +725,7 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
       }                                                                                                             \
       configured = true;                                                                                            \
     }                                                                                                               \
+    AXK_INSTANCE(INST_ATTENTION_PREFILL, HD, HPB);                                                                  \
     attention_prefill_kernel<HD, HPB><<<grid, 256 * HPB, lds, (hipStream_t)stream>>>(                               \
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,      \
         positions, seq_rows, (bf16_t*)out, tiles, n_heads, n_kv_heads, page_size, window, scale);                   \
@@ -792,6 +794,7 @@ extern "C" int axk_attention_decode(const void* q, int q_stride, const void* k_c
       }                                                                                                              \
       configured = true;                                                                                             \
     }                                                                                                                \
+    AXK_INSTANCE(INST_ATTENTION_DECODE, HD, BW);                                                                     \
     attention_decode_kernel<HD, BW><<<(unsigned)n_work * n_kv_heads * (4 / BW), BW * 64, lds, (hipStream_t)stream>>>( \
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,       \
         positions, seq_rows, token_index, n_tokens, work, partial, max_chunks, n_heads, n_kv_heads, page_size,       \

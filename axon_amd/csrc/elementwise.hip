@@ -1,24 +1,8 @@
 // Row-wise kernels: embedding gather, RMSNorm, rotary tables, rotary + paged cache store,
 // SwiGLU, fills.  Each computes a row the same way whatever other rows share the launch.
-#include <stdarg.h>
-#include <stdio.h>
-
 #include "api.h"
 #include "common.h"
-
-// ---------------------------------------------------------------------------- error channel
-static thread_local char g_error[512] = "";
-
-void axk_set_error(const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_error, sizeof g_error, fmt, ap);
-  va_end(ap);
-}
-
-extern "C" const char* axk_last_error(void) { return g_error; }
-extern "C" int axk_is_bf16(void) { return AXON_BF16; }
-extern "C" int axk_elem_size(void) { return (int)sizeof(elem_t); }
+#include "instances.h"
 
 // ---------------------------------------------------------------------------- embedding
 // One block per token; the row is widened exactly (bf16 -> f32) or copied.
@@ -144,11 +128,14 @@ extern "C" int axk_rmsnorm(const float* x, const int32_t* rows, const void* gain
   AXK_REQUIRE(n_rows >= 0 && dim > 0, "rmsnorm: bad sizes rows=%d dim=%d", n_rows, dim);
   if (n_rows == 0) return 0;
   const bool vec = dim % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0;
-  if (vec)
+  if (vec) {
+    AXK_INSTANCE(INST_RMSNORM, 1);
     rmsnorm_vec_kernel<<<n_rows, NORM_THREADS, 0, (hipStream_t)stream>>>(x, rows, gain, gain_is_f32, (elem_t*)out, dim,
                                                                         eps);
-  else
+  } else {
+    AXK_INSTANCE(INST_RMSNORM, 0);
     rmsnorm_kernel<<<n_rows, NORM_THREADS, 0, (hipStream_t)stream>>>(x, rows, gain, gain_is_f32, (elem_t*)out, dim, eps);
+  }
   AXK_LAUNCH_CHECK("rmsnorm");
   return 0;
 }

@@ -9,6 +9,7 @@
 // product (true 32-bit), and the bfloat16 build's fallback for shapes the MFMA kernels refuse.
 #include "api.h"
 #include "common.h"
+#include "instances.h"
 
 #define FMA_BN 64
 #define FMA_BK 16
@@ -130,12 +131,13 @@ static int launch_fma(const elem_t* x, int x_stride, const elem_t* w, const void
   const bool vec_w = (k % 4 == 0) && ((uintptr_t)w % vbytes == 0);
   const bool vec_x = (k % 4 == 0) && (x_stride % 4 == 0) && ((uintptr_t)x % vbytes == 0);
 #define FMA_LAUNCH(BM, GLU)                                                                                      \
+  AXK_INSTANCE(INST_GEMM_FMA, BM, GLU);                                                                          \
   gemm_fma_kernel<BM, GLU><<<dim3(ceil_div(n, FMA_BN), ceil_div(m, BM)), FMA_THREADS, 0, stream>>>(              \
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, vec_x, vec_w)
   if (mode == MODE_SWIGLU) {
-    if (m <= 16) FMA_LAUNCH(16, true); else FMA_LAUNCH(64, true);
+    if (m <= 16) { FMA_LAUNCH(16, true); } else { FMA_LAUNCH(64, true); }
   } else {
-    if (m <= 16) FMA_LAUNCH(16, false); else FMA_LAUNCH(64, false);
+    if (m <= 16) { FMA_LAUNCH(16, false); } else { FMA_LAUNCH(64, false); }
   }
 #undef FMA_LAUNCH
   AXK_LAUNCH_CHECK("gemm_fma");

@@ -37,15 +37,14 @@
 // * gemm_tile (M > 64): a block of 4 or 8 waves owns a BM x BN tile of the output, walks K in
 //   steps of 64 through LDS stages filled by direct global -> LDS loads (the next step's loads
 //   in flight while this one multiplies), and each wave keeps a tile of 32x32x16 MFMA
-//   accumulators.  The segments are either kept apart in registers (a second set of
-//   accumulators takes each finished segment's sums; SEG) or, where the output gives too few
-//   tiles for 256 CUs, given to blocks of their own (gridDim.y = S), whose sums go through a
-//   workspace and are added in segment order by gemm_split_reduce, which also applies the
-//   epilogue.  X rows land in LDS with their 16-byte slots permuted so that fragment reads of
+//   accumulators.  With S > 1 segments each goes to blocks of its own (gridDim.y = S), whose sums
+//   go through a workspace and are added in segment order by gemm_split_reduce, which also
+//   applies the epilogue.  X rows land in LDS with their 16-byte slots permuted so that fragment reads of
 //   neighbouring rows fall into different banks; W blocks land as they are.  Blocks are numbered
 //   so that the blocks of one XCD (every eighth block) share weight tiles in that XCD's L2.
 #include "api.h"
 #include "common.h"
+#include "instances.h"
 
 #if AXON_BF16
 
@@ -82,14 +81,11 @@ __device__ inline bf16x8 as_frag(u32x4 v) { return __builtin_bit_cast(bf16x8, v)
 // A block then owns BN / 2 output columns; each wave's share of the LDS tile holds the gate
 // rows of its columns and, after them, the up rows of the same columns, so that a lane ends
 // with both values of an output element.
-//
-// SEG: the block walks all of K and keeps the `segs` segments apart: at the end of a segment its
-// sums are added to a second set of accumulators and the first starts from zero again.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK, int STAGES, bool SEG>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK, int STAGES>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const void* __restrict__ bias,
                  int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode, int m_blocks,
-                 int n_blocks, float* __restrict__ partial, int segs) {
+                 int n_blocks, float* __restrict__ partial) {
   extern __shared__ __align__(16) unsigned char smem[];
   static_assert(BK == 64 || BK == 32, "segments of K are counted in steps of 64: whole K tiles");
   constexpr int PER64 = 64 / BK;                       // K tiles in a step of 64
@@ -172,17 +168,12 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   };
 
   f32x16 acc[TM][TN];
-  f32x16 total[SEG ? TM : 1][SEG ? TN : 1];     // SEG: the sums of the segments that are finished
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        acc[i][j][e] = 0.0f;
-        if (SEG) total[i][j][e] = 0.0f;
-      }
-  int seg_at = 0, seg_end = SEG ? (int)((long)(nk / PER64) / segs) * PER64 : 0;   // SEG: the segment under way ends before K tile seg_end
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   // fragment addresses: row = tile row + lane % 32, k chunk = 2 ks + lane / 32, slot = chunk ^ SWZ(row)
   const int frow = lane & 31, fhalf = lane >> 5, fsw = SWZ(frow);
@@ -248,28 +239,8 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
         multiply(cur, TN / 2, TN);
       }
     }
-    if (SEG && kt + 1 == seg_end) {
-      // a segment's chain is complete: its sums join the finished ones, in segment order
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            total[i][j][e] += acc[i][j][e];
-            acc[i][j][e] = 0.0f;
-          }
-      ++seg_at;
-      seg_end = (int)((long)(seg_at + 1) * (nk / PER64) / segs) * PER64;
-    }
   }
 #undef SWZ
-  if (SEG) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = total[i][j];
-  }
 
   // epilogue: lane holds column n = lane % 32 of each tile and rows (e/4)*8 + (lane/32)*4 + e%4
   if (partial) {
@@ -330,8 +301,27 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   }
 }
 
+// The same for a width that is no multiple of 4 (rows of the workspace are then not 16-byte
+// aligned): a thread an element, the same additions in the same order.  No gated epilogue here: a
+// [gate; up] matrix has whole row tiles.
+__global__ void __launch_bounds__(256)
+gemm_split_reduce_any_kernel(const float* __restrict__ partial, int splits, int M, int N, const void* __restrict__ bias,
+                             int bias_is_f32, void* __restrict__ out, int out_stride, int mode) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)M * N) return;
+  const int m = (int)(idx / N), n = (int)(idx % N);
+  const size_t plane = (size_t)M * N;
+  float v = partial[idx];
+  for (int z = 1; z < splits; ++z) v += partial[(size_t)z * plane + idx];
+  if (bias) v += load_vec(bias, bias_is_f32, n);
+  const size_t at = (size_t)m * out_stride + n;
+  if (mode == MODE_STORE) reinterpret_cast<bf16_t*>(out)[at] = float_to_bf16(v);
+  else if (mode == MODE_ADD_F32) reinterpret_cast<float*>(out)[at] += v;
+  else reinterpret_cast<float*>(out)[at] = v;
+}
+
 // The sums of the split-K blocks, added in block order, then the epilogue of the product.
-// One thread per 4 consecutive columns of a row (N is a multiple of 4 on this path).
+// One thread per 4 consecutive columns of a row (N a multiple of 4).
 __global__ void __launch_bounds__(256)
 gemm_split_reduce_kernel(const float* __restrict__ partial, int splits, int M, int N, const void* __restrict__ bias,
                          int bias_is_f32, void* __restrict__ out, int out_stride, int mode) {
@@ -487,27 +477,39 @@ static int launch_split_reduce_rope(const float* partial, int splits, int m, int
 // order, then the epilogue (with the rotary store, or the norm of the new rows, where asked).
 static int add_split_sums(const float* partial, int splits, int m, int n, const void* bias, int bias_is_f32, void* out,
                           int out_stride, int mode, const SplitNorm* norm, const RopeStore* rope, hipStream_t stream) {
-  if (rope != nullptr) return launch_split_reduce_rope(partial, splits, m, n, bias, bias_is_f32, out, out_stride, *rope, stream);
+  if (rope != nullptr) {
+    AXK_INSTANCE(INST_GEMM_SPLIT_REDUCE, 2);
+    return launch_split_reduce_rope(partial, splits, m, n, bias, bias_is_f32, out, out_stride, *rope, stream);
+  }
   if (norm != nullptr) {
+    AXK_INSTANCE(INST_GEMM_SPLIT_REDUCE, 1);
     gemm_split_reduce_norm_kernel<<<m, SRN_THREADS, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, (float*)out,
                                                                  out_stride, *norm);
     AXK_LAUNCH_CHECK("gemm_split_reduce_norm");
     return 0;
   }
+  if (n % 4 != 0) {
+    AXK_INSTANCE(INST_GEMM_SPLIT_REDUCE, 3);
+    gemm_split_reduce_any_kernel<<<(unsigned)(((size_t)m * n + 255) / 256), 256, 0, stream>>>(partial, splits, m, n, bias,
+                                                                                             bias_is_f32, out, out_stride, mode);
+    AXK_LAUNCH_CHECK("gemm_split_reduce");
+    return 0;
+  }
+  AXK_INSTANCE(INST_GEMM_SPLIT_REDUCE, 0);
   gemm_split_reduce_kernel<<<ceil_div(m * (n / 4), 256), 256, 0, stream>>>(partial, splits, m, n, bias, bias_is_f32, out,
                                                                           out_stride, mode);
   AXK_LAUNCH_CHECK("gemm_split_reduce");
   return 0;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, bool SEG = false, int BK = 64, int STAGES = 2>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool GLU, int BK = 64, int STAGES = 2>
 static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                        int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs = 1,
                        float* partial = nullptr, const SplitNorm* norm = nullptr, const RopeStore* rope = nullptr) {
   static bool configured = false;
   constexpr int lds_bytes = STAGES * (BM + BN) * BK * 2;
   static_assert(lds_bytes <= 160 * 1024, "the stages do not fit the LDS of a CU");
-  auto kernel = &gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, GLU, BK, STAGES, SEG>;
+  auto kernel = &gemm_tile_kernel<BM, BN, WAVES_M, WAVES_N, GLU, BK, STAGES>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        lds_bytes);
@@ -517,12 +519,12 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
     }
     configured = true;
   }
-  // SEG: every block walks all segments; else a block a segment (gridDim.y) and the sums through `partial`
-  const int splits = SEG ? 1 : segs;
+  // a block a segment (gridDim.y), the sums through `partial`
+  const int splits = segs;
   const int m_blocks = ceil_div(m, BM), n_blocks = ceil_div(n, GLU ? BN / 2 : BN);
+  AXK_INSTANCE(INST_GEMM_TILE, BM, BN, WAVES_M, WAVES_N, GLU);
   kernel<<<dim3(m_blocks * n_blocks, splits), WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
-      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks, splits > 1 ? partial : nullptr,
-      segs);
+      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks, splits > 1 ? partial : nullptr);
   AXK_LAUNCH_CHECK("gemm_tile");
   return splits > 1 ? add_split_sums(partial, splits, m, n, bias, bias_is_f32, out, out_stride, mode, norm, rope, stream) : 0;
 }
@@ -1246,6 +1248,7 @@ static int launch_normed_of(const NormedRows& in, const bf16_t* w, const void* b
       }                                                                                                               \
       configured = true;                                                                                              \
     }                                                                                                                 \
+    AXK_INSTANCE(INST_GEMM_NORMED, UNITS, SEGS, EPI, MPAD, KCV);                                                      \
     kernel<<<shape.blocks, (nw + NORMED_NORM_WAVES) * 64, lds, stream>>>(in, w, bias, bias_is_f32, out, out_stride, m, n, k, \
                                                                          mode, rope, units);                          \
   }
@@ -1270,7 +1273,8 @@ static int launch_normed(const NormedRows& in, const bf16_t* w, const void* bias
   if (shape.per_wave == 1) BY_SEGS(1)
   if constexpr (EPI == EPI_GLU) {
     if (shape.per_wave == 2) BY_SEGS(2)
-    if (shape.per_wave == 3) BY_SEGS(3)
+    // three pairs a wave: only matrices so large that K is one segment (normed_shape, gemm_segments)
+    if (shape.per_wave == 3 && segs == 1) return launch_normed_of<3, 1, EPI>(ARGS_NORMED);
   }
 #undef BY_SEGS
 #undef ARGS_NORMED
@@ -1413,7 +1417,14 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
 #pragma unroll
       for (int j = 0; j < MT16; ++j) {
         const int m = j * 16 + (lane & 15);
-        if (m < M) *reinterpret_cast<float4*>(dst + (size_t)m * N) = make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+        if (m >= M) continue;
+        if (N % 4 == 0) {
+          *reinterpret_cast<float4*>(dst + (size_t)m * N) = make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+        } else {                                                   // rows of the workspace that are not 16-byte aligned
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < N) dst[(size_t)m * N + e] = acc[i][j][e];
+        }
       }
     }
     return;
@@ -1429,6 +1440,7 @@ template <int NT16, int WAVES, int EPI>
 static int launch_rows_of(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                           int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs, float* partial, int units) {
   constexpr int lds_bytes = ROWS_NS * 8 * 1024;
+  AXK_INSTANCE(INST_GEMM_ROWS, NT16, WAVES, EPI);
   gemm_rows_kernel<NT16, WAVES, ROWS_NS, EPI><<<dim3(ceil_div(units, WAVES), segs), WAVES * 64, lds_bytes, stream>>>(
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, segs > 1 ? partial : nullptr, units);
   AXK_LAUNCH_CHECK("gemm_rows");
@@ -1465,6 +1477,7 @@ static int launch_stream(const bf16_t* x, int x_stride, const bf16_t* w, const v
                          int out_stride, int m, int n, int k, int mode, hipStream_t stream, const RopeStore& rope) {
   // the ring as deep as the registers allow: (NT16 + MT16) 8 registers a step
   constexpr int FIT = 384 / ((NT16 + MT16) * 8), DEPTH = FIT < 8 ? FIT : 8;
+  AXK_INSTANCE(INST_GEMM_STREAM, NT16, MT16, SEGS, EPI);
   gemm_stream_kernel<NT16, MT16, SEGS, DEPTH, EPI><<<ceil_div(n, EPI == EPI_GLU ? 16 : NT16 * 16), SEGS * 64, 0, stream>>>(
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, rope);
   AXK_LAUNCH_CHECK("gemm_stream");
@@ -1482,7 +1495,14 @@ static int launch_stream_rows(const bf16_t* x, int x_stride, const bf16_t* w, co
     case 2: return launch_stream<NT16, MT16, 2, EPI>(ARGS);             \
     case 4: return launch_stream<NT16, MT16, 4, EPI>(ARGS);             \
   }
-  BY_SEGS(1)
+  // two row tiles a block without a paired epilogue: matrices of 16,384 rows or more, which have
+  // one or two segments, never four (gemm_segments)
+  if constexpr (NT16 == 2 && EPI == EPI_PLAIN) {
+    if (segs == 1) return launch_stream<NT16, 1, 1, EPI>(ARGS);
+    if (segs == 2) return launch_stream<NT16, 1, 2, EPI>(ARGS);
+  } else {
+    BY_SEGS(1)
+  }
 #undef BY_SEGS
 #undef ARGS
   axk_set_error("gemm_stream: %d segments", segs);
@@ -1556,30 +1576,39 @@ static int tiles32_of(int n, int mode) { return mode == MODE_SWIGLU ? n / 16 : (
 // (measured on the products of a 7B layer: from 17 rows on, by 10 to 30 %).
 #define AXON_STREAM_MAX_M 16
 
-// More rows than the streaming kernel takes, S > 1 segments: a block a segment (the blocks' sums
-// go through a workspace and are added in segment order by a second kernel; measured faster for
-// every product of the 7B and 14B layers up to 8,192 rows, and the only way to occupy the chip
-// when the output is small), unless the workspace would pass 2 GB: then blocks walk all of K
-// and keep the segments apart in registers.  Decided by the sizes alone.
-static bool segments_across_blocks(int m, int n, int k, int mode, int segs) {
-  if (segs <= 1 || n % 4 != 0) return false;
-  return (size_t)segs * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float) <= ((size_t)2048 << 20);
+// More rows than the streaming kernel takes, S > 1 segments: a block a segment; the blocks' sums
+// go through a workspace and are added in segment order by a second kernel (measured faster for
+// every product of the 7B and 14B layers up to 8,192 rows than keeping the segments apart in one
+// block's registers, and the only way to occupy the chip when the output is small).  The
+// workspace holds the sums of at most GEMM_PASS_BYTES: a product of more rows runs in passes of
+// `rows_a_pass` rows, one after the other (a row's bits do not depend on the rows beside it).
+#define GEMM_PASS_BYTES ((size_t)2048 << 20)
+
+static int rows_a_pass(int n, int mode, int segs) {
+  const size_t row_bytes = (size_t)segs * (mode == MODE_SWIGLU ? 2 : 1) * n * sizeof(float);
+  const size_t rows = GEMM_PASS_BYTES / row_bytes / 256 * 256;       // whole tiles of 256 rows
+  return (int)(rows < 256 ? 256 : rows > (1u << 30) ? (1u << 30) : rows);
 }
 
 size_t gemm_workspace_bytes(int m, int n, int k, int mode) {
   if (k % 64 != 0 || m <= AXON_STREAM_MAX_M) return 0;
   const int s = gemm_segments(tiles32_of(n, mode), k);
-  if (!segments_across_blocks(m, n, k, mode, s)) return 0;
-  return (size_t)s * (mode == MODE_SWIGLU ? 2 : 1) * m * n * sizeof(float);
+  if (s <= 1) return 0;
+  const int rows = m < rows_a_pass(n, mode, s) ? m : rows_a_pass(n, mode, s);
+  return (size_t)s * (mode == MODE_SWIGLU ? 2 : 1) * rows * n * sizeof(float);
 }
 
 // Whether the product that adds into the rows runs with a block a segment, so that the kernel that
 // adds the segments' sums can also norm the finished rows (gemm_split_reduce_norm_kernel: rows of
-// up to SRN_MAX_N columns).
+// up to SRN_MAX_N columns, in whole float4).
 int gemm_then_norm_ok(int m, int n, int k) {
-  return gemm_pack_ok(n, k, 0) && m > AXON_STREAM_MAX_M && n <= SRN_MAX_N &&
-         segments_across_blocks(m, n, k, MODE_ADD_F32, gemm_segments(tiles32_of(n, MODE_ADD_F32), k));
+  return gemm_pack_ok(n, k, 0) && m > AXON_STREAM_MAX_M && n <= SRN_MAX_N && n % 4 == 0 &&
+         gemm_segments(tiles32_of(n, MODE_ADD_F32), k) > 1;
 }
+
+static int gemm_mfma_pass(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                          int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs, const SplitNorm* norm,
+                          float* ws, const RopeStore* rope_after);
 
 static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                               int out_stride, int m, int n, int k, int mode, hipStream_t stream,
@@ -1595,17 +1624,16 @@ static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, co
     return -1;
   }
   const int segs = gemm_segments(tiles32_of(n, mode), k);
-#define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream
   if (m <= AXON_STREAM_MAX_M) {
     if (norm || rope_after) {
       axk_set_error("gemm: M=%d goes to the streaming kernel, which has these epilogues of its own", m);
       return -1;
     }
-    if (mode == MODE_SWIGLU) return launch_stream_any<EPI_GLU>(ARGS, segs, RopeStore());
-    return launch_stream_any<EPI_PLAIN>(ARGS, segs, RopeStore());
+    if (mode == MODE_SWIGLU)
+      return launch_stream_any<EPI_GLU>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, segs, RopeStore());
+    return launch_stream_any<EPI_PLAIN>(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, segs, RopeStore());
   }
-  const bool across = segments_across_blocks(m, n, k, mode, segs);
-  if ((norm || rope_after) && (!across || mode != (norm ? MODE_ADD_F32 : MODE_STORE))) {
+  if ((norm || rope_after) && (segs <= 1 || mode != (norm ? MODE_ADD_F32 : MODE_STORE))) {
     axk_set_error("gemm: M=%d N=%d K=%d mode %d does not run with a block a segment: no kernel adds sums after it", m, n,
                   k, mode);
     return -1;
@@ -1616,28 +1644,45 @@ static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, co
                   workspace_bytes);
     return -1;
   }
-  float* ws = (float*)workspace;
+  const int pass = segs > 1 ? rows_a_pass(n, mode, segs) : m;
+  if (m <= pass)
+    return gemm_mfma_pass(x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, segs, norm,
+                          (float*)workspace, rope_after);
+  // in passes: every operand that has a row per row of X moves on with it
+  const size_t out_elem = mode == MODE_STORE || mode == MODE_SWIGLU ? sizeof(bf16_t) : sizeof(float);
+  for (int m0 = 0; m0 < m; m0 += pass) {
+    const int rows = m - m0 < pass ? m - m0 : pass;
+    SplitNorm norm_at;
+    RopeStore rope_at;
+    if (norm) {
+      norm_at = *norm;
+      norm_at.values += (size_t)m0 * n;
+    }
+    if (rope_after) {
+      rope_at = *rope_after;
+      rope_at.table += (size_t)m0 * (rope_at.head_dim / 2) * 2;
+      rope_at.positions += m0;
+      rope_at.seq_rows += m0;
+    }
+    const int rc = gemm_mfma_pass(x + (size_t)m0 * x_stride, x_stride, w, bias, bias_is_f32,
+                                  (char*)out + (size_t)m0 * out_stride * out_elem, out_stride, rows, n, k, mode, stream, segs,
+                                  norm ? &norm_at : nullptr, (float*)workspace, rope_after ? &rope_at : nullptr);
+    if (rc != 0) return rc;
+  }
+  return 0;
+}
+
+// One pass: more than AXON_STREAM_MAX_M rows whose segments' sums (if S > 1) fit the workspace.
+static int gemm_mfma_pass(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
+                          int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs, const SplitNorm* norm,
+                          float* ws, const RopeStore* rope_after) {
+#define ARGS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream
   const bool glu = mode == MODE_SWIGLU;
   if (m <= 64) {
-    // the segments in registers only where the sums cannot go through the workspace (one tile of 64 rows)
-    if (segs > 1 && !across) {
-      if (glu) return launch_tile<64, 256, 1, 4, true, true>(ARGS, segs);
-      return launch_tile<64, 128, 1, 4, false, true, 64, 3>(ARGS, segs);
-    }
     // W streamed, X shared through LDS; a block a segment.  Two row tiles a wave where the matrix is large.
     if (glu) return launch_rows<2, EPI_GLU>(ARGS, segs, ws, nullptr, nullptr);
     if (n >= 32 * 512) return launch_rows<2, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
     return launch_rows<1, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
-  }
-  if (segs > 1 && !across) {
-    // the segments in registers: 128 x 256 tiles (8 waves) where they occupy the chip, else 128 x 128
-    const long wide = (long)ceil_div(m, 128) * ceil_div(n, glu ? 128 : 256);
-    if (wide >= 200) {
-      if (glu) return launch_tile<128, 256, 2, 4, true, true>(ARGS, segs);
-      return launch_tile<128, 256, 2, 4, false, true>(ARGS, segs);
-    }
-    if (glu) return launch_tile<128, 128, 2, 2, true, true>(ARGS, segs);
-    return launch_tile<128, 128, 2, 2, false, true>(ARGS, segs);
   }
   if (m <= 256) {
     if (glu) return launch_tile<128, 128, 2, 2, true>(ARGS, segs, ws);
@@ -1646,9 +1691,8 @@ static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, co
   // 256 x 256 tiles (8 waves) where they fill the chip: one round of at least 140 blocks (on 256
   // CUs), or several rounds of which the last is not mostly idle; else 128 x 128 tiles, four times
   // as many blocks at twice the traffic from L2 per product.  Thresholds are measured ones.
-  const int splits = across ? segs : 1;
   const int n_per_block = glu ? 128 : 256;
-  const long big = (long)ceil_div(m, 256) * ceil_div(n, n_per_block) * splits;
+  const long big = (long)ceil_div(m, 256) * ceil_div(n, n_per_block) * segs;
   const long rounds = (big + 255) / 256;
   const bool use_big = big <= 256 ? big >= 140 : big * 10 >= rounds * 256 * 7;
   if (glu) {
@@ -1658,7 +1702,7 @@ static int gemm_mfma_dispatch(const bf16_t* x, int x_stride, const bf16_t* w, co
   // one round of 256 x 256 tiles that leaves a quarter of the CUs idle, and N in whole tiles of
   // 192 columns that still fit one round: the narrower tile (measured 1.1 times the cost per
   // product, three quarters of the products per block).
-  if (use_big && splits == 1 && big <= 192 && n % 192 == 0 && (long)ceil_div(m, 256) * (n / 192) <= 256)
+  if (use_big && segs == 1 && big <= 192 && n % 192 == 0 && (long)ceil_div(m, 256) * (n / 192) <= 256)
     return launch_tile<256, 192, 4, 2, false>(ARGS, segs, ws, norm);
   if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS, segs, ws, norm, rope_after);
   return launch_tile<128, 128, 2, 2, false>(ARGS, segs, ws, norm, rope_after);
@@ -1683,7 +1727,7 @@ int gemm_qkv_rope_ok(int m, int n, int k, int head_dim, int rotary_dim) {
   if (m < 1 || k % 64 != 0 || rotary_dim != head_dim || head_dim % 32 != 0 || n % head_dim != 0) return 0;
   if (!gemm_pack_ok(n, k, 0)) return 0;
   if (m <= AXON_STREAM_MAX_M) return 1;
-  return segments_across_blocks(m, n, k, MODE_STORE, gemm_segments(tiles32_of(n, MODE_STORE), k));
+  return gemm_segments(tiles32_of(n, MODE_STORE), k) > 1;
 }
 
 int launch_gemm_qkv_rope(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, bf16_t* out,

@@ -180,7 +180,7 @@ topk_slice_kernel(float* __restrict__ logits, int stride, const int32_t* __restr
   const int r = blockIdx.y, s = blockIdx.x, slices = gridDim.x;
   const int lo = s * TOPK_SLICE, count = min(n - lo, TOPK_SLICE);
   float* row = logits + (size_t)r * stride;
-  int k = min(k_of_row[r], n);
+  int k = min(min(k_of_row[r], n), k_stride);        // never past the places of a slice, whatever the caller asks
   if (k <= 0) return;
   for (int i = threadIdx.x; i < count; i += TOPK_THREADS) vals[i] = row[lo + i];
   __syncthreads();
@@ -227,7 +227,7 @@ topk_merge_kernel(const uint64_t* __restrict__ slice_keys, const int32_t* __rest
   __shared__ int hist[256];
   __shared__ int vars[2], s_count;
   const int r = blockIdx.x;
-  const int k = min(k_of_row[r], n);
+  const int k = min(min(k_of_row[r], n), min(k_stride, cands_stride));   // never past the row of candidates
   if (k <= 0) return;
   const uint64_t* keys = slice_keys + (size_t)r * slices * k_stride;
   const int32_t* counts = slice_count + r * slices;

@@ -143,6 +143,21 @@ class LLM:
         trace = StepTrace.from_env()
         ahead_ok = trace is None
         behind = None            # (picks on their way, the requests they belong to)
+        # The clocks of `GenStats`.  Steps are queued ahead of the device, so a step's own time is not
+        # known on the host; what is known is when the host had to wait.  Everything between two
+        # marks is charged to the kind of step (decoding only, or feeding prompts) that was being
+        # prepared, waits for earlier steps included, and the device is waited for where the kind
+        # changes and at the end: the two clocks add up to the wall time, and tokens divided by
+        # their clock can never beat a synchronised measurement of the same steps.
+        clock = {"mark": time.time(), "kind": None}
+
+        def charge(decoding: bool) -> None:
+            now = time.time()
+            if decoding:
+                stats.decode_seconds += now - clock["mark"]
+            else:
+                stats.prompt_seconds += now - clock["mark"]
+            clock["mark"] = now
 
         def settle(behind) -> List[int]:
             """Fill in the picks that were on their way; the requests that picked a stop token."""
@@ -189,6 +204,11 @@ class LLM:
                         continue
                 if not plan:
                     raise RuntimeError("the scheduler has requests but planned nothing: the cache pool is too small")
+                decoding = all(p.count == 1 and p.start > 0 for p in plan)
+                if clock["kind"] is not None and clock["kind"] != decoding:
+                    torch.cuda.synchronize()         # the steps of the other kind have run: their time is theirs
+                    charge(clock["kind"])
+                clock["kind"] = decoding
                 t_step = time.time()
                 if feed:
                     logits = self.engine.step_from_picks([p.id for p in plan])
@@ -241,17 +261,18 @@ class LLM:
                     torch.cuda.synchronize()
                     waiting, running, _ = sched.counts()
                     trace.line(t_step, (time.time() - t_step) * 1e3, plan, waiting, running, len(preempted))
-                dt = time.time() - t_step
-                if all(p.count == 1 and p.start > 0 for p in plan):
-                    stats.decode_seconds += dt
+                charge(decoding)
+                if decoding:
                     stats.decode_steps += 1
                     stats.decode_tokens += len(plan)
                 else:
-                    stats.prompt_seconds += dt
                     stats.prompt_tokens += sum(p.count for p in plan if p.wants_logits and p.count > 1)
             if behind is not None:
                 settle(behind)
                 behind = None
+            if clock["kind"] is not None:
+                torch.cuda.synchronize()
+                charge(clock["kind"])
         finally:
             for rid in order:
                 self.engine.release(rid)

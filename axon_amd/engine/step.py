@@ -74,6 +74,7 @@ class StepContext:
         self.decode_index: Optional[torch.Tensor] = None
         self.decode_shapes: Dict = {}
         self.decode_inputs: Dict = {}       # what the mixers asked to have on the device (Mixer.decode_input)
+        self.decode_scratch: Dict = {}      # workspaces that stay in place (Mixer.decode_scratch)
 
     def no_rotation(self) -> torch.Tensor:
         return torch.empty((self.n_tokens, 0, 2), dtype=torch.float32, device=self.rt.device)
@@ -119,7 +120,7 @@ class Engine:
         # graphs, once a step.
         n_runs = len(model.order)
         safe = [model.run_is_graph_safe(i) for i in range(n_runs)]
-        self._ends_safe = all(getattr(p, "graph_safe", False) for p in (model.embedding, model.final_norm, model.head))
+        self._ends_safe = model.ends_are_graph_safe()
         self._segments = []                 # (captured?, first run, end run)
         for i, ok in enumerate(safe):
             if self._segments and self._segments[-1][0] == ok:
@@ -148,6 +149,14 @@ class Engine:
                 self._input_mixers.append(b.mixer)
                 self._inputs[asked[0]] = torch.full((cap,), -1, dtype=torch.int32, device=rt.device)
                 self._input_hosts[asked[0]] = [torch.full((cap,), -1, dtype=torch.int32).pin_memory() for _ in range(4)]
+        # workspaces mixers want in decoding steps (Mixer.decode_scratch): one per name, sized for the
+        # most requests and the longest context, allocated at the first decoding step
+        self._scratch_sizes: Dict = {}
+        for b in model.blocks:
+            asked = b.mixer.decode_scratch(cfg.max_seqs, self.max_seq_len)
+            if asked is not None:
+                self._scratch_sizes[asked[0]] = max(self._scratch_sizes.get(asked[0], 0), int(asked[1]))
+        self._scratch: Optional[Dict] = None
         self._meta = torch.zeros((3, cfg.max_seqs), dtype=torch.int32, device=rt.device)
         # staging in pinned memory, a ring: a step's inputs and picks travel while the host
         # prepares the next step
@@ -339,6 +348,7 @@ class Engine:
         ctx.decode_index = self._index[:T]
         ctx.decode_shapes = shapes
         ctx.decode_inputs = inputs
+        ctx.decode_scratch = self._scratch
         return ctx
 
     def _decode_forward(self, T: int, spans: List[Span], shapes: Dict, inputs: Dict):
@@ -356,7 +366,7 @@ class Engine:
         last (logits into the static buffer)."""
         _, first, end = self._segments[index]
         if first == 0:
-            self.model.embedding.forward(ctx, out=x)
+            self.model.embed(ctx, out=x)
         self.model.forward_runs(ctx, x, first, end)
         if end == len(self.model.order):
             logits = self.model.logits(ctx, x, ctx.decode_index, out=self._logits[:ctx.n_tokens])
@@ -405,6 +415,9 @@ class Engine:
         captured once and replayed afterwards.  Returns a view of a static logits buffer, valid
         until the next decoding step; `last_picks` holds the greedy pick of each row."""
         T = len(positions)
+        if self._scratch is None:
+            self._scratch = {name: torch.empty(n, dtype=torch.float32, device=self.rt.device)
+                             for name, n in self._scratch_sizes.items()}
         if self._logits is None:
             self._logits = torch.empty((self.cfg.max_seqs, self.model.vocab_size), dtype=torch.float32,
                                        device=self.rt.device)

@@ -6,6 +6,9 @@ Two kinds of library are built from `axon_amd/csrc`:
   (`bfloat16`, `float32`), compiled with hipcc.  A call that needs a dtype compiles that
   dtype only.
 * `libaxon_host.so`: the host runtime (cache manager, scheduler), plain C++.
+* `libaxon_ext_<name>_<dtype>.so`: one library per kernel source that a part outside the package
+  registered (`register_kernel_source`), built like the kernel library, with this package's
+  headers on the include path.
 
 Built files live in `axon_amd/_built/` when that can be written, else in a per-user folder
 under the temporary directory.  A stamp beside each library holds a hash of its sources and
@@ -28,7 +31,10 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 ARCH = "gfx950"
 
 KERNEL_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "attention.hip", "attention_mfma.hip",
-                  "sampling.hip"]
+                  "sampling.hip", "instances.hip", "support.hip"]
+# what a library built from a part's own kernel sources gets beside them (the error channel, the
+# list of its kernel instances)
+EXTENSION_SUPPORT = ["support.hip", "instances.hip"]
 HOST_SOURCES = ["host/cache.cpp", "host/scheduler.cpp", "host/sampler.cpp"]
 
 # Packed 32-bit float instructions are switched off for all device code.  No contraction of a
@@ -71,7 +77,51 @@ def built_dir() -> str:
 
 
 def _existing(sources: List[str]) -> List[str]:
+    """Sources are named relative to the package's csrc, or by an absolute path."""
     return [s for s in sources if os.path.exists(os.path.join(CSRC, s))]
+
+
+# --------------------------------------------------------------------------- a part's own kernels
+# A part that brings HIP kernels of its own adds files and edits none of this package's:
+# `register_kernel_source(path, {entry point: argument types})` names a .hip file anywhere (it may
+# include this package's common.h and api.h; its entry points are extern "C", return 0 or a
+# negative code after axk_set_error, as the package's own do).  The file is compiled per compute
+# dtype into a library of its own, at the first call of one of its entry points
+# (`Kernels.call(name, ...)`).
+_EXTENSIONS: dict = {}        # absolute path -> {entry point: ctypes argument types}
+
+
+def register_kernel_source(path: str, signatures: dict) -> None:
+    path = os.path.abspath(path)
+    if not os.path.isfile(path):
+        raise BuildError(f"register_kernel_source: {path} does not exist")
+    for other, sigs in _EXTENSIONS.items():
+        if other == path:
+            continue
+        if _stem(other) == _stem(path):       # the library is named after the file
+            raise BuildError(f"register_kernel_source: {path} and {other} have the same file name")
+        for name in signatures:
+            if name in sigs:
+                raise BuildError(f"register_kernel_source: {name} is already an entry point of {other}")
+    _EXTENSIONS[path] = {name: list(args) for name, args in signatures.items()}
+
+
+def _stem(path: str) -> str:
+    return "".join(c if c.isalnum() else "_" for c in os.path.splitext(os.path.basename(path))[0])
+
+
+def registered_kernel_sources() -> dict:
+    return dict(_EXTENSIONS)
+
+
+def build_extension(path: str, dtype: str, force: bool = False) -> str:
+    """The library of one registered source for one compute dtype; compiled if missing or stale."""
+    path = os.path.abspath(path)
+    lib_name = f"libaxon_ext_{_stem(path)}_{dtype}.so"
+    flags = HIP_FLAGS + [DTYPE_FLAG[dtype]]
+    sources = [path] + EXTENSION_SUPPORT
+    hipcc = "hipcc" if not force and _fresh(lib_name, sources, flags) else _find("hipcc", ["/opt/rocm/bin/hipcc"])
+    return _build(lib_name, sources, hipcc, flags, [f"--offload-arch={ARCH}", "-fPIC"], force)
 
 
 def _stamp(sources: List[str], flags: List[str]) -> str:
@@ -80,7 +130,7 @@ def _stamp(sources: List[str], flags: List[str]) -> str:
     names = sorted(set(_existing(sources)) | {f for f in os.listdir(CSRC) if f.endswith(".h")}
                    | {os.path.join("host", f) for f in os.listdir(os.path.join(CSRC, "host")) if f.endswith(".h")})
     for s in names:
-        h.update(s.encode())
+        h.update((os.path.basename(s) if os.path.isabs(s) else s).encode())     # a built library travels with the tree
         with open(os.path.join(CSRC, s), "rb") as f:
             h.update(f.read())
     return h.hexdigest()
@@ -124,7 +174,7 @@ def _build(lib_name: str, sources: List[str], compiler: str, flags: List[str], l
     objs = []
 
     def one(src: str) -> str:
-        obj = os.path.join(obj_dir, src.replace("/", "_") + ".o")
+        obj = os.path.join(obj_dir, os.path.relpath(os.path.join(CSRC, src), CSRC).replace("/", "_").replace("..", "up") + ".o")
         _run([compiler] + flags + ["-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj], f"{lib_name}: {src}")
         return obj
 

@@ -30,6 +30,11 @@ def _stream() -> c_void_p:
     return c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+# for the callers of `Kernels.call`: a tensor's (or a packed matrix's) address, the current stream
+ptr, current_stream = _ptr, _stream
+register_kernel_source = build.register_kernel_source
+
+
 _SIGNATURES = {
     "axk_embed": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
     "axk_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_void_p],
@@ -123,18 +128,58 @@ class Kernels:
         self.lib.axk_topk_workspace.restype = ctypes.c_long
         self.lib.axk_argmax_workspace.argtypes = [c_int, c_int]
         self.lib.axk_argmax_workspace.restype = ctypes.c_long
+        self.lib.axk_instances.argtypes = [c_char_p, ctypes.c_long, c_int]
+        self.lib.axk_instances.restype = ctypes.c_long
+        self.lib.axk_instances_reset.argtypes = []
+        self.lib.axk_instances_reset.restype = None
         if bool(self.lib.axk_is_bf16()) != (dtype_name == "bfloat16"):
             raise KernelError(f"{self.path} was not built for {dtype_name}")
+        self._extensions: Dict[str, ctypes.CDLL] = {}      # a registered source's path -> its library
+
+    # ------------------------------------------------------------------ a part's own kernels
+    def call(self, name: str, *args) -> None:
+        """Call the entry point `name` of a kernel source that a part registered
+        (`register_kernel_source(path, {name: argument types})`); its library is compiled for this
+        compute dtype and loaded at the first call.  Arguments as ctypes takes them (`ptr(tensor)`,
+        `current_stream()`, ints, floats).  A refusal raises `KernelError` with the library's message."""
+        for path, signatures in build.registered_kernel_sources().items():
+            if name in signatures:
+                break
+        else:
+            raise KernelError(f"no registered kernel source has an entry point '{name}'")
+        lib = self._extensions.get(path)
+        if lib is None:
+            lib = ctypes.CDLL(build.build_extension(path, self.dtype_name), mode=ctypes.RTLD_LOCAL)
+            lib.axk_last_error.restype = c_char_p
+            if bool(lib.axk_is_bf16()) != (self.dtype_name == "bfloat16"):
+                raise KernelError(f"the library of {path} was not built for {self.dtype_name}")
+            for entry, argtypes in signatures.items():
+                fn = getattr(lib, entry)
+                fn.argtypes, fn.restype = list(argtypes), c_int
+            self._extensions[path] = lib
+        if getattr(lib, name)(*args) != 0:
+            raise KernelError(lib.axk_last_error().decode())
 
     # ------------------------------------------------------------------ helpers
     def _check(self, rc: int) -> None:
         if rc != 0:
             raise KernelError(self.lib.axk_last_error().decode())
 
+    def instances(self, launched: bool = False) -> List[str]:
+        """The kernel instances compiled into the library (the instances of the templates that the
+        dispatches choose from), or those `launched` since `reset_instances`."""
+        need = self.lib.axk_instances(None, 0, 1 if launched else 0)
+        buf = ctypes.create_string_buffer(need)
+        self.lib.axk_instances(buf, need, 1 if launched else 0)
+        return [n for n in buf.value.decode().split("\n") if n]
+
+    def reset_instances(self) -> None:
+        self.lib.axk_instances_reset()
+
     # what launches kernels: wrapped while a step is profiled
     _LAUNCHING = ("embed", "rmsnorm", "rope_table", "rope_kv_write", "gemm_qkv_rope", "attention", "attention_prefill",
                   "attention_decode", "gemm", "gemm_normed_glu", "gemm_normed_qkv_rope", "swiglu", "argmax", "topk",
-                  "fill_i32", "fill_f32")
+                  "fill_i32", "fill_f32", "call")
     _MATRIX_AT = {"gemm": 1, "gemm_qkv_rope": 1, "gemm_normed_glu": 3, "gemm_normed_qkv_rope": 3}   # which argument is W
 
     def set_launch_hook(self, hook) -> None:
@@ -150,7 +195,7 @@ class Kernels:
 
             def told(*a, _plain=plain, _name=name, **kw):
                 out = _plain(self, *a, **kw)
-                label, nbytes = _name, 0
+                label, nbytes = (str(a[0]) if _name == "call" else _name), 0
                 if _name in self._MATRIX_AT:
                     w = a[self._MATRIX_AT[_name]]
                     data = w.data if isinstance(w, PackedMatrix) else w

@@ -99,17 +99,19 @@ class DecoderModel:
             b.load(store, rt)
         self.final_norm.load(store, rt)
         self.head.load(store, rt)
-        # a head tied to the embedding may have repacked the matrix for its product: the embedding
-        # then reads that copy, and the row-major one is dropped
-        if (getattr(self.head, "source_name", None) == getattr(self.embedding, "name", None)
-                and not isinstance(self.head.weight, torch.Tensor)):
-            self.embedding.table = self.head.weight
-            store.forget(self.embedding.name)
+        # a head tied to the embedding may keep the matrix in a form of its own (repacked for its
+        # product): the head says so, the embedding then reads that copy and the other is dropped
+        if self.head.shares_with(self.embedding):
+            self.embedding.read_from(self.head, store)
 
     # ------------------------------------------------------------------ the step
+    def embed(self, ctx, out=None) -> torch.Tensor:
+        """The residual stream before the first run: float32 [T, hidden] (into `out` if given)."""
+        return self.embedding.forward(ctx, out=out)
+
     def forward(self, ctx) -> torch.Tensor:
         """The residual stream after every run: float32 [T, hidden]."""
-        x = self.embedding.forward(ctx)
+        x = self.embed(ctx)
         self.forward_runs(ctx, x, 0, len(self.order))
         return x
 
@@ -133,6 +135,11 @@ class DecoderModel:
         """Whether run i's block and its parts are all fixed launch sequences (see Part.graph_safe)."""
         block = self.blocks[self.order[i].layer]
         return all(getattr(p, "graph_safe", False) for p in (block, block.mixer, block.feed_forward))
+
+    def ends_are_graph_safe(self) -> bool:
+        """Whether what runs before the first run and behind the last (`embed`, `logits`) is a fixed
+        launch sequence too, so that it can be captured with the runs beside it."""
+        return all(getattr(p, "graph_safe", False) for p in (self.embedding, self.final_norm, self.head))
 
     def logits(self, ctx, x: torch.Tensor, rows: torch.Tensor, out=None) -> torch.Tensor:
         """Final norm and head at the rows asked for: float32 [len(rows), vocab]."""

@@ -71,7 +71,11 @@ class AttentionPlan:
                 self.decode_work = torch.tensor(work, dtype=torch.int32).to(dev)
         if n_single:
             n = ctx.rt.k.attention_decode_workspace(n_single, n_heads, head_dim, self.max_chunks)
-            self.partial = torch.empty(n, dtype=torch.float32, device=dev)
+            lasting = ctx.decode_scratch.get(("attention_partial", window, n_heads, head_dim)) if ctx.decode_only else None
+            if lasting is not None and lasting.numel() >= n:
+                self.partial = lasting           # one workspace for every decoding step and graph
+            else:
+                self.partial = torch.empty(n, dtype=torch.float32, device=dev)
 
 
 def pair_tiles(tiles, seen):
@@ -131,6 +135,7 @@ class GQAttention(Mixer):
         self.n = {k: base + names.get(k, k + "_proj") for k in ("q", "k", "v", "o")}
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
         self._max_context = None
+        self._workspace = None
         self.decode_chunk = 1 << 30          # until `load` has asked the kernels: one chunk
         self._work_list = lambda positions, window: list(range(len(positions)))
 
@@ -172,10 +177,21 @@ class GQAttention(Mixer):
     def decode_input_capacity(self, max_seqs: int, max_seq_len: int) -> int:
         return round_up_by_eighths(max_seqs * decode_chunks_of(max(0, max_seq_len - 1), 0, self.decode_chunk))
 
+    def decode_scratch(self, max_seqs: int, max_seq_len: int):
+        """The blocks' partial results of the decoding kernel, laid out by the longest context in
+        chunks rounded up to a power of two (see `decode_shape`)."""
+        if self._workspace is None:              # no kernel of this build and these sizes wants one
+            return None
+        most = decode_chunks_of(max(0, max_seq_len - 1), self.window, self.decode_chunk)
+        chunks = 1 << (most - 1).bit_length()
+        return ("attention_partial", self.window, self.nh, self.hd), self._workspace(max_seqs, self.nh, self.hd, chunks)
+
     def load(self, store, rt) -> None:
         self.decode_chunk = rt.k.attention_decode_chunk
         self._work_list = rt.k.attention_decode_work
         self._max_context = rt.k.attention_decode_max_context
+        if rt.k.attention_fast_ok(self.hd, 64, self.nh, self.nkv):
+            self._workspace = rt.k.attention_decode_workspace
         self.w_qkv = rt.k.prepare_weight(store.fused_matrix([self.n[k] + ".weight" for k in ("q", "k", "v")]))
         biases = [store.vector(self.n[k] + ".bias", optional=True) for k in ("q", "k", "v")] if self.qkv_bias else []
         present = [b is not None for b in biases]

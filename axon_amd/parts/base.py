@@ -176,6 +176,13 @@ class Mixer(Part):
         this many positions each."""
         return 0
 
+    def decode_scratch(self, max_seqs: int, max_seq_len: int) -> Optional[Tuple[Any, int]]:
+        """(name, float32 elements) of a workspace this mixer's kernels want in steps of single
+        tokens, sized for this many live requests of up to this many positions each, or None.  The
+        engine allocates one per name, once, and hands it back as `ctx.decode_scratch[name]`: every
+        decoding step and every captured graph then uses the same memory, whatever its shape."""
+        return None
+
     def finishes_following_norm(self, ctx) -> bool:
         """Whether `forward` takes a FollowingNorm as a further argument in this step: its last
         product also writes the finished norm of the rows it has added into.  Optional."""

@@ -11,7 +11,7 @@ from typing import List
 
 import torch
 
-from ..kernels import MODE_STORE_F32
+from ..kernels import MODE_STORE_F32, PackedMatrix
 from .base import Part, TensorDecl, register_embedding, register_head
 
 
@@ -29,6 +29,12 @@ class TokenEmbedding(Part):
 
     def load(self, store, rt) -> None:
         self.table = store.matrix(self.name)
+
+    def read_from(self, head, store) -> None:
+        """Read the rows out of `head`'s copy of this matrix (a head that `shares_with` this
+        embedding); the copy loaded here is dropped."""
+        self.table = head.weight
+        store.forget(self.name)
 
     def forward(self, ctx, out=None):
         if out is None:
@@ -61,6 +67,12 @@ class LMHead(Part):
         # packed for the matrix-core products where it can be; a tied embedding then reads the
         # packed matrix too (the model hands it over), so that the matrix is in memory once
         self.weight = rt.k.prepare_weight(weight)
+
+    def shares_with(self, embedding) -> bool:
+        """Whether this head was loaded from `embedding`'s tensor and keeps it in a form that the
+        embedding kernel reads as well (packed): the matrix then need be in memory only once."""
+        return (self.source_name is not None and self.source_name == getattr(embedding, "name", None)
+                and isinstance(self.weight, PackedMatrix))
 
     def forward(self, ctx, h, out=None):
         """h: [rows, hidden] in the compute dtype -> float32 logits [rows, vocab]."""

@@ -61,9 +61,12 @@ def prompts_for(name: str, lengths, seed: int = 0):
 
 def tolerance(dtype: str, ref: torch.Tensor) -> float:
     """The allowed max |difference| of logits: float32 within rounding of a float64 oracle;
-    bfloat16 (8 bits of mantissa in every stored activation) within 2 % of the logits' scale."""
-    scale = max(1.0, float(ref.abs().max()))
-    return (2e-5 if dtype == "float32" else 2e-2) * scale
+    bfloat16 (8 bits of mantissa in every stored activation) within 1 % of the range the logits
+    span, three times what grading bfloat16 against float32 observes on these configurations
+    (tests/test_invariance_gpu.py: at most 0.31 % of the range)."""
+    if dtype == "float32":
+        return 2e-5 * max(1.0, float(ref.abs().max()))
+    return 1e-2 * max(float(ref.max() - ref.min()), 1e-3)
 
 
 def engine_for(model_dir: str, dtype: str, page_size: int, num_pages: int, max_seqs: int = 4, **kw):

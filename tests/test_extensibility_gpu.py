@@ -6,6 +6,7 @@ built, loaded from a folder written by the random-weights mode and stepped, with
 to the framework's files, and compared with a plain implementation written here."""
 import json
 import os
+from ctypes import c_float, c_int, c_void_p
 
 import pytest
 import torch
@@ -14,6 +15,7 @@ import axon_amd
 from axon_amd.config import (LayerSpec, ModelConfig, ModelSpec, PartSpec, Run, register_architecture)
 from axon_amd.config.base import get_number, get_whole
 from axon_amd.engine import StepEntry
+from axon_amd.kernels import MODE_ADD_F32, MODE_STORE_F32, KernelError, current_stream, ptr, register_kernel_source
 from axon_amd.parts import (FeedForward, Mixer, StateSpec, TensorDecl, build_part, register_feed_forward, register_mixer,
                             register_position)
 from axon_amd.parts.rope import RotaryEncoding
@@ -25,9 +27,17 @@ pytestmark = pytest.mark.gpu
 
 
 # --------------------------------------------------------------------------- toy parts
+# The toy mixer brings a HIP kernel of its own: a file in the tests' folder, registered with its entry
+# point's argument types.  The engine compiles it (per compute dtype, at the first call) into a
+# library of its own; no file of the framework names it.
+register_kernel_source(os.path.join(os.path.dirname(os.path.abspath(__file__)), "toy_kernels", "decay_scan.hip"),
+                       {"toy_decay_scan": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_int, c_void_p]})
+
+
 class DecayMixer(Mixer):
     """A toy recurrent mixer: s_t = decay * s_{t-1} + W_in h_t, out_t = W_out s_t.  Its state
-    (one vector per request) lives in the cache manager's state slots; it has no pages."""
+    (one vector per request) lives in the cache manager's state slots; it has no pages.  The two
+    products are the engine's own kernels, the scan over a request's tokens its own."""
 
     def __init__(self, params, prefix=""):
         super().__init__(params, prefix)
@@ -41,7 +51,7 @@ class DecayMixer(Mixer):
         return StateSpec(self.width)
 
     def load(self, store, rt):
-        self.w_in, self.w_out = store.matrix(self.n_in).float(), store.matrix(self.n_out).float()
+        self.w_in, self.w_out = store.matrix(self.n_in), store.matrix(self.n_out)       # in the compute dtype
 
     # values of its own on the device in steps of single tokens (here only to show the way: the
     # positions, padded to a multiple of four)
@@ -54,16 +64,15 @@ class DecayMixer(Mixer):
     def forward(self, ctx, binding, h, residual):
         if ctx.decode_only:
             self.seen_on_device = ctx.decode_inputs["toy_positions"].clone()
-        arena = ctx.cache.state(binding.state_index)
-        u = h.float() @ self.w_in.T
-        for span in ctx.spans:                                   # each request's tokens, in order
-            s = arena[span.slot, :self.width].clone()
-            outs = []
-            for t in range(span.q_start, span.q_start + span.q_len):
-                s = self.decay * s + u[t]
-                outs.append(s)
-            arena[span.slot, :self.width] = s
-            residual[span.q_start:span.q_start + span.q_len] += torch.stack(outs) @ self.w_out.T
+        k, T = ctx.rt.k, h.shape[0]
+        arena = ctx.cache.state(binding.state_index)             # [slots, elements] float32
+        u = torch.empty((T, self.width), dtype=torch.float32, device=h.device)
+        k.gemm(h, self.w_in, u, None, MODE_STORE_F32)
+        spans = torch.tensor([[s.slot, s.q_start, s.q_len] for s in ctx.spans], dtype=torch.int32).to(h.device)
+        outs = torch.empty((T, self.width), dtype=ctx.rt.dtype, device=h.device)
+        k.call("toy_decay_scan", ptr(u), ptr(arena), arena.stride(0), ptr(spans), len(ctx.spans), self.decay, ptr(outs),
+               self.width, current_stream())                     # each request's tokens, in order
+        k.gemm(outs, self.w_out, residual, None, MODE_ADD_F32)
 
 
 class HalvedRope(RotaryEncoding):
@@ -294,3 +303,29 @@ def test_the_toy_model_steps_like_its_plain_twin(toy_dir, dtype):
             for tok in o:
                 assert tok == P.argmax_last(toy_plain(w, hist)[-1].float())
                 hist.append(tok)
+
+
+def test_a_parts_own_kernel_source_is_built_and_called_without_a_change_to_the_framework(toy_dir):
+    """The registered source compiles into a library of its own for each compute dtype, its entry
+    point is reached through `Kernels.call`, refuses what it says it refuses with its own message,
+    and an unknown name is an error."""
+    from axon_amd.kernels import kernels
+    for dtype, torch_dtype in (("float32", torch.float32), ("bfloat16", torch.bfloat16)):
+        k = kernels(dtype)
+        u = torch.arange(12, dtype=torch.float32).view(4, 3).cuda()
+        state = torch.tensor([[1.0, 2.0, 3.0, 0.0], [0.0, 0.0, 0.0, 0.0]]).cuda()           # stride 4, width 3
+        spans = torch.tensor([[1, 0, 1], [0, 1, 3]], dtype=torch.int32).cuda()
+        out = torch.zeros(4, 3, dtype=torch_dtype, device="cuda")
+        k.call("toy_decay_scan", ptr(u), ptr(state), 4, ptr(spans), 2, 0.5, ptr(out), 3, current_stream())
+        want, s = [], torch.tensor([1.0, 2.0, 3.0])
+        for t in (1, 2, 3):
+            s = 0.5 * s + u[t].cpu()
+            want.append(s)
+        assert torch.equal(out[0].float().cpu(), u[0].cpu())                                # slot 1 started from zero
+        assert torch.equal(out[1:].float().cpu(), torch.stack(want).to(torch_dtype).float())
+        assert torch.equal(state[0, :3].cpu(), s) and state[0, 3] == 0
+        with pytest.raises(KernelError, match="toy_decay_scan: 1 spans, width 5, state stride 4"):
+            k.call("toy_decay_scan", ptr(u), ptr(state), 4, ptr(spans), 1, 0.5, ptr(out), 5, current_stream())
+        with pytest.raises(KernelError, match="no registered kernel source"):
+            k.call("toy_missing")
+

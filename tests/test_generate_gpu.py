@@ -259,8 +259,14 @@ def test_a_step_that_does_not_fit_takes_nothing(model_dirs):
         want = fresh.step([StepEntry(rid, prompt, [len(prompt) - 1])], end=[rid])
         assert torch.equal(got, want)
     assert cache.free_pages(0) == 6
-    with pytest.raises(Exception):                                                       # longer than any kernel's list of work
-        engine_for(d, "bfloat16", page_size=8, num_pages=6, max_seq_len=1 << 20)
+    # a context longer than the attention kernels' list of work can name is refused when the engine is
+    # built, with that reason; the longest one they take is accepted
+    from axon_amd.engine.step import StepError
+    from axon_amd.kernels import kernels
+    limit = kernels("bfloat16").attention_decode_max_context
+    with pytest.raises(StepError, match="contexts of up to"):
+        engine_for(d, "bfloat16", page_size=8, num_pages=6, max_seq_len=limit + 1)
+    assert engine_for(d, "bfloat16", page_size=8, num_pages=6, max_seq_len=limit).max_seq_len == limit
 
 
 def test_logits_are_the_callers_own(model_dirs):

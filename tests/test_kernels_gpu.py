@@ -230,6 +230,28 @@ def test_gemm_rows_do_not_depend_on_the_batch(dtype):
             assert torch.equal(part, whole[:m]), (N, K, m)
 
 
+@pytest.mark.parametrize("N", [16400, 152064])
+@pytest.mark.parametrize("K", [256, 3584])
+def test_products_with_the_rows_of_a_real_vocabulary(N, K):
+    """From 16,384 rows of W on the products for up to 16 rows and for 17 to 64 take two row tiles a
+    wave: the head of every real model runs through those.  1 to 65 rows against the float64 product
+    (computed on the device: W has up to a gigabyte), and a row bit for bit whatever its step."""
+    k = kernels("bfloat16")
+    g = torch.Generator(device="cuda").manual_seed(21)
+    x = torch.randn(65, K, generator=g, device="cuda").bfloat16()
+    w = (torch.randn(N, K, generator=g, device="cuda") * 0.05).bfloat16()
+    want = x.double() @ w.double().T
+    wp = k.prepare_weight(w)
+    del w
+    whole = torch.empty(65, N, dtype=torch.float32, device="cuda")
+    k.gemm(x, wp, whole, None, MODE_STORE_F32)
+    assert float((whole.double() - want).abs().max()) <= 2e-5 * math.sqrt(K) * max(1.0, float(want.abs().max()))
+    for m in (1, 8, 16, 17, 64):
+        part = torch.empty(m, N, dtype=torch.float32, device="cuda")
+        k.gemm(x[:m], wp, part, None, MODE_STORE_F32)
+        assert torch.equal(part, whole[:m]), (N, K, m)
+
+
 # the products of a layer of the measured sizes (hidden, q rows, kv rows, feed-forward width, head_dim)
 LAYER_SIZES = {"7b": (3584, 3584, 512, 18944, 128), "14b": (5120, 5120, 1024, 13824, 128)}
 
@@ -640,13 +662,18 @@ def test_the_page_size_does_not_change_a_bit_of_the_attention(nh, nkv, hd, T, wi
     assert all(torch.equal(results[0], r) for r in results[1:])
 
 
-def test_matrix_core_attention_finds_a_far_key_and_respects_the_windows_edge():
+@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("far", [15, 63, 64, 255, 256])
+def test_matrix_core_attention_finds_a_far_key_and_respects_the_windows_edge(hd, far):
+    """One loud key hundreds of positions back, in the first blocks of the context: found without a
+    window, excluded when the window starts one position after it, found when it starts at it.
+    `far` puts that edge inside a block of 64 positions (15), at the last place of a block and the
+    first of the next (63, 64) and at the edge of the decoding kernel's chunks of 256 (255, 256)."""
     k = kernels("bfloat16")
-    nh, nkv, hd, page, T = 4, 2, 128, 16, 700
+    nh, nkv, page, T = 4, 2, 16, 700
     q = rnd(T, nh, hd, seed=7) * 0.1
     kk = rnd(T, nkv, hd, seed=8) * 0.1
     vv = rnd(T, nkv, hd, seed=9)
-    far = 15
     kk[far, 1] = 0
     kk[far, 1, 3] = 40.0
     q[T - 1, 2] = 0
@@ -662,7 +689,9 @@ def test_matrix_core_attention_finds_a_far_key_and_respects_the_windows_edge():
     tile = torch.tensor([[T - 40, 40]], dtype=torch.int32).cuda()
     partial = torch.empty(k.attention_decode_workspace(1, nh, hd, 16), dtype=torch.float32, device="cuda")
     for w, seen in ((0, True), (T - 1 - far, False), (T - far, True)):
-        ref = P.causal_attention(qr, kr, vr, w)[T - 1]
+        # the last token alone: its row of the plain formula
+        lo = 0 if w == 0 else max(0, T - w)
+        ref = torch.stack([torch.softmax((kr[lo:T, h // 2] @ qr[T - 1, h]) * scale, 0) @ vr[lo:T, h // 2] for h in range(nh)])
         for which in ("decode", "prefill"):
             out = torch.zeros(T, nh * hd, dtype=torch.bfloat16, device="cuda")
             if which == "decode":

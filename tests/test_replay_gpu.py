@@ -153,7 +153,9 @@ def test_every_schedule_matches_the_plain_implementation(name, dtype, model_dirs
                       ("portions", changing_portions(prompts)), ("mixed", mixed(prompts, seed=len(name))),
                       ("refed", given_up_and_fed_again(prompts, seed=len(name)))):
         budget = max_tokens_for(tb, None)
-        out = run_trace(model_dir, dtype, tb.steps, str(tmp_path / label), budget, extra=page)
+        # the mixed schedule with pages handed out in a shuffled order, and its decoding steps from graphs
+        more = ["--shuffle-pages", "5", "--graphs"] if label == "mixed" else []
+        out = run_trace(model_dir, dtype, tb.steps, str(tmp_path / label), budget, extra=page + more)
         rows = tb.collect(out)
         check(rows, refs, ids, dtype)
         results[label] = rows
