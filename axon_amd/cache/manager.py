@@ -77,6 +77,8 @@ def host_lib():
             "axh_rng_next_f64": (ctypes.c_double, [c_void_p]),
             "axh_sample_pick_keys": (c_int, [c_void_p, c_int, ctypes.c_float, ctypes.c_float, ctypes.c_float,
                                              ctypes.c_double]),
+            "axh_sample_pick_keys_rows": (None, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                 c_void_p]),
             "axh_sample_pick_row": (c_int, [c_void_p, c_int, c_void_p, c_int, ctypes.c_float, c_int, ctypes.c_float,
                                             ctypes.c_float, ctypes.c_float, ctypes.c_double]),
             "axh_argmax_row": (c_int, [c_void_p, c_int]),
@@ -120,6 +122,13 @@ class CacheGroup:
             self.storage = torch.zeros((plan.n_layers, s.entries, plan.n_pages, s.heads, plan.page_size, s.head_dim),
                                        dtype=dtype if s.dtype is None else getattr(torch, s.dtype), device=device)
             self.block_table = torch.zeros((max_seqs, max_pages_per_seq), dtype=torch.int32, device=device)
+            # staging of changed rows on their way to the device (CacheManager.sync_tables): max_seqs rows
+            # and, in a last row, the slots they belong to
+            shape = (max_seqs + 1, max(max_pages_per_seq, max_seqs))
+            self.stages = [torch.zeros(shape, dtype=torch.int32).pin_memory() for _ in range(4)]
+            self.stage_events = [None] * 4
+            self.stage_at = 0
+            self.stage_device = torch.zeros(shape, dtype=torch.int32, device=device)
 
     def layer(self, index: int) -> Tuple[torch.Tensor, ...]:
         """The arrays of one layer of the group: for attention (keys, values), each
@@ -242,16 +251,35 @@ class CacheManager:
         if not self._dirty:
             return
         slots = sorted(self._dirty)
+        n = len(slots)
         for gi, g in enumerate(self.groups):
-            rows = torch.zeros((len(slots), self.max_pages_per_seq), dtype=torch.int32)
+            if g.block_table is None:
+                rows = torch.zeros((n, self.max_pages_per_seq), dtype=torch.int32)
+            else:
+                # Through pinned memory, without waiting for the device: the rows as they are now go into
+                # one of a ring of staging buffers (with the slots they belong to in the buffer's last
+                # row), one copy brings them over and a scatter puts them in place, in stream order.
+                # A staging buffer is written again only after the copy that read it has run.
+                at = g.stage_at = (g.stage_at + 1) % len(g.stages)
+                if g.stage_events[at] is not None:
+                    g.stage_events[at].synchronize()
+                stage = g.stages[at]
+                rows = stage[:n, :self.max_pages_per_seq]
+                rows.zero_()
+                stage[self.max_seqs, :n] = torch.tensor(slots, dtype=torch.int32)
             for i, slot in enumerate(slots):
-                n = self.lib.axh_cache_row(self._h, gi, slot, c_void_p(rows[i].data_ptr()), self.max_pages_per_seq)
-                if n < 0:
+                got = self.lib.axh_cache_row(self._h, gi, slot, c_void_p(rows[i].data_ptr()), self.max_pages_per_seq)
+                if got < 0:
                     raise CacheError(f"no block table row for group {gi}, slot {slot}")
             g.host_table[slots] = rows
             if g.block_table is not None:
-                index = torch.tensor(slots, dtype=torch.int64).to(self.device)
-                g.block_table.index_copy_(0, index, rows.to(self.device))
+                g.stage_device[:n].copy_(stage[:n], non_blocking=True)
+                g.stage_device[self.max_seqs].copy_(stage[self.max_seqs], non_blocking=True)
+                event = g.stage_events[at] or torch.cuda.Event()
+                event.record()
+                g.stage_events[at] = event
+                g.block_table.index_copy_(0, g.stage_device[self.max_seqs, :n].long(),
+                                          g.stage_device[:n, :self.max_pages_per_seq])
         self._dirty.clear()
 
     # ------------------------------------------------------------------ accounting

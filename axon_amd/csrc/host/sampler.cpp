@@ -141,6 +141,16 @@ int axh_sample_pick_keys(const uint64_t* keys, int k, float temp, float top_p, f
   return pick_sorted(sorted, temp, top_p, min_p, u);
 }
 
+// The picks of a step's rows in one call: row r has k[r] candidate keys at keys + r * k_stride and
+// takes one number from its own stream states[r] (four 64-bit words), as one
+// axh_sample_pick_keys(.., axh_rng_next_f64(states[r])) per row would.
+void axh_sample_pick_keys_rows(const uint64_t* keys, int k_stride, int n_rows, const int* k, const float* temp,
+                               const float* top_p, const float* min_p, uint64_t* const* states, int* picks) {
+  for (int r = 0; r < n_rows; ++r)
+    picks[r] = axh_sample_pick_keys(keys + (size_t)r * k_stride, k[r], temp[r], top_p[r], min_p[r],
+                                    axh_rng_next_f64(states[r]));
+}
+
 // The whole pipeline on a row of logits held by the host (top_k 0: every token is a
 // candidate).  `recent`: the ids the penalty looks at (already cut to the last N); the
 // penalty divides a positive logit and multiplies any other (src/sample.rs:307-326).

@@ -17,11 +17,12 @@ from typing import Dict, List, Optional, Sequence, Union
 import torch
 
 from ..config import EngineConfig, ModelConfig, config_from_dict
-from ..sampling import Sampler, SamplingParams, pick_rows
+from ..cache.manager import OutOfPages
+from ..sampling import PendingRowPicks, Sampler, SamplingParams
 from .loading import load_model, random_model
 from .runtime import Runtime
 from .scheduler import Scheduler
-from .step import Engine, StepEntry
+from .step import Engine, StepEntry, StepError
 
 
 @dataclass
@@ -143,6 +144,13 @@ class LLM:
         trace = StepTrace.from_env()
         ahead_ok = trace is None
         behind = None            # (picks on their way, the requests they belong to)
+        # Sampled tokens are drawn on the host, so a step cannot start before the one before it has
+        # ended.  What it can do is have everything but its tokens ready by then: while the device
+        # runs a decoding step whose rows will all decode again, the next step is prepared
+        # (Engine.prepare_continue: pages, tables, positions), and once the tokens are drawn it
+        # only takes them and starts.  If the next plan is another after all (a request drew a stop
+        # token, one was admitted) the prepared step is dropped.
+        prepared = None          # the requests of a step that is ready but for its tokens
         # The clocks of `GenStats`.  Steps are queued ahead of the device, so a step's own time is not
         # known on the host; what is known is when the host had to wait.  Everything between two
         # marks is charged to the kind of step (decoding only, or feeding prompts) that was being
@@ -184,6 +192,11 @@ class LLM:
                 plan, preempted = sched.plan([cache.free_pages(g) for g in range(n_groups)])
                 feed = (behind is not None and not preempted and [p.id for p in plan] == behind[1]
                         and all(p.count == 1 and p.wants_logits for p in plan))
+                take_prepared = (prepared is not None and not preempted and [p.id for p in plan] == prepared
+                                 and all(p.count == 1 and p.wants_logits for p in plan))
+                if prepared is not None and not take_prepared:
+                    self.engine.drop_prepared()
+                prepared = None
                 stopped = []
                 if behind is not None and not feed:
                     stopped = settle(behind)
@@ -214,6 +227,8 @@ class LLM:
                     logits = self.engine.step_from_picks([p.id for p in plan])
                     stopped = settle(behind)     # the step before: read while this one runs
                     behind = None
+                elif take_prepared:
+                    logits = self.engine.run_prepared([reqs[p.id].tokens[p.start] for p in plan])
                 else:
                     entries = [StepEntry(p.id, reqs[p.id].tokens[p.start:p.start + p.count],
                                          [p.count - 1] if p.wants_logits else []) for p in plan]
@@ -229,8 +244,19 @@ class LLM:
                     elif greedy_step and self.engine.last_picks is not None:
                         picks = self.engine.last_picks.tolist()     # a decoding step picked greedily already
                     else:
-                        picks = pick_rows(self.rt, logits, [reqs[p.id].sampler for p in wanted],
-                                          [reqs[p.id].tokens for p in wanted])
+                        on_their_way = PendingRowPicks(self.rt, logits, [reqs[p.id].sampler for p in wanted],
+                                                       [reqs[p.id].tokens for p in wanted])
+                        # the device is busy with the step and the candidates: time to prepare the next step
+                        if (ahead_ok and len(wanted) == len(plan) and all(p.count == 1 for p in plan)
+                                and all(len(reqs[p.id].out) + 1 < reqs[p.id].max_new for p in plan)
+                                and sched.counts()[0] == 0
+                                and all(cache.free_pages(g) >= 2 * len(plan) + 2 for g in range(n_groups))):
+                            try:
+                                self.engine.prepare_continue([p.id for p in plan])
+                                prepared = [p.id for p in plan]
+                            except (OutOfPages, StepError):
+                                prepared = None
+                        picks = on_their_way.finish()
                 at = 0
                 for p in plan:
                     r = reqs[p.id]
@@ -274,6 +300,7 @@ class LLM:
                 torch.cuda.synchronize()
                 charge(clock["kind"])
         finally:
+            self.engine.drop_prepared()
             for rid in order:
                 self.engine.release(rid)
         stats.seconds = time.time() - t0

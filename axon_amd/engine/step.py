@@ -166,6 +166,7 @@ class Engine:
         self._ring_at = 0
         self._last_decode: Optional[List[Hashable]] = None      # the requests of the last decoding step, in order
         self._pending: Optional[PendingPicks] = None
+        self._prepared = None             # a decoding step that is ready but for its tokens (prepare_continue)
         self._index = torch.arange(cfg.max_seqs, dtype=torch.int32, device=rt.device)
         self._logits = None
         self._picks = torch.zeros(cfg.max_seqs, dtype=torch.int32, device=rt.device)
@@ -247,6 +248,7 @@ class Engine:
         self.last_picks = None
         self._last_decode = None
         self._pending = None
+        self._prepared = None
         if entries:
             tokens, positions, rows, want_rows, spans = [], [], [], [], []
             for e in entries:
@@ -316,9 +318,19 @@ class Engine:
         on the device, so the host need not have read it yet: it can queue this step and read
         the previous step's picks (`picks_async`) while this one runs.  Returns the logits as
         `step` does."""
+        self.prepare_continue(ids)
+        return self.run_prepared(None)
+
+    def prepare_continue(self, ids: Sequence[Hashable]) -> None:
+        """Everything of one more decoding step of the last decoding step's requests (the same
+        ones, in the same order) that does not depend on their next tokens: pages, block tables,
+        positions, what the mixers want on the device.  The host can do this while the device
+        still runs the step before and the tokens are not decided yet; `run_prepared(tokens)`
+        then starts the step.  Raises (and leaves everything as it was) if it cannot be done:
+        OutOfPages, a request at its longest."""
         ids = list(ids)
         if self._last_decode is None or ids != self._last_decode:
-            raise StepError("step_from_picks continues the last decoding step: the same requests in the same order")
+            raise StepError("a decoding step is continued by the same requests in the same order")
         reqs = [self.live[rid] for rid in ids]
         for rid, req in zip(ids, reqs):
             if req.n_cached + 1 > self.max_seq_len:
@@ -328,13 +340,31 @@ class Engine:
         rows = [req.slot for req in reqs]
         spans = [Span(req.slot, i, 1, req.n_cached) for i, req in enumerate(reqs)]
         self.cache.sync_tables()
-        logits = self._decode_step(None, positions, rows, spans)
+        self._prepared = (ids, reqs, self._decode_prepare(positions, rows, spans))
+
+    def run_prepared(self, tokens: Optional[Sequence[int]]) -> torch.Tensor:
+        """Start the step that `prepare_continue` prepared, with these tokens (one a request, in
+        order), or with the greedy picks of the step before, taken on the device, if None."""
+        if self._prepared is None:
+            raise StepError("run_prepared follows prepare_continue")
+        ids, reqs, prepared = self._prepared
+        self._prepared = None
+        if tokens is not None:
+            tokens = [int(t) for t in tokens]
+            if len(tokens) != len(ids) or any(not 0 <= t < self.model.vocab_size for t in tokens):
+                raise StepError(f"run_prepared: {len(ids)} requests need a token of the vocabulary each")
+        logits = self._decode_launch(prepared, tokens)
         for req in reqs:
             req.n_cached += 1
             if self.has_window:
                 self.cache.trim(req.slot, req.n_cached)
         self.steps += 1
         return logits
+
+    def drop_prepared(self) -> None:
+        """Forget a prepared step that will not run (the pages it reserved stay with their
+        requests, which use them at their next token or give them back at their end)."""
+        self._prepared = None
 
     def picks_async(self) -> Optional[PendingPicks]:
         """The last decoding step's greedy picks as a copy that is under way (None after any
@@ -414,6 +444,11 @@ class Engine:
         device buffers; with graphs on, the launches of this (number of tokens, shape) are
         captured once and replayed afterwards.  Returns a view of a static logits buffer, valid
         until the next decoding step; `last_picks` holds the greedy pick of each row."""
+        return self._decode_launch(self._decode_prepare(positions, rows, spans), tokens)
+
+    def _decode_prepare(self, positions, rows, spans):
+        """What a step of single tokens needs beside the tokens: positions and slots on their way
+        to the device, the step's shape, the values the mixers asked for."""
         T = len(positions)
         if self._scratch is None:
             self._scratch = {name: torch.empty(n, dtype=torch.float32, device=self.rt.device)
@@ -427,14 +462,8 @@ class Engine:
         if self._ring_events[at] is not None:
             self._ring_events[at].synchronize()
         host = self._meta_hosts[at]
-        if tokens is None:
-            # the tokens are the previous step's picks, already on the device
-            host[1:, :T] = torch.tensor([positions, rows], dtype=torch.int32)
-            self._meta[1:].copy_(host[1:], non_blocking=True)
-            self._meta[0, :T].copy_(self._picks[:T])
-        else:
-            host[:, :T] = torch.tensor([tokens, positions, rows], dtype=torch.int32)
-            self._meta.copy_(host, non_blocking=True)
+        host[1:, :T] = torch.tensor([positions, rows], dtype=torch.int32)
+        self._meta[1:].copy_(host[1:], non_blocking=True)
         shapes = {}
         for mixer in self._shape_mixers:
             name, value = mixer.decode_shape(positions)
@@ -446,10 +475,21 @@ class Engine:
             if n > self._inputs[name].numel():
                 raise StepError(f"{name}: {n} values for the device, room for {self._inputs[name].numel()}")
             staged = self._input_hosts[name][at]
-            staged[:n] = torch.tensor(values, dtype=torch.int32)
+            staged[:n] = torch.as_tensor(values, dtype=torch.int32)
             self._inputs[name][:n].copy_(staged[:n], non_blocking=True)
             inputs[name] = self._inputs[name][:n]
             shapes[("values of", name)] = n          # a graph reads exactly this many
+        return T, at, spans, shapes, inputs
+
+    def _decode_launch(self, prepared, tokens) -> torch.Tensor:
+        T, at, spans, shapes, inputs = prepared
+        host = self._meta_hosts[at]
+        if tokens is None:
+            # the tokens are the previous step's picks, already on the device
+            self._meta[0, :T].copy_(self._picks[:T])
+        else:
+            host[0, :T] = torch.tensor(tokens, dtype=torch.int32)
+            self._meta[0].copy_(host[0], non_blocking=True)
         if not self.graphs_ok:
             logits = self._decode_forward(T, spans, shapes, inputs)
         else:

@@ -11,6 +11,7 @@ import ctypes
 from ctypes import c_char_p, c_float, c_int, c_void_p
 from typing import Dict, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from . import build
@@ -135,6 +136,7 @@ class Kernels:
         if bool(self.lib.axk_is_bf16()) != (dtype_name == "bfloat16"):
             raise KernelError(f"{self.path} was not built for {dtype_name}")
         self._extensions: Dict[str, ctypes.CDLL] = {}      # a registered source's path -> its library
+        self._chunk_factor = None
 
     # ------------------------------------------------------------------ a part's own kernels
     def call(self, name: str, *args) -> None:
@@ -424,6 +426,11 @@ class Kernels:
             float(scale), _stream()))
         return out
 
+    def _decode_chunk_and_factor(self):
+        if self._chunk_factor is None:
+            self._chunk_factor = (int(self.lib.axk_attention_decode_chunk()), int(self.lib.axk_attention_decode_item_factor()))
+        return self._chunk_factor
+
     @property
     def attention_decode_chunk(self) -> int:
         """Positions of one chunk of the decoding kernel: a token's range (from the chunk that
@@ -442,15 +449,18 @@ class Kernels:
         """The work list of the decoding kernel for single tokens at `positions` (in the order
         of their slots): one item per (token, chunk), slot * factor + chunk, a token's chunks
         side by side; padded with -1 to `pad_to` items."""
-        chunk, factor = self.attention_decode_chunk, int(self.lib.axk_attention_decode_item_factor())
-        items = []
-        for slot, pos in enumerate(positions):
-            lo = max(0, pos + 1 - window) if window > 0 else 0
-            n = (pos - lo // chunk * chunk) // chunk + 1
-            if n > factor:
-                raise KernelError(f"attention_decode: a context of {pos + 1} positions is more than {factor} chunks")
-            items.extend(slot * factor + c for c in range(n))
-        return items + [-1] * max(0, pad_to - len(items))
+        chunk, factor = self._decode_chunk_and_factor()
+        pos = np.asarray(positions, dtype=np.int64)
+        lo = np.maximum(0, pos + 1 - window) if window > 0 else np.zeros_like(pos)
+        n = (pos - lo // chunk * chunk) // chunk + 1
+        if n.size and int(n.max()) > factor:
+            raise KernelError(f"attention_decode: a context of {int(pos.max()) + 1} positions is more than {factor} chunks")
+        total = int(n.sum())
+        first = np.cumsum(n) - n                                   # where each token's items start
+        items = np.repeat(np.arange(pos.size, dtype=np.int64) * factor - first, n) + np.arange(total, dtype=np.int64)
+        out = np.full(max(total, pad_to), -1, dtype=np.int32)
+        out[:total] = items
+        return out.tolist()
 
     def attention_decode(self, q, q_stride, k_cache, v_cache, block_table, positions, seq_rows, out, token_index,
                          partial, max_chunks, n_heads, n_kv_heads, head_dim, page_size, window, scale,

@@ -1,3 +1,3 @@
-from .sampler import Rng, Sampler, SamplingParams, argmax_row, pick_rows, random_seed
+from .sampler import PendingRowPicks, Rng, Sampler, SamplingParams, argmax_row, pick_rows, random_seed
 
-__all__ = ["Rng", "Sampler", "SamplingParams", "argmax_row", "pick_rows", "random_seed"]
+__all__ = ["PendingRowPicks", "Rng", "Sampler", "SamplingParams", "argmax_row", "pick_rows", "random_seed"]

@@ -109,50 +109,99 @@ def argmax_row(logits: torch.Tensor) -> int:
     return host_lib().axh_argmax_row(ctypes.c_void_p(logits.data_ptr()), logits.numel())
 
 
+class _Pinned:
+    """Pinned host buffers that are used again: a ring per (purpose, dtype, size class), so that a
+    buffer is written again only long after the copy that read it has run."""
+
+    def __init__(self):
+        self.rings = {}
+
+    def take(self, purpose: str, numel: int, dtype) -> torch.Tensor:
+        size = 1 << max(6, (max(numel, 1) - 1).bit_length())
+        ring = self.rings.setdefault((purpose, dtype, size), {"at": 0, "bufs": []})
+        if len(ring["bufs"]) < 8:
+            ring["bufs"].append(torch.empty(size, dtype=dtype).pin_memory())
+            return ring["bufs"][-1][:numel]
+        ring["at"] = (ring["at"] + 1) % 8
+        return ring["bufs"][ring["at"]][:numel]
+
+
+_PINNED = _Pinned()
+
+
+class PendingRowPicks:
+    """The picks of a step's rows, decided in two halves: what runs on the device is queued when
+    this is made (penalty and top-k, the copy of the candidates), `finish()` waits for it and
+    lets the native sampler draw.  Between the two the host is free to prepare the next step."""
+
+    def __init__(self, rt, logits: torch.Tensor, samplers: Sequence[Optional[Sampler]], histories: Sequence[Sequence[int]]):
+        rows, vocab = logits.shape
+        self.samplers, self.histories, self.logits = samplers, histories, logits
+        self.picks: List[Optional[int]] = [None] * rows
+        self.greedy = [r for r in range(rows) if samplers[r] is None or samplers[r].params.greedy]
+        self.device_rows = [r for r in range(rows) if r not in self.greedy and 1 <= samplers[r].params.top_k <= DEVICE_TOPK_MAX]
+        self.host_rows = [r for r in range(rows) if r not in self.greedy and r not in self.device_rows]
+        self.greedy_out = self.keys_host = self.event = None
+        dev = logits.device
+        if self.greedy:
+            sel = logits if len(self.greedy) == rows else logits[torch.tensor(self.greedy, device=dev)]
+            self.greedy_out = torch.empty(len(self.greedy), dtype=torch.int32, device=dev)
+            rt.k.argmax(sel, self.greedy_out)
+        if self.device_rows:
+            n = len(self.device_rows)
+            recents = [samplers[r].recent(histories[r]) for r in self.device_rows]
+            width = max(1, max(len(x) for x in recents))
+            self.ks = [min(samplers[r].params.top_k, vocab) for r in self.device_rows]
+            # one copy to the device, through pinned memory (it does not wait for the step that is
+            # running): the recent tokens, how many, k, and the penalties' bits
+            staged = _PINNED.take("topk in", n * width + 3 * n, torch.int32)
+            flat = staged.numpy()
+            flat[:] = 0
+            rec = flat[:n * width].reshape(n, width)
+            for i, x in enumerate(recents):
+                rec[i, :len(x)] = x
+            flat[n * width:n * width + n] = [len(x) for x in recents]
+            flat[n * width + n:n * width + 2 * n] = self.ks
+            flat[n * width + 2 * n:].view(np.float32)[:] = [samplers[r].params.repeat_penalty for r in self.device_rows]
+            on = staged.to(dev, non_blocking=True)
+            sel = logits if n == rows else logits[torch.tensor(self.device_rows, device=dev)].contiguous()
+            self.k_stride = max(self.ks)
+            cands = torch.empty((n, self.k_stride), dtype=torch.int64, device=dev)      # a row's first k places are written
+            rt.k.topk(sel, on[:n * width].view(n, width), on[n * width:n * width + n], on[n * width + 2 * n:].view(torch.float32),
+                      on[n * width + n:n * width + 2 * n], cands, k_max=self.k_stride)
+            self.keys_host = _PINNED.take("topk out", n * self.k_stride, torch.int64)
+            self.keys_host.copy_(cands.view(-1), non_blocking=True)
+            self.event = torch.cuda.Event()
+            self.event.record()
+
+    def finish(self) -> List[int]:
+        picks = self.picks
+        if self.greedy:
+            for r, v in zip(self.greedy, self.greedy_out.tolist()):
+                picks[r] = v
+        if self.device_rows:
+            n = len(self.device_rows)
+            self.event.synchronize()
+            # every row's pick in one call of the native sampler, each from its own stream
+            ss = [self.samplers[r] for r in self.device_rows]
+            params = np.array([[s.params.temperature, s.params.top_p, s.params.min_p] for s in ss], dtype=np.float32).T.copy()
+            ks = np.array(self.ks, dtype=np.int32)
+            states = (ctypes.c_void_p * n)(*[ctypes.addressof(s.rng.state) for s in ss])
+            out = np.empty(n, dtype=np.int32)
+            host_lib().axh_sample_pick_keys_rows(
+                ctypes.c_void_p(self.keys_host.data_ptr()), self.k_stride, n, ctypes.c_void_p(ks.ctypes.data),
+                ctypes.c_void_p(params[0].ctypes.data), ctypes.c_void_p(params[1].ctypes.data),
+                ctypes.c_void_p(params[2].ctypes.data), states, ctypes.c_void_p(out.ctypes.data))
+            for r, v in zip(self.device_rows, out.tolist()):
+                picks[r] = v
+        for r in self.host_rows:
+            picks[r] = self.samplers[r].pick_row(self.logits[r].cpu().contiguous(), self.histories[r])
+        return picks
+
+
 def pick_rows(rt, logits: torch.Tensor, samplers: Sequence[Optional[Sampler]],
               histories: Sequence[Sequence[int]]) -> List[int]:
     """The next token of every row of `logits` (device, float32 [rows, vocab]).  `samplers[r]`
     is None for a greedy row; `histories[r]` is the row's tokens so far, the one the logits
     follow included.  Sampled rows' logits are penalised in place."""
-    rows, vocab = logits.shape
-    picks: List[Optional[int]] = [None] * rows
-    greedy = [r for r in range(rows) if samplers[r] is None or samplers[r].params.greedy]
-    device_rows = [r for r in range(rows) if r not in greedy and 1 <= samplers[r].params.top_k <= DEVICE_TOPK_MAX]
-    host_rows = [r for r in range(rows) if r not in greedy and r not in device_rows]
-    dev = logits.device
-    if greedy:
-        if len(greedy) == rows:
-            out = torch.empty(rows, dtype=torch.int32, device=dev)
-            rt.k.argmax(logits, out)
-            for r, v in enumerate(out.tolist()):
-                picks[r] = v
-        else:
-            sel = logits[torch.tensor(greedy, device=dev)]
-            out = torch.empty(len(greedy), dtype=torch.int32, device=dev)
-            rt.k.argmax(sel, out)
-            for r, v in zip(greedy, out.tolist()):
-                picks[r] = v
-    if device_rows:
-        n = len(device_rows)
-        recents = [samplers[r].recent(histories[r]) for r in device_rows]
-        width = max(1, max(len(x) for x in recents))
-        ks = [min(samplers[r].params.top_k, vocab) for r in device_rows]
-        # one copy to the device: the recent tokens, how many, k, and the penalties' bits
-        flat = np.zeros(n * width + 3 * n, dtype=np.int32)
-        rec = flat[:n * width].reshape(n, width)
-        for i, x in enumerate(recents):
-            rec[i, :len(x)] = x
-        flat[n * width:n * width + n] = [len(x) for x in recents]
-        flat[n * width + n:n * width + 2 * n] = ks
-        flat[n * width + 2 * n:].view(np.float32)[:] = [samplers[r].params.repeat_penalty for r in device_rows]
-        on = torch.from_numpy(flat).to(dev)
-        sel = logits if n == rows else logits[torch.tensor(device_rows, device=dev)].contiguous()
-        cands = torch.empty((n, max(ks)), dtype=torch.int64, device=dev)      # a row's first k places are written
-        rt.k.topk(sel, on[:n * width].view(n, width), on[n * width:n * width + n], on[n * width + 2 * n:].view(torch.float32),
-                  on[n * width + n:n * width + 2 * n], cands, k_max=max(ks))
-        host = cands.cpu()
-        for i, r in enumerate(device_rows):
-            picks[r] = samplers[r].pick_keys(host[i, :ks[i]].contiguous())
-    for r in host_rows:
-        picks[r] = samplers[r].pick_row(logits[r].cpu().contiguous(), histories[r])
-    return picks
+    return PendingRowPicks(rt, logits, samplers, histories).finish()

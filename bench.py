@@ -216,11 +216,20 @@ def main() -> int:
         ps = [prompt(prompt_len) for _ in range(args.batch)]
         n_new = min(steps, 64)
         llm.generate(ps, max_new_tokens=n_new)                        # the graphs of these steps are captured here
+        llm.generate(ps, max_new_tokens=n_new, temperature=0.8, top_k=40, seed=1)
         for label, kw in (("greedy", {}), ("stop_token", dict(stop=[V - 1])),
                           ("sampled", dict(temperature=0.8, top_k=40, seed=1))):
             llm.generate(ps, max_new_tokens=n_new, **kw)
             st = llm.last_stats
             points[f"generate_b{args.batch}_{label}"] = round(st.decode_tokens / max(st.decode_seconds, 1e-9), 1)
+            points_ms[f"generate_b{args.batch}_{label}"] = round(st.decode_seconds / max(st.decode_steps, 1) * 1e3, 4)
+        # generation's clock waits for the device where the kind of step changes and at the end, so its
+        # figures cannot beat the synchronised steps above by more than what a shorter context gives
+        # (these requests generate fewer tokens than the headline's); if one does, say so
+        beyond = {k: v for k, v in points.items() if k.startswith("generate_") and v > 1.02 * head["tok_s"]}
+        if beyond:
+            more["clock_check"] = f"generate points above 1.02 x the synchronised {head['tok_s']:.1f} tok/s: {beyond}"
+            print(f"bench.py: {more['clock_check']}", file=sys.stderr)
     achieved = head["bytes"] / (head["ms"] / 1e3) / 1e9
     line = {
         "metric": f"decode tok/s ({name}, {args.dtype}, batch {args.batch}, {prompt_len}-token prompts)",
