@@ -1,9 +1,13 @@
 """The command line, in the manner of the reference's `axon` (src/cli.rs:35-68, 856-1248):
 
-    axon gen MODEL "IDS" [-n N] [--ctx N] [--dtype T] [sampling flags]   generate (greedy unless --temp > 0)
+    axon gen MODEL "IDS" ["IDS" ...] [-n N] [--ctx N] [--dtype T] [sampling flags]   generate (greedy unless --temp > 0)
     axon logits MODEL "IDS" [-k K] [--all N]                             top-K next-token logits after the prompt
     axon info MODEL                                                      print a summary and exit
     axon random-weights CONFIG.json OUT [--seed S] [--std F]             write a model folder with random weights
+
+MODEL is a folder with config.json and model.safetensors; with `--random-weights SEED` it is a
+config.json (or a folder holding one) and the weights are drawn from the seed, nothing is read or
+written.  `gen` takes any number of prompts and batches them; a line of ids is printed for each.
 
 There is no tokenizer here: a prompt is a list of token ids ("5 17 3" or "5,17,3"), and what
 `gen` prints is token ids.  Sampling flags have the reference's names, defaults and order
@@ -50,6 +54,9 @@ def _engine_flags(p: argparse.ArgumentParser) -> None:
     p.add_argument("--page-size", type=int, default=64, help="positions in one cache page (default 64: a block of the attention kernels)")
     p.add_argument("--num-pages", type=int, default=0, help="pages in the cache pool (default: what the request needs)")
     p.add_argument("--device", default="cuda:0", help="the GPU to run on (default cuda:0)")
+    p.add_argument("--random-weights", type=int, default=None, metavar="SEED",
+                   help="MODEL is a config.json: run it with random weights drawn from this seed")
+    p.add_argument("--std", type=float, default=0.02, help="with --random-weights: their standard deviation (default 0.02)")
     p.add_argument("--verbose", action="store_true", help="print what was loaded and the settings in use")
 
 
@@ -75,7 +82,7 @@ def build_parser() -> argparse.ArgumentParser:
     sub = ap.add_subparsers(dest="command")
     g = sub.add_parser("gen", help="generate (greedy unless --temp > 0)")
     g.add_argument("model")
-    g.add_argument("prompt", help='token ids, e.g. "5 17 3"')
+    g.add_argument("prompt", nargs="+", help='token ids, e.g. "5 17 3"; several prompts are generated side by side')
     g.add_argument("-n", type=int, default=32, dest="n", help="tokens to generate (default 32)")
     g.add_argument("--stop", default="", help="token ids that end generation (not printed)")
     _engine_flags(g)
@@ -98,16 +105,29 @@ def build_parser() -> argparse.ArgumentParser:
     return ap
 
 
-def _load(args, need_tokens: int):
+def _load(args, need_tokens: int, requests: int = 1):
+    """`need_tokens`: the positions the longest request reaches; `requests`: how many run side by side."""
+    import os
+
     import axon_amd
+    from axon_amd.config import config_from_dict
     from axon_amd.engine.loading import read_model_config
-    cfg = read_model_config(args.model)
+    if args.random_weights is not None:
+        path = os.path.join(args.model, "config.json") if os.path.isdir(args.model) else args.model
+        with open(path) as f:
+            cfg = config_from_dict(json.load(f))
+    else:
+        cfg = read_model_config(args.model)
     ctx = args.ctx or cfg.model_spec().max_positions
     if need_tokens > ctx:
         _refuse(f"the prompt and the tokens to generate need {need_tokens} positions, the context is {ctx}")
-    pages = args.num_pages or -(-need_tokens // args.page_size) + 1
-    llm = axon_amd.load(args.model, dtype=args.dtype, device=args.device, page_size=args.page_size, num_pages=pages,
-                        max_seqs=2, max_seq_len=ctx, max_batch_tokens=max(2048, 1))
+    pages = args.num_pages or requests * (-(-need_tokens // args.page_size) + 1)
+    settings = dict(dtype=args.dtype, device=args.device, page_size=args.page_size, num_pages=pages,
+                    max_seqs=max(2, requests), max_seq_len=ctx, max_batch_tokens=2048)
+    if args.random_weights is not None:
+        llm = axon_amd.load(cfg, random_seed=args.random_weights, init_std=args.std, **settings)
+    else:
+        llm = axon_amd.load(args.model, **settings)
     if args.verbose:
         print(f"model: {cfg.architecture}  {json.dumps(cfg.to_dict())}", file=sys.stderr)
         print(f"engine: dtype {llm.rt.dtype_name}, page {args.page_size}, pages {pages}, context {ctx}", file=sys.stderr)
@@ -116,7 +136,7 @@ def _load(args, need_tokens: int):
 
 def run_gen(args) -> int:
     from axon_amd.sampling import SamplingParams, random_seed
-    ids = parse_ids(args.prompt)
+    prompts = [parse_ids(p) for p in args.prompt]
     if args.n < 0:
         _refuse("-n needs a whole number")
     temp = args.temp if args.temp is not None else 0.0
@@ -132,16 +152,17 @@ def run_gen(args) -> int:
     if temp > 0 and seed is None:
         params.seed = random_seed()
         print(f"seed: {params.seed}", file=sys.stderr)
-    llm, cfg = _load(args, len(ids) + args.n)
+    llm, cfg = _load(args, max(len(ids) for ids in prompts) + args.n, len(prompts))
     vocab = llm.model.vocab_size
-    if any(i >= vocab for i in ids):
+    if any(i >= vocab for ids in prompts for i in ids):
         _refuse(f"a token id is outside the vocabulary of {vocab}")
     stop = parse_ids(args.stop) if args.stop.strip() else []
-    out = llm.generate([ids], max_new_tokens=args.n, stop=stop, sampling=params)[0]
-    print(" ".join(str(t) for t in out))
+    for out in llm.generate(prompts, max_new_tokens=args.n, stop=stop, sampling=params):
+        print(" ".join(str(t) for t in out))
     st = llm.last_stats
     rate = lambda n, s: n / s if s > 0 else float("inf")
-    print(f"prompt eval: {len(ids)} tok in {st.prompt_seconds:.3f} s ({rate(len(ids), st.prompt_seconds):.1f} tok/s)",
+    fed = sum(len(ids) for ids in prompts)
+    print(f"prompt eval: {fed} tok in {st.prompt_seconds:.3f} s ({rate(fed, st.prompt_seconds):.1f} tok/s)",
           file=sys.stderr)
     print(f"decode: {st.decode_tokens} tok, {st.decode_steps} passes in {st.decode_seconds:.3f} s "
           f"({rate(st.decode_tokens, st.decode_seconds):.1f} tok/s)", file=sys.stderr)

@@ -27,6 +27,7 @@
 // matched to the positions a lane holds by reading V^T accordingly (values are cached
 // position-contiguous: [page][kv head][dim][slot]).
 #include <math.h>
+#include <stdlib.h>
 
 #include "api.h"
 #include "common.h"
@@ -57,8 +58,11 @@ __device__ inline uint32_t pack_bf16(float a, float b) { return pack2_bf16(a, b)
 // ============================================================================ one block of 64 positions
 // A stage of LDS holds a block's K [64][HD] and V^T [HD][64], brought by direct global -> LDS
 // loads of 16 bytes a lane (an instruction fills 1 KB: 1024 / (2 HD) rows of K, or 8 rows of
-// V^T).  16-byte slots of a row are permuted (slot ^ row & 7) so that fragment reads of
-// neighbouring rows fall into different banks.
+// V^T).  16-byte slots of a row are permuted so that the fragment reads of 16 neighbouring rows
+// fall into 16 different slots of the 256 bytes (64 banks) that LDS serves in a cycle: rows of
+// 256 bytes (K at head size 128) by slot ^ (row & 15), rows of 128 bytes (K at head size 64, V^T),
+// of which two lie side by side, by slot ^ ((row >> 1) & 7).  (With slot ^ (row & 7) for both, two
+// of every 16 rows met in a slot: the counters showed more cycles of bank conflicts than of reads.)
 #define ATT_ZERO16 (f32x16{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f})
 
 template <int HD>
@@ -71,6 +75,9 @@ struct AttStage {
   static constexpr int K_ROWS_PER_INSTR = 1024 / KROW;
   static constexpr int K_INSTR = ATT_BLOCK / K_ROWS_PER_INSTR;   // load instructions of a block's K
   static constexpr int V_INSTR = HD / 8;                         // and of its V^T
+  // the permutation of a row's slots (see above)
+  __device__ static __forceinline__ int k_swizzle(int row) { return KROW == 256 ? (row & 15) : ((row >> 1) & 7); }
+  __device__ static __forceinline__ int v_swizzle(int dim) { return (dim >> 1) & 7; }
 };
 
 // Pages hold a power of two of positions (axk_attention_fast_ok): the page of a position and its
@@ -89,18 +96,18 @@ __device__ __forceinline__ int att_k_page(int instr, int lane, int p0, int hi, c
 template <int HD>
 __device__ __forceinline__ int att_v_page(int instr, int lane, int p0, int hi, const int32_t* table_row, int page_size) {
   const int d = instr * 8 + (lane >> 3);
-  const int chunk = (lane & 7) ^ (d & 7);
+  const int chunk = (lane & 7) ^ AttStage<HD>::v_swizzle(d);
   return table_row[page_index(min(p0 + chunk * 8, hi), page_size)];
 }
 
 // K: lane i of instruction `instr` brings row i / KCH of the instruction's rows, into slot i % KCH,
-// which holds the row's chunk slot ^ (row & 7).
+// which holds the row's chunk slot ^ k_swizzle(row).
 template <int HD>
 __device__ __forceinline__ void att_issue_k(unsigned char* stage, int instr, int lane, int page, int p0, int hi,
                                             const bf16_t* k_head, size_t page_stride, int page_size) {
   using S = AttStage<HD>;
   const int row = instr * S::K_ROWS_PER_INSTR + lane / S::KCH;
-  const int chunk = (lane % S::KCH) ^ (row & 7);
+  const int chunk = (lane % S::KCH) ^ S::k_swizzle(row);
   const int p = min(p0 + row, hi);
   const bf16_t* base = k_head + (size_t)page * page_stride;          // scalar arithmetic where the page is the wave's
   const bf16_t* src = base + (unsigned)(page_offset(p, page_size) * HD + chunk * 8);
@@ -108,13 +115,13 @@ __device__ __forceinline__ void att_issue_k(unsigned char* stage, int instr, int
 }
 
 // V^T: lane i brings row (dim) i / 8 of the instruction's 8 dims, into slot i % 8, which holds the
-// 8 positions of chunk slot ^ (dim & 7).
+// 8 positions of chunk slot ^ v_swizzle(dim).
 template <int HD>
 __device__ __forceinline__ void att_issue_v(unsigned char* stage, int instr, int lane, int page, int p0, int hi,
                                             const bf16_t* v_head, size_t page_stride, int page_size) {
   using S = AttStage<HD>;
   const int d = instr * 8 + (lane >> 3);
-  const int chunk = (lane & 7) ^ (d & 7);
+  const int chunk = (lane & 7) ^ S::v_swizzle(d);
   const int p = min(p0 + chunk * 8, hi);
   const bf16_t* base = v_head + (size_t)page * page_stride;
   const bf16_t* src = base + (unsigned)(d * page_size + (page_offset(p, page_size) & ~7));
@@ -130,7 +137,7 @@ __device__ __forceinline__ void att_clear_unwritten(unsigned char* stage, int p0
   for (int idx = t; idx < HD * ATT_BLOCK; idx += n_threads) {
     const int d = idx / ATT_BLOCK, col = idx % ATT_BLOCK;
     if (col >= first_bad) {
-      const int slot = (col >> 3) ^ (d & 7);
+      const int slot = (col >> 3) ^ AttStage<HD>::v_swizzle(d);
       *reinterpret_cast<uint16_t*>(stage + AttStage<HD>::K_BYTES + d * 128 + slot * 16 + (col & 7) * 2) = 0;
     }
   }
@@ -155,7 +162,7 @@ __device__ __forceinline__ void attention_scores(unsigned st, const bf16x8 (&qf)
   constexpr int KS = HD / 16;
   const int l32 = lane & 31, half = lane >> 5;
   const int k_row = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);
-  const unsigned k_at = st + k_row * S::KROW, k_swz = k_row & 7;
+  const unsigned k_at = st + k_row * S::KROW, k_swz = S::k_swizzle(k_row);
 
   // S^T [64 positions][32 queries] = K Q^T: two tiles of 32 positions, two k steps a group
   f32x16 s_acc[2];                    // each chain starts from the constant zero
@@ -237,7 +244,7 @@ __device__ __forceinline__ void attention_values(unsigned st, const bf16x8 (&pf)
   using S = AttStage<HD>;
   constexpr int DT = HD / 32;
   const int l32 = lane & 31, half = lane >> 5;
-  const unsigned v_at = st + S::K_BYTES + l32 * 128, v_swz = l32 & 7;
+  const unsigned v_at = st + S::K_BYTES + l32 * 128, v_swz = S::v_swizzle(l32);      // the same for every tile of 32 dims
   u32x4 vf[2][4];
   auto read_v = [&](u32x4 (&dst)[4], int dt) {
     const unsigned row = v_at + dt * 32 * 128;
@@ -733,7 +740,8 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
   // two query heads of a kv head a block (they share each K and V block in LDS) where that still
   // gives the chip's 256 CUs about a block each; else one head a block
   const int blocks_of_pairs = n_tiles * n_kv_heads * ((group + 1) / 2);
-  if (group >= 2 && blocks_of_pairs >= 200) {
+  const char* force = getenv("AXON_ATT_HPB");
+  if (force ? force[0] == '2' : (group >= 2 && blocks_of_pairs >= 200)) {
     if (head_dim == 64) LAUNCH(64, 2) else LAUNCH(128, 2)
   } else {
     if (head_dim == 64) LAUNCH(64, 1) else LAUNCH(128, 1)

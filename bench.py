@@ -45,6 +45,47 @@ WORKLOAD = {"7b": (2048, 256), "14b": (1024, 256), "32b": (4096, 128)}
 PREFILL_TOKENS = 2048
 
 
+def bandwidth(torch):
+    """What reading memory costs here, measured with the engine's own streaming product (one row of X
+    times a packed matrix: every byte of W is read once, 32 KB in flight a wave): a matrix of 1 GB
+    (the sustained rate a decoding step can hope for), and matrices of the sizes of a step's smaller
+    kernels read cold (right behind a read of 1 GB of other data, with no idle gap) and again right
+    after themselves (what a launch of its own costs a kernel, and what the memory-side cache gives)."""
+    from axon_amd.kernels import MODE_STORE_F32, kernels
+    k = kernels("bfloat16")
+    K = 4096
+    x = torch.randn(1, K, device="cuda").bfloat16()
+
+    def matrix(mb):
+        n = mb * (1 << 20) // (2 * K)
+        w = k.prepare_weight((torch.randn(n, K, device="cuda") * 0.05).bfloat16())
+        y = torch.empty(1, n, dtype=torch.float32, device="cuda")
+        return (lambda: k.gemm(x, w, y, None, MODE_STORE_F32)), n * K * 2
+
+    def timed(fn):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) * 1e3
+
+    other, _ = matrix(1024)
+    out = {"unit": "us and TB/s", "reads": {}}
+    for mb in (16, 32, 64, 128, 256, 1024):
+        run, nbytes = matrix(mb)
+        run()
+        cold, warm = [], []
+        for _ in range(5):
+            other()
+            cold.append(timed(run))
+            run()
+            warm.append(timed(run))
+        out["reads"][f"{mb} MB"] = {"cold_us": round(min(cold), 1), "cold_TBps": round(nbytes / min(cold) / 1e6, 2),
+                                    "again_us": round(min(warm), 1), "again_TBps": round(nbytes / min(warm) / 1e6, 2)}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -59,9 +100,10 @@ def main() -> int:
                     "measured configurations name; the engine's own default is 64, a block of its attention kernels)")
     ap.add_argument("--sizes", default="7b", choices=sorted(SIZES), help="layer sizes of Qwen2.5-7B (the default), 14B or 32B")
     ap.add_argument("--no-points", action="store_true", help="only the headline batch and the prefill point")
-    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "mixed"],
+    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "mixed", "bandwidth"],
                     help="for profiling: time only the prefill step (repeated --steps times), only decoding, or only "
-                         "the mixed step")
+                         "the mixed step; bandwidth: no model, what reading memory once costs on this GPU (a long "
+                         "read, and reads of the sizes of a decoding step's kernels, cold and right after themselves)")
     ap.add_argument("--profile", action="store_true", help="also launch one decode step kernel by kernel and print each "
                     "kernel's time and matrix bytes on stderr")
     args = ap.parse_args()
@@ -73,6 +115,10 @@ def main() -> int:
 
     import axon_amd
     from axon_amd.engine import StepEntry
+
+    if args.phase == "bandwidth":
+        print(json.dumps(bandwidth(torch)))
+        return 0
 
     cfg = dict(SIZES[args.sizes])
     name = f"Qwen2.5-{args.sizes.upper()} sizes"
@@ -125,12 +171,14 @@ def main() -> int:
     # ---- decode at a batch size: prefill every request, then time K steps
     weight_bytes = (L * ((nh + 2 * nkv) * hd * dim + nh * hd * dim + 3 * ffn * dim) + V * dim) * elem
 
-    def decode(batch: int, n_steps: int, warmup: int, profile: bool = False):
-        ids = [f"d{batch}_{i}" for i in range(batch)]
+    def decode(batch: int, n_steps: int, warmup: int, profile: bool = False, eng=eng, prompt_len=prompt_len, portion=0):
+        ids = [f"d{batch}_{prompt_len}_{i}" for i in range(batch)]
         last = []
         for rid in ids:
             pr = prompt(prompt_len)
-            eng.step([StepEntry(rid, pr[:-1], [])])
+            fed = pr[:-1]
+            for a in range(0, len(fed), portion or len(fed)):          # long prompts in portions
+                eng.step([StepEntry(rid, fed[a:a + (portion or len(fed))], [])])
             last.append(pr[-1])
         if profile:
             rows, total = eng.profile([StepEntry(rid, [t], [0]) for rid, t in zip(ids, last)])
@@ -198,7 +246,43 @@ def main() -> int:
         print(json.dumps({"phase": "mixed", "mixed": mixed(max(args.steps, 3)), "layers": L}))
         return 0
 
+    # ---- contexts of 32,768 positions: a second engine over the same weights (the measured
+    # configuration names a context of 8,192; positions enter the arithmetic only through the
+    # rotary angles), its pool sized for eight such requests.  A prompt of 32,768 tokens in portions
+    # of 8,192, then decoding at batch 1 and 8 with every request that deep.
+    def long_contexts(decode, first_engine, ctx=32768, portion=8192):
+        nonlocal eng
+        from axon_amd.config import EngineConfig
+        from axon_amd.engine import Engine
+        first_engine.release_all()
+        llm.engine = eng = None
+        del first_engine
+        torch.cuda.empty_cache()
+        room = ctx + 64 + 64
+        long = Engine(llm.model, llm.rt, EngineConfig(dtype=args.dtype, page_size=page, num_pages=8 * -(-room // page) + 8,
+                                                      max_seqs=8, max_batch_tokens=portion, max_seq_len=room))
+        p = prompt(ctx)
+        times = []
+        for rep in range(2):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for a in range(0, ctx, portion):
+                long.step([StepEntry("long", p[a:a + portion], [portion - 1] if a + portion >= ctx else [])],
+                          end=["long"] if a + portion >= ctx else [])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        s = times[-1]
+        flops = L * layer_flops(ctx, ctx * (ctx + 1) / 2) + 2 * dim * V
+        out = {f"prefill_{ctx}_in_portions_of_{portion}": {"value": round(ctx / s, 1), "tokens": ctx, "ms": round(s * 1e3, 3),
+                                                         "frac": round(flops / s / PEAK_FLOPS[args.dtype], 4)}}
+        for b in (1, 8):
+            r = decode(b, 32, 4, eng=long, prompt_len=ctx, portion=portion)
+            out[f"decode_b{b}_ctx{ctx}"] = {"value": round(r["tok_s"], 1), "ms": round(r["ms"], 4), "frac": round(r["frac"], 4)}
+        long.release_all()
+        return out
+
     head = decode(args.batch, steps, args.warmup, profile=args.profile)
+    cache_pages, graphs_on = eng.cache.plans[0].n_pages, bool(eng.graphs_ok)
     points, points_ms, points_frac, more = {}, {}, {}, {}
     if points_on:
         for b in (1, 64):
@@ -230,6 +314,8 @@ def main() -> int:
         if beyond:
             more["clock_check"] = f"generate points above 1.02 x the synchronised {head['tok_s']:.1f} tok/s: {beyond}"
             print(f"bench.py: {more['clock_check']}", file=sys.stderr)
+        if args.sizes == "7b" and not args.layers:
+            more.update(long_contexts(decode, eng))
     achieved = head["bytes"] / (head["ms"] / 1e3) / 1e9
     line = {
         "metric": f"decode tok/s ({name}, {args.dtype}, batch {args.batch}, {prompt_len}-token prompts)",
@@ -239,8 +325,8 @@ def main() -> int:
         "config": {"model": name, "layers": L, "layers_of_config": full_layers, "hidden": dim,
                    "heads": nh, "kv_heads": nkv, "head_dim": hd, "intermediate": ffn, "vocab": V, "batch": args.batch,
                    "global_batch": args.batch, "seq_len": prompt_len, "generated": steps, "context": ctx_len,
-                   "page_size": page, "cache_pages": eng.cache.plans[0].n_pages, "parallelism": "single GPU",
-                   "graphs": bool(eng.graphs_ok), "batch_invariant": True},
+                   "page_size": page, "cache_pages": cache_pages, "parallelism": "single GPU",
+                   "graphs": graphs_on, "batch_invariant": True},
         "prefill": prefill_point,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_BYTES_PER_S, 4)},

@@ -294,6 +294,20 @@ def test_command_line_gen_and_logits(model_dirs):
                        capture_output=True, text=True, timeout=300)
     assert [int(t) for t in r.stdout.split()] == P.sample_generate(
         cfg, w, p, 6, temp=0.7, top_k=40, top_p=0.9, min_p=0.0, repeat_penalty=1.1, repeat_last_n=64, seed=4)
+    # several prompts in one call: a line each, the lines of the prompts run alone
+    q = prompts_for("A", [12], seed=12)[0]
+    r = subprocess.run(axon + ["gen", d, ids, " ".join(map(str, q)), "-n", "5", "--dtype", "float32", "--page-size", "8"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert [[int(t) for t in line.split()] for line in r.stdout.splitlines()] == [
+        P.greedy_generate(cfg, w, p, 5), P.greedy_generate(cfg, w, q, 5)]
+    assert f"prompt eval: {len(p) + len(q)} tok" in r.stderr
+    # a configuration and a seed in place of a model folder: the same seed, the same tokens
+    config = os.path.join(d, "config.json")
+    runs = [subprocess.run(axon + ["gen", config, ids, "-n", "6", "--random-weights", seed, "--std", "0.3", "--dtype", "float32"],
+                           capture_output=True, text=True, timeout=300) for seed in ("3", "3", "4")]
+    assert all(r.returncode == 0 for r in runs), runs[0].stderr
+    assert runs[0].stdout == runs[1].stdout != runs[2].stdout and len(runs[0].stdout.split()) == 6
     r = subprocess.run(axon + ["logits", d, ids, "-k", "3", "--dtype", "float32"], capture_output=True, text=True,
                        timeout=300)
     assert r.returncode == 0, r.stderr
