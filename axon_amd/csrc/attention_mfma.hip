@@ -27,7 +27,6 @@
 // matched to the positions a lane holds by reading V^T accordingly (values are cached
 // position-contiguous: [page][kv head][dim][slot]).
 #include <math.h>
-#include <stdlib.h>
 
 #include "api.h"
 #include "common.h"
@@ -740,8 +739,7 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
   // two query heads of a kv head a block (they share each K and V block in LDS) where that still
   // gives the chip's 256 CUs about a block each; else one head a block
   const int blocks_of_pairs = n_tiles * n_kv_heads * ((group + 1) / 2);
-  const char* force = getenv("AXON_ATT_HPB");
-  if (force ? force[0] == '2' : (group >= 2 && blocks_of_pairs >= 200)) {
+  if (group >= 2 && blocks_of_pairs >= 200) {
     if (head_dim == 64) LAUNCH(64, 2) else LAUNCH(128, 2)
   } else {
     if (head_dim == 64) LAUNCH(64, 1) else LAUNCH(128, 1)
