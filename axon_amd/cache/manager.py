@@ -82,6 +82,8 @@ def host_lib():
             "axh_sample_pick_row": (c_int, [c_void_p, c_int, c_void_p, c_int, ctypes.c_float, c_int, ctypes.c_float,
                                             ctypes.c_float, ctypes.c_float, ctypes.c_double]),
             "axh_argmax_row": (c_int, [c_void_p, c_int]),
+            "axh_step_layout": (c_long, [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_long,
+                                         c_void_p, c_long, c_void_p, IP, c_char_p, c_int]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(lib, name)

@@ -15,13 +15,15 @@ The reference runs prompt portions and decode rows as two passes of one schedule
 """
 from __future__ import annotations
 
+import ctypes
 from collections import ChainMap
 from dataclasses import dataclass
 from typing import Dict, Hashable, Iterable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
-from ..cache.manager import CacheManager
+from ..cache.manager import CacheManager, host_lib
 from ..config.engine import EngineConfig
 from ..models.decoder import DecoderModel
 from .runtime import Runtime, Workspace
@@ -205,40 +207,56 @@ class Engine:
             self.release(rid)
 
     # ------------------------------------------------------------------ the step
-    def _validate(self, entries: Sequence[StepEntry]) -> None:
+    def _layout(self, entries: Sequence[StepEntry]):
+        """The entries of a step checked and their tokens laid side by side, by the native host
+        library in one call (csrc/host/step.cpp): (meta int32 [3, T]: token ids, positions and
+        slots of the step's tokens; the rows whose logits are wanted).  Every request of the step
+        has its slot by now.  A refused step raises StepError and has written nothing."""
+        n = len(entries)
+        try:
+            flat = [np.asarray(e.tokens, dtype=np.int64).reshape(-1) for e in entries]
+            wants = [np.asarray(e.want, dtype=np.int64).reshape(-1) for e in entries]
+        except (TypeError, ValueError, OverflowError) as err:
+            raise StepError(f"a step's tokens and wanted places are whole numbers: {err}") from None
+        counts = np.array([len(t) for t in flat], dtype=np.int64)
+        want_counts = np.array([len(w) for w in wants], dtype=np.int64)
+        tokens = np.concatenate(flat) if n else np.zeros(0, dtype=np.int64)
+        want = np.concatenate(wants) if n else np.zeros(0, dtype=np.int64)
+        slots = np.array([self.live[e.id].slot for e in entries], dtype=np.int32)
+        cached = np.array([self.live[e.id].n_cached for e in entries], dtype=np.int64)
+        T = int(counts.sum())
+        meta = np.empty((3, max(T, 1)), dtype=np.int32)
+        want_rows = np.empty(max(len(want), 1), dtype=np.int32)
+        refused, message = ctypes.c_int(-1), ctypes.create_string_buffer(200)
+        ptr = lambda a: ctypes.c_void_p(a.ctypes.data)
+        rc = host_lib().axh_step_layout(n, ptr(slots), ptr(cached), ptr(counts), ptr(tokens), ptr(want), ptr(want_counts),
+                                        self.model.vocab_size, self.max_seq_len, ptr(meta), meta.shape[1], ptr(want_rows),
+                                        ctypes.byref(refused), message, len(message))
+        if rc < 0:
+            who = f"request {entries[refused.value].id!r}: " if refused.value >= 0 else ""
+            raise StepError(who + message.value.decode())
+        return meta[:, :T], want_rows[:len(want)], counts
+
+    def step(self, entries: Sequence[StepEntry], end: Iterable[Hashable] = ()) -> Optional[torch.Tensor]:
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         seen = set()
-        vocab = self.model.vocab_size
         for e in entries:
             if e.id in seen:
                 raise StepError(f"request {e.id!r} appears twice in one step")
             seen.add(e.id)
-            n = len(e.tokens)
-            if n == 0:
-                raise StepError(f"request {e.id!r} brings no tokens")
-            for t in e.tokens:
-                if not 0 <= int(t) < vocab:
-                    raise StepError(f"request {e.id!r}: token {t} is outside the vocabulary of {vocab}")
-            for w in e.want:
-                if not 0 <= int(w) < n:
-                    raise StepError(f"request {e.id!r}: wanted place {w} is outside its {n} tokens")
-            after = self.n_cached(e.id) + n
-            if after > self.max_seq_len:
-                raise StepError(f"request {e.id!r} would reach {after} positions, at most {self.max_seq_len}")
         new = sum(1 for e in entries if e.id not in self.live)
         if new > self.cache.free_slots():
             raise StepError(f"{len(self.live) + new} live requests, at most {self.cfg.max_seqs}")
-
-    def step(self, entries: Sequence[StepEntry], end: Iterable[Hashable] = ()) -> Optional[torch.Tensor]:
-        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
-        self._validate(entries)
-        # pages for every entry or for none: a step that does not fit leaves the cache as it was
+        # Everything is checked, and pages are taken for every entry or for none, before anything
+        # runs: a step that is refused or does not fit leaves the cache as it was.
         opened = []
         try:
             for e in entries:
                 if e.id not in self.live:
                     self.live[e.id] = LiveRequest(self.cache.open())
                     opened.append(e.id)
-            self.cache.reserve_many([(self.live[e.id].slot, self.live[e.id].n_cached + len(e.tokens)) for e in entries])
+            meta, want_rows, counts = self._layout(entries)
+            self.cache.reserve_many([(self.live[e.id].slot, self.live[e.id].n_cached + int(n)) for e, n in zip(entries, counts)])
         except Exception:
             for rid in opened:
                 self.release(rid)
@@ -250,31 +268,26 @@ class Engine:
         self._pending = None
         self._prepared = None
         if entries:
-            tokens, positions, rows, want_rows, spans = [], [], [], [], []
-            for e in entries:
+            spans, at = [], 0
+            for e, n in zip(entries, counts):
                 req = self.live[e.id]
-                at = len(tokens)
-                n = len(e.tokens)
-                spans.append(Span(req.slot, at, n, req.n_cached))
-                tokens.extend(int(t) for t in e.tokens)
-                positions.extend(range(req.n_cached, req.n_cached + n))
-                rows.extend([req.slot] * n)
-                want_rows.extend(at + int(w) for w in e.want)
-            T = len(tokens)
+                spans.append(Span(req.slot, at, int(n), req.n_cached))
+                at += int(n)
+            T = at
             self.cache.sync_tables()
             if T == len(entries) and len(want_rows) == T and T <= self.cfg.max_seqs:
-                logits = self._decode_step(tokens, positions, rows, spans)
+                logits = self._decode_step(meta[0].tolist(), meta[1].tolist(), meta[2].tolist(), spans)
                 self._last_decode = [e.id for e in entries]
             else:
-                meta = torch.tensor([tokens, positions, rows], dtype=torch.int32).to(self.rt.device)
-                ctx = StepContext(self.rt, self.cache, self.ws, meta, T, spans)
+                on_device = torch.from_numpy(np.ascontiguousarray(meta)).to(self.rt.device)
+                ctx = StepContext(self.rt, self.cache, self.ws, on_device, T, spans)
                 x = self.model.forward(ctx)
-                if want_rows:
-                    sel = torch.tensor(want_rows, dtype=torch.int32).to(self.rt.device)
+                if len(want_rows):
+                    sel = torch.from_numpy(want_rows.copy()).to(self.rt.device)
                     logits = self.model.logits(ctx, x, sel)
-            for e in entries:
+            for e, n in zip(entries, counts):
                 req = self.live[e.id]
-                req.n_cached += len(e.tokens)
+                req.n_cached += int(n)
                 if self.has_window:
                     self.cache.trim(req.slot, req.n_cached)
             self.steps += 1

@@ -35,7 +35,7 @@ KERNEL_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "attention.hip
 # what a library built from a part's own kernel sources gets beside them (the error channel, the
 # list of its kernel instances)
 EXTENSION_SUPPORT = ["support.hip", "instances.hip"]
-HOST_SOURCES = ["host/cache.cpp", "host/scheduler.cpp", "host/sampler.cpp"]
+HOST_SOURCES = ["host/cache.cpp", "host/scheduler.cpp", "host/sampler.cpp", "host/step.cpp"]
 
 # Packed 32-bit float instructions are switched off for all device code.  No contraction of a
 # product and a sum into a multiply-add unless the source writes one (fmaf): two kernels that
