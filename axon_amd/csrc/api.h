@@ -73,6 +73,7 @@ int axk_attention(const void* q, int q_stride, const void* k_cache, const void* 
 // each with its own maximum, folded ascending): a position's result is bit for bit the same from
 // either, alone or in any batch.
 int axk_attention_fast_ok(int head_dim, int page_size, int n_heads, int n_kv_heads);
+int axk_attention_prefill_tile(void);      // the most tokens of a run (128)
 int axk_attention_prefill(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                           const int32_t* block_table, int table_stride, const int32_t* positions,
                           const int32_t* seq_rows, void* out, const int32_t* tiles, int n_tiles,

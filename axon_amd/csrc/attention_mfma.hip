@@ -314,7 +314,7 @@ __device__ __forceinline__ float attention_inverse(float l) { return __fdiv_rn(1
 // the same kv head share every K and V^T block in LDS (the path from L2 into LDS carries about 32
 // bytes a cycle and CU, which is what one head's products use up).  Two stages: the next block's
 // loads are in flight while this one is multiplied.
-#define PF_TOKENS 128
+#define PF_TOKENS 128     // (axk_attention_prefill_tile says so to the caller)
 
 template <int HD, int HPB, bool ONE_PAGE>
 __device__ __forceinline__ void
@@ -752,6 +752,9 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
   return -1;
 #endif
 }
+
+// The most consecutive tokens of one request that a run of axk_attention_prefill's tiles holds.
+extern "C" int axk_attention_prefill_tile(void) { return 128; }
 
 // Positions of one chunk of a decoding token's range, and the factor of the token's slot in an
 // item of the work list (item = slot * factor + chunk).

@@ -426,6 +426,11 @@ class Kernels:
             float(scale), _stream()))
         return out
 
+    @property
+    def attention_prefill_tile(self) -> int:
+        """The most consecutive tokens of one request in a run of `attention_prefill`'s tiles."""
+        return int(self.lib.axk_attention_prefill_tile())
+
     def _decode_chunk_and_factor(self):
         if self._chunk_factor is None:
             self._chunk_factor = (int(self.lib.axk_attention_decode_chunk()), int(self.lib.axk_attention_decode_item_factor()))

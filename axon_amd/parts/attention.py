@@ -24,9 +24,6 @@ from ..kernels import MODE_ADD_F32, MODE_STORE, PackedMatrix
 from .base import CacheBinding, CacheSpec, Mixer, PrecedingNorm, TensorDecl, build_part, register_mixer
 
 
-PREFILL_TILE = 128     # tokens of one request per tile of the prompt kernel
-
-
 class AttentionPlan:
     """How the matrix-core kernels split a step: prompt portions (2 tokens or more) go to the
     prompt kernel in tiles of up to 128 tokens, single tokens to the decoding kernel.  Made
@@ -47,13 +44,14 @@ class AttentionPlan:
             n_single = ctx.n_tokens
         else:
             tiles, seen, singles, chunks = [], [], [], 1
+            tile = ctx.rt.k.attention_prefill_tile          # tokens of one request a tile of the prompt kernel holds
             for s in ctx.spans:
                 if s.q_len == 1:
                     singles.append(s.q_start)
                     chunks = max(chunks, decode_chunks_of(s.start_pos, window, ctx.rt.k.attention_decode_chunk))
                 else:
-                    for at in range(0, s.q_len, PREFILL_TILE):
-                        n = min(PREFILL_TILE, s.q_len - at)
+                    for at in range(0, s.q_len, tile):
+                        n = min(tile, s.q_len - at)
                         tiles.append((s.q_start + at, n))
                         last = s.start_pos + at + n                 # positions the tile's last token sees
                         seen.append(min(last, window + n) if window > 0 else last)

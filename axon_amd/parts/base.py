@@ -130,7 +130,9 @@ class Norm(Part):
 
     def preceding(self, ctx, x) -> Optional[PrecedingNorm]:
         """This norm of the rows x as work for the first product of the part after it, or None if
-        it always runs on its own (the default)."""
+        it always runs on its own (the default).  What is handed over is (gain, eps): the RMS
+        norm's arithmetic.  A norm of another kind does not offer itself, runs as a pass of its
+        own, and is right, only a launch slower."""
         return None
 
     def following(self, ctx, n_rows: int) -> Optional[FollowingNorm]:
