@@ -151,20 +151,24 @@ __device__ __forceinline__ void att_clear_unwritten(unsigned char* stage, int p0
 // `whole`: every column of the wave sees every position of the block (no mask needed);
 // else column l32 sees the positions my_lo .. my_pos.
 // attention_scores leaves m_b (log2 domain), l_b and the rounded weights as the four B operands
-// of O^T (k step s2: the positions 32 (s2 / 2) + 16 (s2 % 2) + 8 half + {0..7}).
+// of O^T (k step s2: the positions 32 (s2 / 2) + 16 (s2 % 2) + 8 half + {0..7}).  It is two
+// halves, the products (attention_raw_scores: the matrix cores) and what follows
+// (attention_weights: the vector unit), which the prompt kernel runs apart.
 // Fragment reads are written as instructions (see common.h): the stage may be one that direct
 // loads of a later block are filling elsewhere in LDS.
+
+// The K row of the stage that lane l32 reads as row l32 of an S^T tile (pi above).
+__device__ __forceinline__ int att_k_row(int l32) { return (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1); }
+
+// S^T [64 positions][32 queries] = K Q^T: two tiles of 32 positions, each one chain over the k
+// steps ascending, from the constant zero.
 template <int HD>
-__device__ __forceinline__ void attention_scores(unsigned st, const bf16x8 (&qf)[HD / 16], int p0, bool whole, int my_pos,
-                                                 int my_lo, float c, int lane, float& m_b, float& l_b, bf16x8 (&pf)[4]) {
+__device__ __forceinline__ void attention_raw_scores(unsigned st, const bf16x8 (&qf)[HD / 16], int lane, f32x16 (&s_acc)[2]) {
   using S = AttStage<HD>;
   constexpr int KS = HD / 16;
   const int l32 = lane & 31, half = lane >> 5;
-  const int k_row = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);
+  const int k_row = att_k_row(l32);
   const unsigned k_at = st + k_row * S::KROW, k_swz = S::k_swizzle(k_row);
-
-  // S^T [64 positions][32 queries] = K Q^T: two tiles of 32 positions, two k steps a group
-  f32x16 s_acc[2];                    // each chain starts from the constant zero
   u32x4 kf[2][4];
   auto read_k = [&](u32x4 (&dst)[4], int ks0) {
 #pragma unroll
@@ -191,9 +195,13 @@ __device__ __forceinline__ void attention_scores(unsigned st, const bf16x8 (&qf)
         s_acc[pt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[g & 1][kk * 2 + pt]),
                                                             qf[2 * g + kk], g + kk == 0 ? ATT_ZERO16 : s_acc[pt], 0, 0, 0);
   }
+}
 
-  // the largest raw score first (the scale is positive), then exp2(score * c - max * c) in one
-  // multiply-add each
+// From the raw scores (which it uses up): the largest first (the scale is positive), then
+// exp2(score * c - max * c) in one multiply-add each.
+__device__ __forceinline__ void attention_weights(f32x16 (&s_acc)[2], int p0, bool whole, int my_pos, int my_lo, float c,
+                                                  int lane, float& m_b, float& l_b, bf16x8 (&pf)[4]) {
+  const int half = lane >> 5;
   if (!whole) {
     asm volatile("" ::: "memory");      // a branch of its own: the blocks every column sees whole pay nothing for the mask
 #pragma unroll
@@ -231,6 +239,14 @@ __device__ __forceinline__ void attention_scores(unsigned st, const bf16x8 (&qf)
     for (int j = 0; j < 4; ++j) w.u[j] = pack_bf16(s_acc[pt][e0 + 2 * j], s_acc[pt][e0 + 2 * j + 1]);
     pf[s2] = w.f;
   }
+}
+
+template <int HD>
+__device__ __forceinline__ void attention_scores(unsigned st, const bf16x8 (&qf)[HD / 16], int p0, bool whole, int my_pos,
+                                                 int my_lo, float c, int lane, float& m_b, float& l_b, bf16x8 (&pf)[4]) {
+  f32x16 s_acc[2];
+  attention_raw_scores<HD>(st, qf, lane, s_acc);
+  attention_weights(s_acc, p0, whole, my_pos, my_lo, c, lane, m_b, l_b, pf);
 }
 
 // o_b = V^T P^T [HD][32 queries], one tile of 32 dims after the other: each is one chain of four
@@ -271,6 +287,74 @@ __device__ __forceinline__ void attention_values(unsigned st, const bf16x8 (&pf)
   }
 }
 
+// A block's o_b and the NEXT block's raw scores in one stretch of matrix products, with the fold
+// of o_b into the running output between them: the vector unit works beside the matrix cores only
+// on what the same wave issues between two products or what the SIMD's other wave has to do, so
+// the prompt kernel keeps its two long vector stretches (the weights of a block, the fold) apart
+// from each other and lays the products of two blocks over one of them.  The chains are those of
+// attention_values (stage st_v, this block) and of attention_raw_scores (stage st_k, the next
+// block), instruction for instruction; only their order among each other is new.
+// For a tile dt of 32 dims: V^T k steps 0-1, V^T k steps 2-3, K k step 2 dt, K k step 2 dt + 1,
+// two products each, their fragments read a unit ahead; consume(dt, e0, tile) is called
+// for a half of the tile (eight registers from e0) after each of its two units of K: by then the
+// tile's chain has left the matrix cores, and the products issued just before run meanwhile.
+template <int HD, typename Consume>
+__device__ __forceinline__ void attention_values_and_next_scores(unsigned st_v, const bf16x8 (&pf)[4], unsigned st_k,
+                                                                 const bf16x8 (&qf)[HD / 16], int lane, f32x16 (&s_acc)[2],
+                                                                 Consume consume) {
+  using S = AttStage<HD>;
+  constexpr int DT = HD / 32, UNITS = 4 * DT;
+  static_assert(HD / 16 == 2 * DT, "two k steps of S^T for every tile of o");
+  const int l32 = lane & 31, half = lane >> 5;
+  const int k_row = att_k_row(l32);
+  // A row of the stage starts at a multiple of its size, and an even chunk number c plus `half` is
+  // c ^ half, so the address of chunk (c + half) ^ swizzle of a row is that of chunk half ^ swizzle
+  // with c exclusive-ored in: one instruction from a base each.  The bases are made opaque, or the
+  // compiler keeps every address in a register of its own across the whole loop of blocks and
+  // runs out of registers.
+  unsigned v_base = st_v + S::K_BYTES + l32 * 128 + ((half ^ S::v_swizzle(l32)) << 4);
+  unsigned k_base = st_k + k_row * S::KROW + ((half ^ S::k_swizzle(k_row)) << 4);
+  asm volatile("" : "+v"(v_base), "+v"(k_base));
+  u32x4 fr[2][2];
+  auto read_unit = [&](u32x4 (&dst)[2], int u) {
+    const int dt = u >> 2, w = u & 3;
+    if (w < 2) {                        // V^T k steps 2 w and 2 w + 1 of tile dt: chunks 4 w + half and 4 w + 2 + half
+      lds_read16_step<32 * 128, DT>(dst[0], v_base ^ ((4 * w) << 4), dt);
+      lds_read16_step<32 * 128, DT>(dst[1], v_base ^ ((4 * w + 2) << 4), dt);
+    } else {                            // K k step ks, the two tiles of 32 positions
+      const int ks = 2 * dt + (w - 2);
+      const unsigned at = k_base ^ (ks << 5);
+      lds_read16<0>(dst[0], at);
+      lds_read16<32 * S::KROW>(dst[1], at);
+    }
+  };
+  f32x16 tile;
+  read_unit(fr[0], 0);
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u) {
+    const int dt = u >> 2, w = u & 3;
+    if (u + 1 < UNITS) {
+      read_unit(fr[(u + 1) & 1], u + 1);
+      wait_lgkmcnt<2>();
+    } else {
+      wait_lgkmcnt<0>();
+    }
+    use_frags<2>(fr[u & 1]);
+    if (w < 2) {
+      tile = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fr[u & 1][0]), pf[2 * w],
+                                                     w == 0 ? ATT_ZERO16 : tile, 0, 0, 0);
+      tile = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fr[u & 1][1]), pf[2 * w + 1], tile, 0, 0, 0);
+    } else {
+      const int ks = 2 * dt + (w - 2);
+#pragma unroll
+      for (int pt = 0; pt < 2; ++pt)
+        s_acc[pt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fr[u & 1][pt]), qf[ks],
+                                                            ks == 0 ? ATT_ZERO16 : s_acc[pt], 0, 0, 0);
+      consume(dt, 8 * (w - 2), tile);
+    }
+  }
+}
+
 // The same chains with the V^T fragments in registers (the decoding kernel loads them straight
 // from the pages): vf[dt][s2] is what attention_values reads from the stage for tile dt, k step s2.
 template <int HD, typename Consume>
@@ -296,14 +380,12 @@ __device__ __forceinline__ void attention_fold(float& m, float& l, float m_b, fl
   m = mn;
 }
 
-// fma(o, a, o_b b), written as the three-address instruction: left to itself the compiler takes the
-// two-address form, whose result lands in the product's register, and moves every value back
-// into the loop's own register afterwards (64 moves a block of positions).
-__device__ __forceinline__ float attention_fold_value(float o, float a, float o_b, float b) {
+// o = fma(o, a, o_b b), written as the instruction with o's register as its result: left to itself
+// the compiler puts the result where the product was and moves every value back into the loop's
+// own register afterwards (64 moves a block of positions, and as many registers held twice).
+__device__ __forceinline__ void attention_fold_into(float& o, float a, float o_b, float b) {
   const float t = __fmul_rn(o_b, b);
-  float r;
-  asm("v_fma_f32 %0, %1, %2, %3" : "=v"(r) : "v"(o), "v"(a), "v"(t));
-  return r;
+  asm("v_fma_f32 %0, %0, %1, %2" : "+v"(o) : "v"(a), "v"(t));
 }
 
 __device__ __forceinline__ float attention_inverse(float l) { return __fdiv_rn(1.0f, l); }
@@ -315,8 +397,11 @@ __device__ __forceinline__ float attention_inverse(float l) { return __fdiv_rn(1
 // bytes a cycle and CU, which is what one head's products use up).  Two stages: the next block's
 // loads are in flight while this one is multiplied.
 #define PF_TOKENS 128     // (axk_attention_prefill_tile says so to the caller)
+#ifndef ATT_LATE_WAVE
+#define ATT_LATE_WAVE(w) (((w) >> 2) & 1)
+#endif
 
-template <int HD, int HPB, bool ONE_PAGE>
+template <int HD, int HPB, bool ONE_PAGE, bool LATE>
 __device__ __forceinline__ void
 attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __restrict__ q, int q_stride,
                        const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
@@ -370,7 +455,7 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
   // ONE_PAGE (pages of 64 positions or more): a block lies in one page, known to the whole wave,
   // and the addresses are a scalar base plus a lane's 32-bit offset.
   int k_page[K_INSTR], v_page[V_INSTR];
-  auto lookup = [&](int b) {
+  auto lookup_k = [&](int b) {
     const int p0 = first_block + b * ATT_BLOCK;
     if (ONE_PAGE) {
       k_page[0] = table_row[page_index(p0, page_size)];
@@ -378,23 +463,34 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
     }
 #pragma unroll
     for (int n = 0; n < K_INSTR; ++n) k_page[n] = att_k_page<HD>(n * NW + block_wave, lane, p0, hi, table_row, page_size);
+  };
+  auto lookup_v = [&](int b) {
+    const int p0 = first_block + b * ATT_BLOCK;
+    if (ONE_PAGE) {
+      v_page[0] = table_row[page_index(p0, page_size)];
+      return;
+    }
 #pragma unroll
     for (int n = 0; n < V_INSTR; ++n) v_page[n] = att_v_page<HD>(n * NW + block_wave, lane, p0, hi, table_row, page_size);
   };
-  auto issue = [&](int b) {
+  auto issue_k = [&](int b) {
     unsigned char* stage = smem + (b & 1) * S::BYTES;
     const int p0 = first_block + b * ATT_BLOCK;
 #pragma unroll
     for (int n = 0; n < K_INSTR; ++n)
       att_issue_k<HD>(stage, n * NW + block_wave, lane, ONE_PAGE ? k_page[0] : k_page[n], p0, hi, k_head, page_stride,
                       page_size);
+  };
+  auto issue_v = [&](int b) {
+    unsigned char* stage = smem + (b & 1) * S::BYTES;
+    const int p0 = first_block + b * ATT_BLOCK;
 #pragma unroll
     for (int n = 0; n < V_INSTR; ++n)
-      att_issue_v<HD>(stage, n * NW + block_wave, lane, ONE_PAGE ? k_page[0] : v_page[n], p0, hi, v_head, page_stride,
+      att_issue_v<HD>(stage, n * NW + block_wave, lane, ONE_PAGE ? v_page[0] : v_page[n], p0, hi, v_head, page_stride,
                       page_size);
   };
 
-  f32x16 o_acc[DT];
+  float o_acc[DT][16];              // (plain registers: the fold below names each as an instruction's operand)
 #pragma unroll
   for (int i = 0; i < DT; ++i)
 #pragma unroll
@@ -402,37 +498,78 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
   float m_run = -INFINITY, l_run = 0.0f;
   const float c = scale * LOG2E;
   const unsigned lds0 = (unsigned)(size_t)(lds_ptr_t)smem;
+  // the blocks of which this wave's rows see anything: the first my_blocks of the tile's
+  const int my_blocks = wave_live ? min(n_blocks, (wave_hi - first_block) / ATT_BLOCK + 1) : 0;
 
-  lookup(0);
-  issue(0);
-  if (n_blocks > 1) lookup(1);
-  for (int b = 0; b < n_blocks; ++b) {
-    wait_vmcnt<0>();                  // this wave's part of block b has landed
-    __builtin_amdgcn_s_barrier();     // so has everyone's, and everyone is done with block b - 1
-    if (b + 1 < n_blocks) {
-      issue(b + 1);                   // into the stage block b - 1 has left, under way during block b's products
-      if (b + 2 < n_blocks) lookup(b + 2);
-    }
-    unsigned char* stage = smem + (b & 1) * S::BYTES;
+  // A wave's work on block b is three stretches: the raw scores (matrix cores), the weights (vector
+  // unit), and the block's o_b with its fold (both).  The raw scores of block b + 1 are laid over
+  // the third stretch of block b, so K runs a block ahead of V^T: at the barrier of block b the
+  // keys of block b + 1 and the values of block b have landed, everyone has left the keys of block
+  // b and the values of block b - 1, and their stages take the keys of block b + 2 and the values
+  // of block b + 1.
+  f32x16 s_acc[2];
+  lookup_k(0);
+  lookup_v(0);
+  issue_k(0);
+  issue_v(0);
+  if (n_blocks > 1) {
+    lookup_k(1);
+    lookup_v(1);
+    issue_k(1);
+    if (n_blocks > 2) lookup_k(2);
+  }
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  // what every wave does between the weights of block b and its products, whether it has any or not
+  auto turn_stages = [&](int b) {
     const int p0 = first_block + b * ATT_BLOCK;
+    wait_vmcnt<0>();                  // this wave's part of the keys of block b + 1 and the values of block b has landed
+    __builtin_amdgcn_s_barrier();     // so has everyone's
+    if (b + 2 < n_blocks) {
+      issue_k(b + 2);
+      if (b + 3 < n_blocks) lookup_k(b + 3);
+    }
+    if (b + 1 < n_blocks) {
+      issue_v(b + 1);
+      if (b + 2 < n_blocks) lookup_v(b + 2);
+    }
     if (p0 + ATT_BLOCK - 1 > hi) {
-      att_clear_unwritten<HD>(stage, p0, hi, tid, 64 * NW);
+      att_clear_unwritten<HD>(smem + (b & 1) * S::BYTES, p0, hi, tid, 64 * NW);
       __syncthreads();
     }
-    if (!wave_live || p0 > wave_hi) continue;  // nothing for this wave's rows in this block (all waves reach the barriers)
-
+  };
+  if (my_blocks > 0) attention_raw_scores<HD>(lds0, qf, lane, s_acc);
+  int b = 0;
+  // One path through the body, whatever the block: after the wave's last block the products of
+  // "the next block's scores" run on whatever the other stage holds and are dropped (sixteen
+  // products a tile).  A second path would have the compiler copy the running output between the
+  // registers of the two, and branches around those products alone cost more than the products.
+  for (; b < my_blocks; ++b) {
+    const int p0 = first_block + b * ATT_BLOCK;
     // A block that every row of the wave sees whole needs no mask (all but the blocks on the
     // diagonal and at the window's edge).
     const bool whole = p0 + ATT_BLOCK - 1 <= pos0 + wave * 32 && p0 >= wave_lo;
     float m_b, l_b, a, bb;
     bf16x8 pf[4];
-    attention_scores<HD>(lds0 + (b & 1) * S::BYTES, qf, p0, whole, my_pos, my_lo, c, lane, m_b, l_b, pf);
-    attention_fold(m_run, l_run, m_b, l_b, a, bb);
-    attention_values<HD>(lds0 + (b & 1) * S::BYTES, pf, lane, [&](int dt, const f32x16& tile) {
+    // The two waves of a SIMD take turns: one has its weights done before the barrier and starts
+    // with the products, the other (LATE) starts with its weights, which the first one's
+    // products leave the vector unit free for; and so on, half a block apart.
+    if (!LATE) {
+      attention_weights(s_acc, p0, whole, my_pos, my_lo, c, lane, m_b, l_b, pf);
+      attention_fold(m_run, l_run, m_b, l_b, a, bb);
+    }
+    turn_stages(b);
+    if (LATE) {
+      attention_weights(s_acc, p0, whole, my_pos, my_lo, c, lane, m_b, l_b, pf);
+      attention_fold(m_run, l_run, m_b, l_b, a, bb);
+    }
+    attention_values_and_next_scores<HD>(lds0 + (b & 1) * S::BYTES, pf, lds0 + ((b + 1) & 1) * S::BYTES, qf, lane, s_acc,
+                                         [&](int dt, int e0, const f32x16& tile) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) o_acc[dt][e] = attention_fold_value(o_acc[dt][e], a, tile[e], bb);
+      for (int e = e0; e < e0 + 8; ++e) attention_fold_into(o_acc[dt][e], a, tile[e], bb);
     });
   }
+  for (; b < n_blocks; ++b) turn_stages(b);   // (all waves reach the barriers)
 
   if (!wave_live || my_row >= count) return;
   const float inv = attention_inverse(l_run);
@@ -453,25 +590,30 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
 // the second count 0 if there is none.  The caller pairs a tile that sees many positions with
 // one that sees few, so that every block has about the same work (a causal prompt's tiles see
 // 1, 2, 3 ... blocks of positions).
-template <int HD, int HPB>
+// ONE_PAGE (pages of 64 positions or more, the launch's choice): each has its own addressing, and a
+// kernel that held both would keep the lane's constants of both in registers.
+template <int HD, int HPB, bool ONE_PAGE>
 __global__ void __launch_bounds__(256 * HPB, 2)
 attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                          const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
                          const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
                          bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int n_heads, int n_kv_heads,
                          int page_size, int window, float scale) {
-  extern __shared__ __align__(16) unsigned char smem[];
+  extern __shared__ __align__(256) unsigned char smem[];       // (a stage's rows start at multiples of their size)
   const int32_t* mine = tiles + 4 * blockIdx.x;
   for (int part = 0; part < 2; ++part) {
     const int t0 = mine[2 * part], count = mine[2 * part + 1];
     if (count <= 0) break;                        // the same for the whole block
     if (part) __syncthreads();                    // everyone has read the first tile's last stage
-    if (page_size >= ATT_BLOCK)
-      attention_prefill_tile<HD, HPB, true>(smem, t0, count, q, q_stride, k_cache, v_cache, block_table, table_stride,
-                                            positions, seq_rows, out, n_heads, n_kv_heads, page_size, window, scale);
+    // waves w and w + 4 of a block share a SIMD: with two heads a block, the second head's waves are the late ones
+    if (HPB == 2 && ATT_LATE_WAVE(__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)))
+      attention_prefill_tile<HD, HPB, ONE_PAGE, true>(smem, t0, count, q, q_stride, k_cache, v_cache, block_table,
+                                                      table_stride, positions, seq_rows, out, n_heads, n_kv_heads, page_size,
+                                                      window, scale);
     else
-      attention_prefill_tile<HD, HPB, false>(smem, t0, count, q, q_stride, k_cache, v_cache, block_table, table_stride,
-                                             positions, seq_rows, out, n_heads, n_kv_heads, page_size, window, scale);
+      attention_prefill_tile<HD, HPB, ONE_PAGE, false>(smem, t0, count, q, q_stride, k_cache, v_cache, block_table,
+                                                       table_stride, positions, seq_rows, out, n_heads, n_kv_heads, page_size,
+                                                       window, scale);
   }
 }
 
@@ -677,13 +819,13 @@ attention_combine_kernel(const float* __restrict__ partial, const int32_t* __res
       for (int j = 0; j < 16; ++j) {
         const float fa = old_factor[i + j], fb = new_factor[i + j];
         l = __builtin_fmaf(l, fa, __fmul_rn(block_sum[i + j], fb));
-        o = attention_fold_value(o, fa, ob[j], fb);
+        attention_fold_into(o, fa, ob[j], fb);
       }
     }
     for (; i < n; ++i) {
       const float fa = old_factor[i], fb = new_factor[i];
       l = __builtin_fmaf(l, fa, __fmul_rn(block_sum[i], fb));
-      o = attention_fold_value(o, fa, src[(size_t)(g0 + i) * (HD + 2) + d], fb);
+      attention_fold_into(o, fa, src[(size_t)(g0 + i) * (HD + 2) + d], fb);
     }
     for (int w = 0; w < HD / 64; ++w) m = fmaxf(m, wave_max[w]);     // blocks past n count as -inf
   }
@@ -717,13 +859,13 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
               q_stride);
   if (n_tiles == 0) return 0;
   const int group = n_heads / n_kv_heads;
-#define LAUNCH(HD, HPB)                                                                                             \
+#define LAUNCH_PAGED(HD, HPB, ONE_PAGE)                                                                             \
   {                                                                                                                 \
     static bool configured = false;                                                                                 \
     constexpr int lds = 2 * (ATT_BLOCK * HD * 2 + HD * ATT_BLOCK * 2);                                                \
     const dim3 grid(n_tiles, n_kv_heads * ((group + HPB - 1) / HPB));                                               \
     if (!configured) {                                                                                              \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<HD, HPB>),         \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<HD, HPB, ONE_PAGE>), \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);                          \
       if (e != hipSuccess) {                                                                                        \
         axk_set_error("attention_prefill: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));          \
@@ -731,11 +873,13 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
       }                                                                                                             \
       configured = true;                                                                                            \
     }                                                                                                               \
-    AXK_INSTANCE(INST_ATTENTION_PREFILL, HD, HPB);                                                                  \
-    attention_prefill_kernel<HD, HPB><<<grid, 256 * HPB, lds, (hipStream_t)stream>>>(                               \
+    AXK_INSTANCE(INST_ATTENTION_PREFILL, HD, HPB, ONE_PAGE);                                                        \
+    attention_prefill_kernel<HD, HPB, ONE_PAGE><<<grid, 256 * HPB, lds, (hipStream_t)stream>>>(                     \
         (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_stride,      \
         positions, seq_rows, (bf16_t*)out, tiles, n_heads, n_kv_heads, page_size, window, scale);                   \
   }
+#define LAUNCH(HD, HPB) \
+  if (page_size >= ATT_BLOCK) LAUNCH_PAGED(HD, HPB, 1) else LAUNCH_PAGED(HD, HPB, 0)
   // two query heads of a kv head a block (they share each K and V block in LDS) where that still
   // gives the chip's 256 CUs about a block each; else one head a block
   const int blocks_of_pairs = n_tiles * n_kv_heads * ((group + 1) / 2);
@@ -745,6 +889,7 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
     if (head_dim == 64) LAUNCH(64, 1) else LAUNCH(128, 1)
   }
 #undef LAUNCH
+#undef LAUNCH_PAGED
   AXK_LAUNCH_CHECK("attention_prefill");
   return 0;
 #else

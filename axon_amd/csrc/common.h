@@ -143,6 +143,17 @@ __device__ inline void lds_read16(u32x4& dst, unsigned lds_address) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(lds_address), "n"(OFFSET));
 }
 
+// The same at OFFSET = i STEP, i < MAX a constant once the caller's loop is unrolled.
+template <int STEP, int MAX>
+__device__ __forceinline__ void lds_read16_step(u32x4& dst, unsigned lds_address, int i) {
+  if constexpr (MAX > 0) {
+    if (i == MAX - 1)
+      lds_read16<(MAX - 1) * STEP>(dst, lds_address);
+    else
+      lds_read16_step<STEP, MAX - 1>(dst, lds_address, i);
+  }
+}
+
 // COUNT such reads, STEP bytes apart.
 template <int COUNT, int STEP, int I = 0>
 __device__ inline void read_frags(u32x4 (&dst)[COUNT], unsigned lds_address) {

@@ -319,13 +319,18 @@ CASES = [
     (BF, ["gemm_tile<256,256,4,2,1>"], check_gemm, (BF, 2048, 2608, 64, MODE_SWIGLU)),
     (BF, ["gemm_tile<128,128,2,2,0>", "gemm_split_reduce<1>"], check_then_norm, (100, 256, 1024)),
     (BF, ["gemm_tile<256,256,4,2,0>", "gemm_split_reduce<2>"], check_qkv_rope, (2048, 28, 4, 128, 3584, 64)),
-    # attention on the matrix cores: (head size, query heads a block) and (head size, waves a block)
-    # (one wave a block in the decoding kernel up to 2,560 blocks of positions, four beyond; two heads
-    # a block in the prompt kernel from 200 such blocks on: the long prompts of real models)
-    (BF, ["attention_prefill<64,1>", "attention_decode<64,1>"], check_attention_mfma, (4, 2, 64, 16, 200, 0)),
-    (BF, ["attention_prefill<128,1>", "attention_decode<128,1>"], check_attention_mfma, (7, 1, 128, 64, 333, 90)),
-    (BF, ["attention_prefill<64,2>", "attention_decode<64,4>"], check_attention_mfma, (32, 1, 64, 64, 1700, 0, 5)),
-    (BF, ["attention_prefill<128,2>", "attention_decode<128,4>"], check_attention_mfma, (14, 2, 128, 16, 3400, 0, 37)),
+    # attention on the matrix cores: (head size, query heads a block, pages of 64 positions or more)
+    # and (head size, waves a block) (one wave a block in the decoding kernel up to 2,560 blocks of
+    # positions, four beyond; two heads a block in the prompt kernel from 200 such blocks on: the long
+    # prompts of real models)
+    (BF, ["attention_prefill<64,1,0>", "attention_decode<64,1>"], check_attention_mfma, (4, 2, 64, 16, 200, 0)),
+    (BF, ["attention_prefill<64,1,1>"], check_attention_mfma, (4, 2, 64, 64, 200, 0)),
+    (BF, ["attention_prefill<128,1,1>", "attention_decode<128,1>"], check_attention_mfma, (7, 1, 128, 64, 333, 90)),
+    (BF, ["attention_prefill<128,1,0>"], check_attention_mfma, (7, 1, 128, 16, 333, 90)),
+    (BF, ["attention_prefill<64,2,1>", "attention_decode<64,4>"], check_attention_mfma, (32, 1, 64, 64, 1700, 0, 5)),
+    (BF, ["attention_prefill<64,2,0>"], check_attention_mfma, (64, 2, 64, 16, 800, 0, 3)),
+    (BF, ["attention_prefill<128,2,0>", "attention_decode<128,4>"], check_attention_mfma, (14, 2, 128, 16, 3400, 0, 37)),
+    (BF, ["attention_prefill<128,2,1>"], check_attention_mfma, (64, 2, 128, 64, 800, 300, 3)),
 ]
 IDS = [f"{dtype[:2]}-{'+'.join(names)}-{i}" for i, (dtype, names, _, _) in enumerate(CASES)]
 
