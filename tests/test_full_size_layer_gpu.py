@@ -1,6 +1,6 @@
 """One layer of the sizes the engine is measured at (width 3584, 28 query heads on 4 kv heads of
 128, feed-forward 18944) and one of the next size up (width 5120, 40 heads on 8, feed-forward
-13824), with a small vocabulary, against the plain implementation: the tiny configurations of
+13824, and the one after that with a feed-forward of 27648), with a small vocabulary, against the plain implementation: the tiny configurations of
 the other tests never meet the kernels that these widths select (products that split K between
 blocks, norms finished by the product before them, the prompt kernel with a group of 7 or 5,
 decoding over several chunks).  A mixed schedule takes every product through each of its
@@ -27,6 +27,10 @@ WIDER = dict(FULL, hidden_size=5120, intermediate_size=13824, num_attention_head
              rms_norm_eps=1e-5)
 
 
+# and the largest measured size: the same width, a feed-forward twice as wide (K 27,648 for the down projection)
+WIDEST = dict(WIDER, intermediate_size=27648)
+
+
 def _layer_case(tmp_path_factory, sizes, name):
     d = str(tmp_path_factory.mktemp(name))
     write_random_model(config_from_dict(sizes), d, seed=31, std=0.02, storage="bfloat16")
@@ -48,6 +52,11 @@ def wider_layer(tmp_path_factory):
     return _layer_case(tmp_path_factory, WIDER, "wider_layer")
 
 
+@pytest.fixture(scope="module")
+def widest_layer(tmp_path_factory):
+    return _layer_case(tmp_path_factory, WIDEST, "widest_layer")
+
+
 @pytest.mark.parametrize("dtype,page", [("bfloat16", 16), ("bfloat16", 64), ("bfloat16", 8), ("float32", 16)])
 def test_a_layer_of_the_measured_sizes_through_every_class_of_rows(dtype, page, full_layer):
     _through_every_class_of_rows(dtype, page, full_layer)
@@ -55,6 +64,10 @@ def test_a_layer_of_the_measured_sizes_through_every_class_of_rows(dtype, page, 
 
 def test_a_layer_of_the_next_size_through_every_class_of_rows(wider_layer):
     _through_every_class_of_rows("bfloat16", 16, wider_layer)
+
+
+def test_a_layer_of_the_largest_size_through_every_class_of_rows(widest_layer):
+    _through_every_class_of_rows("bfloat16", 16, widest_layer)
 
 
 def _through_every_class_of_rows(dtype, page, case):
