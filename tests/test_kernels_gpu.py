@@ -501,8 +501,34 @@ def test_topk_with_penalty_on_the_device(V, width):
         pen = torch.tensor(pen, dtype=torch.float32)
         assert torch.equal(dev[r].cpu().nan_to_num(7.0), pen.nan_to_num(7.0))   # penalised in place, each id once
         want = [i for _, i in P.candidates(pen.tolist(), int(ks[r]))]
-        got = sorted(cands[r, :int(ks[r])].tolist(), reverse=True)
+        got = sorted((c & 0xFFFFFFFFFFFFFFFF for c in cands[r, :int(ks[r])].tolist()), reverse=True)   # keys are unsigned
         assert [g & 0xFFFFFFFF for g in got] == want, r
+
+
+@pytest.mark.parametrize("V", [1, 2, 7, 64, 65, 300])
+def test_topk_of_a_whole_small_vocabulary(V):
+    """k as large as the vocabulary: logits of both signs, zeros of both signs, infinities and NaN
+    all among the candidates, in the plain sampler's order (NaN last, equal logits: the larger id
+    first; src/sample.rs:280-305, 391-429)."""
+    k = kernels("float32")
+    logits = rnd(5, V, seed=21, scale=2.0)
+    if V >= 7:
+        logits[0, 1], logits[0, 3] = 0.0, -0.0
+        logits[1, 2], logits[1, 5] = float("nan"), float("-inf")
+        logits[2, 0], logits[2, 6] = float("inf"), float("nan")
+        logits[3, 4] = logits[3, 2] = logits[3].max() + 1
+    else:
+        logits[1, 0] = float("nan")
+        logits[2, V - 1] = float("-inf")
+    ks = torch.full((5,), V, dtype=torch.int32)
+    dev = logits.clone().cuda()
+    cands = torch.zeros(5, max(V, 8), dtype=torch.int64, device="cuda")
+    none = torch.zeros(5, 8, dtype=torch.int32, device="cuda")
+    k.topk(dev, none, torch.zeros(5, dtype=torch.int32, device="cuda"), torch.ones(5, device="cuda"), ks.cuda(), cands, k_max=V)
+    for r in range(5):
+        want = [i for _, i in P.candidates(logits[r].tolist(), V)]
+        got = sorted((c & 0xFFFFFFFFFFFFFFFF for c in cands[r, :V].tolist()), reverse=True)
+        assert [g & 0xFFFFFFFF for g in got] == want, (V, r)
 
 
 # --------------------------------------------------------------------------- matrix-core attention
