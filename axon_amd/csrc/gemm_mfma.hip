@@ -106,14 +106,32 @@ gemm_tile_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-  // Block numbering: every eighth block runs on the same XCD; give one XCD consecutive m
-  // blocks of the same n block, so a weight tile is fetched into one L2 and reused there.
+  // Block numbering: every eighth block runs on the same XCD, 32 of them at a time.  An XCD takes
+  // every eighth n block and walks its share in squares of up to 8 m blocks x 4 n blocks, so that
+  // the 32 blocks at work share 12 tiles of operands in that XCD's L2 (with many m blocks, all m
+  // blocks of one n block in a row would share 33), the squares of the same four n blocks one
+  // after the other.
   const int bid = blockIdx.x;
   int mb, nb;
   if (bid < (n_blocks / 8) * 8 * m_blocks) {
-    const int xcd = bid & 7, j = bid >> 3;
-    nb = (j / m_blocks) * 8 + xcd;
-    mb = j % m_blocks;
+    constexpr int GM = 8, GN = 4;
+    const int xcd = bid & 7, j = bid >> 3, mine = n_blocks / 8;       // this XCD's n blocks: xcd, xcd + 8, ...
+    const int whole_groups = mine / GN;
+    int g = j / (GN * m_blocks), rest = j % (GN * m_blocks), gn = GN;
+    if (g >= whole_groups) {                                          // the last, narrower group of n blocks
+      g = whole_groups;
+      rest = j - whole_groups * GN * m_blocks;
+      gn = mine - whole_groups * GN;
+    }
+    const int whole_rows = m_blocks / GM;
+    int ms = rest / (gn * GM), r = rest % (gn * GM), gm = GM;
+    if (ms >= whole_rows) {                                           // the last, shorter square
+      ms = whole_rows;
+      r = rest - whole_rows * gn * GM;
+      gm = m_blocks - whole_rows * GM;
+    }
+    mb = ms * GM + r % gm;
+    nb = (g * GN + r / gm) * 8 + xcd;
   } else {  // the last, incomplete group of n blocks: plain order
     const int r = bid - (n_blocks / 8) * 8 * m_blocks;
     nb = (n_blocks / 8) * 8 + r / m_blocks;
