@@ -10,8 +10,8 @@
 // The block size does not depend on the page size, the batch or the context length, so a
 // token's result is the same however the step was cut.
 //
-// attention_rows: one wave per (token, query head), any head_dim that is a multiple of 16 up
-// to 256, any page size, any window.  Prefill portions and decode tokens alike.
+// attention_rows: one wave (or eight, see below) per (token, query head), any head_dim that is a
+// multiple of 16 up to 256, any page size, any window.  Prefill portions and decode tokens alike.
 #include <math.h>
 
 #include "api.h"
@@ -27,23 +27,28 @@ __device__ inline const elem_t* cache_row(const elem_t* base, const int32_t* tab
   return base + (((size_t)page * n_kv_heads + kvh) * page_size + (pos % page_size)) * head_dim;
 }
 
-__global__ void __launch_bounds__(AXON_WAVE)
+// WAVES waves a block take WAVES neighbouring blocks of 64 positions at a time, each wave its own,
+// and every wave then folds them in ascending order (all waves hold the same running values):
+// the arithmetic of a wave alone, spread over more of the chip when tokens x heads are few.
+template <int WAVES>
+__global__ void __launch_bounds__(AXON_WAVE * WAVES)
 attention_rows_kernel(const elem_t* __restrict__ q, int q_stride, const elem_t* __restrict__ k_cache,
                       const elem_t* __restrict__ v_cache, const int32_t* __restrict__ block_table, int table_stride,
                       const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
                       elem_t* __restrict__ out, int n_heads, int n_kv_heads, int head_dim, int page_size, int window,
-                      float scale) {
+                      float scale, bool vec_k) {
   __shared__ float qs[ATT_MAX_HD];
-  __shared__ float es[ATT_BLOCK];
-  __shared__ const elem_t* vrow[ATT_BLOCK];
-  const int t = blockIdx.x, qh = blockIdx.y, lane = threadIdx.x;
+  __shared__ float es[WAVES][ATT_BLOCK];
+  __shared__ const elem_t* vrow[WAVES][ATT_BLOCK];
+  __shared__ float part[WAVES][WAVES > 1 ? ATT_MAX_HD + 2 : 1];   // a wave's block: o_b, then m_b and l_b
+  const int t = blockIdx.x, qh = blockIdx.y, lane = threadIdx.x % AXON_WAVE, wave = threadIdx.x / AXON_WAVE;
   const int kvh = qh / (n_heads / n_kv_heads);
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
   const int32_t* table_row = block_table + (size_t)seq_rows[t] * table_stride;
 
   const elem_t* qrow = q + (size_t)t * q_stride + (size_t)qh * head_dim;
-  for (int d = lane; d < head_dim; d += AXON_WAVE) qs[d] = to_float(qrow[d]);
+  for (int d = threadIdx.x; d < head_dim; d += AXON_WAVE * WAVES) qs[d] = to_float(qrow[d]);
   __syncthreads();
 
   constexpr int DPL = ATT_MAX_HD / AXON_WAVE;  // output dims per lane at most
@@ -51,45 +56,72 @@ attention_rows_kernel(const elem_t* __restrict__ q, int q_stride, const elem_t* 
 #pragma unroll
   for (int i = 0; i < DPL; ++i) O[i] = 0.0f;
 
-  for (int b0 = (lo / ATT_BLOCK) * ATT_BLOCK; b0 <= pos; b0 += ATT_BLOCK) {
+  for (int g0 = (lo / ATT_BLOCK) * ATT_BLOCK; g0 <= pos; g0 += ATT_BLOCK * WAVES) {
+    const int b0 = g0 + ATT_BLOCK * wave;   // this wave's block; beyond pos it only keeps the barriers' count
     const int p = b0 + lane;
     const bool live = p >= lo && p <= pos;
     float s = -INFINITY;
     if (live) {
       const elem_t* kr = cache_row(k_cache, table_row, p, page_size, n_kv_heads, kvh, head_dim);
       float dot = 0.0f;
-      for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
+      for (int d = 0; d < head_dim; d += 4) {   // head_dim is a multiple of 16
+        float k4[4];
+        load4_guarded(kr + d, 4, vec_k, k4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dot = fmaf(qs[d + i], k4[i], dot);
+      }
       s = dot * scale;
-      vrow[lane] = v_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * head_dim * page_size + (p % page_size);
+      vrow[wave][lane] =
+          v_cache + ((size_t)table_row[p / page_size] * n_kv_heads + kvh) * head_dim * page_size + (p % page_size);
     }
     const float mb = wave_max(s);
     const float e = live ? expf(s - mb) : 0.0f;
     const float lb = wave_sum(e);
-    es[lane] = e;
+    es[wave][lane] = e;
     __syncthreads();
     float ob[DPL];
 #pragma unroll
     for (int i = 0; i < DPL; ++i) ob[i] = 0.0f;
     const int first = max(lo - b0, 0), last = min(pos - b0, ATT_BLOCK - 1);
     for (int j = first; j <= last; ++j) {
-      const float ej = es[j];
-      const elem_t* vr = vrow[j];
+      const float ej = es[wave][j];
+      const elem_t* vr = vrow[wave][j];
 #pragma unroll
       for (int i = 0; i < DPL; ++i) {
         const int d = lane + i * AXON_WAVE;
         if (d < head_dim) ob[i] = fmaf(ej, to_float(vr[(size_t)d * page_size]), ob[i]);
       }
     }
-    __syncthreads();
-    const float mn = fmaxf(M, mb);
-    const float alpha = expf(M - mn);
-    const float wgt = expf(mb - mn);
-    L = fmaf(lb, wgt, L * alpha);
+    if (WAVES > 1) {
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) O[i] = fmaf(ob[i], wgt, O[i] * alpha);
-    M = mn;
+      for (int i = 0; i < DPL; ++i) {
+        const int d = lane + i * AXON_WAVE;
+        if (d < head_dim) part[wave][d] = ob[i];
+      }
+      if (lane == 0) {
+        part[wave][ATT_MAX_HD] = mb;
+        part[wave][ATT_MAX_HD + 1] = lb;
+      }
+    }
+    __syncthreads();
+    for (int w = 0; w < WAVES && g0 + ATT_BLOCK * w <= pos; ++w) {
+      const float m_w = WAVES > 1 ? part[w][ATT_MAX_HD] : mb, l_w = WAVES > 1 ? part[w][ATT_MAX_HD + 1] : lb;
+      const float mn = fmaxf(M, m_w);
+      const float alpha = expf(M - mn);
+      const float wgt = expf(m_w - mn);
+      L = fmaf(l_w, wgt, L * alpha);
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const int d = lane + i * AXON_WAVE;
+        const float o_w = WAVES > 1 ? (d < head_dim ? part[w][d] : 0.0f) : ob[i];
+        O[i] = fmaf(o_w, wgt, O[i] * alpha);
+      }
+      M = mn;
+    }
+    if (WAVES > 1) __syncthreads();   // the next round writes `part` again
   }
 
+  if (wave != 0) return;
   elem_t* orow = out + ((size_t)t * n_heads + qh) * head_dim;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) {
@@ -112,10 +144,15 @@ extern "C" int axk_attention(const void* q, int q_stride, const void* k_cache, c
   AXK_REQUIRE(window >= 0, "attention: window %d is negative", window);
   if (n_tokens == 0) return 0;
   dim3 grid(n_tokens, n_heads);
-  AXK_INSTANCE(INST_ATTENTION_ROWS, AXON_BF16);
-  attention_rows_kernel<<<grid, AXON_WAVE, 0, (hipStream_t)stream>>>(
-      (const elem_t*)q, q_stride, (const elem_t*)k_cache, (const elem_t*)v_cache, block_table, table_stride, positions,
-      seq_rows, (elem_t*)out, n_heads, n_kv_heads, head_dim, page_size, window, scale);
+  const bool vec_k = (uintptr_t)k_cache % (4 * sizeof(elem_t)) == 0;
+#define ROWS_LAUNCH(WAVES)                                                                                         \
+  AXK_INSTANCE(INST_ATTENTION_ROWS, AXON_BF16, WAVES);                                                             \
+  attention_rows_kernel<WAVES><<<grid, AXON_WAVE * WAVES, 0, (hipStream_t)stream>>>(                               \
+      (const elem_t*)q, q_stride, (const elem_t*)k_cache, (const elem_t*)v_cache, block_table, table_stride,      \
+      positions, seq_rows, (elem_t*)out, n_heads, n_kv_heads, head_dim, page_size, window, scale, vec_k)
+  // few tokens x heads (a decoding step): eight waves each, so that the chip has waves to run
+  if ((long)n_tokens * n_heads < 1024) { ROWS_LAUNCH(8); } else { ROWS_LAUNCH(1); }
+#undef ROWS_LAUNCH
   AXK_LAUNCH_CHECK("attention_rows");
   return 0;
 }

@@ -73,6 +73,27 @@ __device__ inline float load_vec(const void* p, int is_f32, int i) {
   return is_f32 ? ((const float*)p)[i] : bf16_to_float(((const bf16_t*)p)[i]);
 }
 
+// Four consecutive elements as floats: one 8- or 16-byte load where `vec` says the address is
+// aligned for it and all four exist, else the `valid` first ones singly and zeros behind them.
+__device__ inline void load4_guarded(const elem_t* __restrict__ p, int valid, bool vec, float out[4]) {
+  if (vec && valid >= 4) {
+#if AXON_BF16
+    const uint2 raw = *reinterpret_cast<const uint2*>(p);
+    union { uint32_t u; float f; } c;
+    c.u = raw.x << 16; out[0] = c.f;
+    c.u = raw.x & 0xffff0000u; out[1] = c.f;
+    c.u = raw.y << 16; out[2] = c.f;
+    c.u = raw.y & 0xffff0000u; out[3] = c.f;
+#else
+    const float4 raw = *reinterpret_cast<const float4*>(p);
+    out[0] = raw.x; out[1] = raw.y; out[2] = raw.z; out[3] = raw.w;
+#endif
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = i < valid ? to_float(p[i]) : 0.0f;
+  }
+}
+
 // ---------------------------------------------------------------------------- reductions
 // Butterfly over the 64 lanes of a wave: every lane ends with the same value, and the order
 // of the additions is fixed by the lane numbers alone.

@@ -15,25 +15,6 @@
 #define FMA_BK 16
 #define FMA_THREADS 256
 
-__device__ inline void load4_guarded(const elem_t* __restrict__ p, int valid, bool vec, float out[4]) {
-  if (vec && valid >= 4) {
-#if AXON_BF16
-    const uint2 raw = *reinterpret_cast<const uint2*>(p);
-    union { uint32_t u; float f; } c;
-    c.u = raw.x << 16; out[0] = c.f;
-    c.u = raw.x & 0xffff0000u; out[1] = c.f;
-    c.u = raw.y << 16; out[2] = c.f;
-    c.u = raw.y & 0xffff0000u; out[3] = c.f;
-#else
-    const float4 raw = *reinterpret_cast<const float4*>(p);
-    out[0] = raw.x; out[1] = raw.y; out[2] = raw.z; out[3] = raw.w;
-#endif
-  } else {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) out[i] = i < valid ? to_float(p[i]) : 0.0f;
-  }
-}
-
 // BM rows x 64 columns per block of 256 threads; thread (ty, tx) owns RM = BM / 16 rows and
 // 4 columns.  K is walked in steps of 16 through LDS; inside a step k ascends.
 template <int BM, bool GLU>
@@ -125,6 +106,83 @@ gemm_fma_kernel(const elem_t* __restrict__ x, int x_stride, const elem_t* __rest
   }
 }
 
+// Up to 16 rows (a decoding step): 16 rows x 16 columns a block, one output a thread, K in steps
+// of 256 through LDS, the next step's loads in flight while this one is multiplied.  Such a
+// product only waits for W, so it wants many blocks with much in flight each (the tile above
+// gives N / 64 blocks with 4 KB each).  The chain of an output is the same: fmaf in ascending k.
+#define FEW_BK 256
+#define FEW_LD (FEW_BK + 4)   // rows 4 banks apart: the 16 rows a wave reads fall into all 64 banks
+template <bool GLU>
+__global__ void __launch_bounds__(FMA_THREADS)
+gemm_fma_few_rows_kernel(const elem_t* __restrict__ x, int x_stride, const elem_t* __restrict__ w,
+                         const void* __restrict__ bias, int bias_is_f32, void* __restrict__ out, int out_stride, int M,
+                         int N, int K, int mode, bool vec_x, bool vec_w) {
+  __shared__ __align__(16) float xs[16][FEW_LD];
+  __shared__ __align__(16) float ws[16][FEW_LD];
+  __shared__ __align__(16) float us[GLU ? 16 : 1][GLU ? FEW_LD : 4];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const int n0 = blockIdx.x * 16;
+
+  // loader: a tile is 16 rows of 64 groups of four k; a thread brings groups tid + 256 j
+  float px[4][4], pw[4][4], pu[GLU ? 4 : 1][4];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int g = tid + FMA_THREADS * j, row = g >> 6, k = k0 + 4 * (g & 63);
+      const int left = max(0, min(4, K - k)), n = n0 + row;
+      load4_guarded(x + (size_t)row * x_stride + k, row < M ? left : 0, vec_x, px[j]);
+      load4_guarded(w + (size_t)n * K + k, n < N ? left : 0, vec_w, pw[j]);
+      if (GLU) load4_guarded(w + (size_t)(N + n) * K + k, n < N ? left : 0, vec_w, pu[j]);
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int g = tid + FMA_THREADS * j, row = g >> 6, kk = 4 * (g & 63);
+      *reinterpret_cast<float4*>(&xs[row][kk]) = make_float4(px[j][0], px[j][1], px[j][2], px[j][3]);
+      *reinterpret_cast<float4*>(&ws[row][kk]) = make_float4(pw[j][0], pw[j][1], pw[j][2], pw[j][3]);
+      if (GLU) *reinterpret_cast<float4*>(&us[row][kk]) = make_float4(pu[j][0], pu[j][1], pu[j][2], pu[j][3]);
+    }
+  };
+
+  float acc = 0.0f, acc_up = 0.0f;
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += FEW_BK) {
+    stage();
+    __syncthreads();
+    if (k0 + FEW_BK < K) fetch(k0 + FEW_BK);
+    const int k_end = min(FEW_BK, K - k0);   // beyond K the last group of four holds zeros
+#pragma unroll 4
+    for (int kk = 0; kk < k_end; kk += 4) {
+      const float4 a = *reinterpret_cast<const float4*>(&xs[ty][kk]);
+      const float4 b = *reinterpret_cast<const float4*>(&ws[tx][kk]);
+      acc = fmaf(a.x, b.x, acc);
+      acc = fmaf(a.y, b.y, acc);
+      acc = fmaf(a.z, b.z, acc);
+      acc = fmaf(a.w, b.w, acc);
+      if (GLU) {
+        const float4 u = *reinterpret_cast<const float4*>(&us[tx][kk]);
+        acc_up = fmaf(a.x, u.x, acc_up);
+        acc_up = fmaf(a.y, u.y, acc_up);
+        acc_up = fmaf(a.z, u.z, acc_up);
+        acc_up = fmaf(a.w, u.w, acc_up);
+      }
+    }
+    __syncthreads();
+  }
+
+  const int m = ty, n = n0 + tx;
+  if (m >= M || n >= N) return;
+  float v = acc;
+  if (bias) v += load_vec(bias, bias_is_f32, n);
+  const size_t at = (size_t)m * out_stride + n;
+  if (GLU) ((elem_t*)out)[at] = from_float(swiglu1(v, acc_up));
+  else if (mode == MODE_STORE) ((elem_t*)out)[at] = from_float(v);
+  else if (mode == MODE_ADD_F32) ((float*)out)[at] += v;
+  else ((float*)out)[at] = v;
+}
+
 static int launch_fma(const elem_t* x, int x_stride, const elem_t* w, const void* bias, int bias_is_f32, void* out,
                       int out_stride, int m, int n, int k, int mode, hipStream_t stream) {
   const size_t vbytes = 4 * sizeof(elem_t);
@@ -132,8 +190,12 @@ static int launch_fma(const elem_t* x, int x_stride, const elem_t* w, const void
   const bool vec_x = (k % 4 == 0) && (x_stride % 4 == 0) && ((uintptr_t)x % vbytes == 0);
 #define FMA_LAUNCH(BM, GLU)                                                                                      \
   AXK_INSTANCE(INST_GEMM_FMA, BM, GLU);                                                                          \
-  gemm_fma_kernel<BM, GLU><<<dim3(ceil_div(n, FMA_BN), ceil_div(m, BM)), FMA_THREADS, 0, stream>>>(              \
-      x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, vec_x, vec_w)
+  if (BM == 16)                                                                                                  \
+    gemm_fma_few_rows_kernel<GLU><<<dim3(ceil_div(n, 16)), FMA_THREADS, 0, stream>>>(                            \
+        x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, vec_x, vec_w);                        \
+  else                                                                                                           \
+    gemm_fma_kernel<64, GLU><<<dim3(ceil_div(n, FMA_BN), ceil_div(m, 64)), FMA_THREADS, 0, stream>>>(            \
+        x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, vec_x, vec_w)
   if (mode == MODE_SWIGLU) {
     if (m <= 16) { FMA_LAUNCH(16, true); } else { FMA_LAUNCH(64, true); }
   } else {

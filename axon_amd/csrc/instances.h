@@ -22,7 +22,7 @@ enum {
   INST_GEMM_NORMED,          // tile pairs a wave, segments, epilogue, rows of X in LDS, float4 a lane
   INST_GEMM_ROWS,            // row tiles, waves, epilogue
   INST_GEMM_SPLIT_REDUCE,    // 0 plain, 1 with the norm, 2 with the rotary store
-  INST_ATTENTION_ROWS,
+  INST_ATTENTION_ROWS,       // bfloat16 build, waves a (token, head)
   INST_ATTENTION_PREFILL,    // head_dim, query heads a block, pages of 64 positions or more
   INST_ATTENTION_DECODE,     // head_dim, waves a block
   INST_RMSNORM,              // 1: rows read as float4

@@ -180,6 +180,12 @@ def check_attention_rows(dtype, nh, nkv, hd, page, T, window):
     hit = launched(k, dtype, lambda: k.attention(q, nh * hd, kc, vc, table, pos, rows, out, nh, nkv, hd, page, window,
                                                   1.0 / math.sqrt(hd)))
     assert (out.cpu().double() - ref).abs().max() <= tol(dtype, ref, 2e-6, 1e-2)
+    # the last tokens alone (few tokens: eight waves each) give the bits they have among all of them
+    few = min(T, 1023 // nh, 40)
+    alone = torch.empty(few, nh * hd, dtype=q.dtype, device="cuda")
+    k.attention(q[T - few:], nh * hd, kc, vc, table, pos[T - few:], rows[T - few:], alone, nh, nkv, hd, page, window,
+                1.0 / math.sqrt(hd))
+    assert torch.equal(alone, out[T - few:])
     return hit
 
 
@@ -236,8 +242,11 @@ CASES = [
     (F32, ["rmsnorm<1>"], check_rmsnorm, (F32, 3584)),
     (BF, ["rmsnorm<0>"], check_rmsnorm, (BF, 777)),
     (BF, ["rmsnorm<1>"], check_rmsnorm, (BF, 3584)),
-    (F32, ["attention_rows<0>"], check_attention_rows, (F32, 6, 3, 80, 4, 65, 0)),
-    (BF, ["attention_rows<1>"], check_attention_rows, (BF, 4, 2, 32, 16, 133, 37)),
+    # eight waves a (token, head) below 1,024 of them, one from there
+    (F32, ["attention_rows<0,8>"], check_attention_rows, (F32, 6, 3, 80, 4, 65, 0)),
+    (F32, ["attention_rows<0,1>"], check_attention_rows, (F32, 6, 3, 80, 4, 700, 0)),
+    (BF, ["attention_rows<1,8>"], check_attention_rows, (BF, 4, 2, 32, 16, 133, 37)),
+    (BF, ["attention_rows<1,1>"], check_attention_rows, (BF, 4, 2, 32, 16, 600, 37)),
     # up to 16 rows: a wave a segment of K.  One row tile a block below 16,384 rows of W, two from there
     (BF, ["gemm_stream<1,1,1,0>"], check_gemm, (BF, 3, 100, 128, MODE_STORE, True)),
     (BF, ["gemm_stream<1,1,2,0>"], check_gemm, (BF, 16, 100, 512, MODE_ADD_F32)),
