@@ -30,11 +30,11 @@
 //   norm inside; waves of their own norm the rows into LDS while the streaming waves fill their
 //   rings, so the norm is no launch of its own in a decoding step.
 //
-// * gemm_rows (17 <= M <= 64): W still streams into registers, but the waves of a block walk the
+// * gemm_rows (17 <= M <= 128): W still streams into registers, but the waves of a block walk the
 //   same segment of K and share X through LDS; a block a segment, the sums of several segments
 //   through a workspace.
 //
-// * gemm_tile (M > 64): a block of 4 or 8 waves owns a BM x BN tile of the output, walks K in
+// * gemm_tile (M > 128): a block of 4 or 8 waves owns a BM x BN tile of the output, walks K in
 //   steps of 64 through LDS stages filled by direct global -> LDS loads (the next step's loads
 //   in flight while this one multiplies), and each wave keeps a tile of 32x32x16 MFMA
 //   accumulators.  With S > 1 segments each goes to blocks of its own (gridDim.y = S), whose sums
@@ -1301,11 +1301,11 @@ static int launch_normed(const NormedRows& in, const bf16_t* w, const void* bias
 }
 
 // ---------------------------------------------------------------------------- gemm_rows
-// 17 to 64 rows of X: still bound by reading W once, but X is now as large as a tile of W, and a
+// 17 to 128 rows of X: still bound by reading W once, but X is now as large as a tile of W, and a
 // wave that fetched its own X for every step (as gemm_stream does) would ask the caches for as
 // many bytes of X as of W.  Here the WAVES waves of a block walk the same K together, each
 // with its own NT16 row tiles of W streamed from memory straight into MFMA operands (a ring of
-// NS - 1 steps of 64 k in flight), and share X: a step's X (64 rows x 64 k, 8 KB) goes straight
+// NS - 1 steps of 64 k in flight), and share X: a step's X (16 MT16 rows x 64 k, 8 or 16 KB) goes straight
 // into LDS once a block, in the blocks of 1 KB that one LDS read of a wave takes (16 rows x 32 k,
 // lane l: row l % 16, 8 k from 8 (l / 16)), each wave fetching its share.  One barrier a step:
 // behind it the step's X is there for everyone and the step before is read by everyone, so its
@@ -1314,7 +1314,7 @@ static int launch_normed(const NormedRows& in, const bf16_t* w, const void* bias
 // [segment][gate | up][M][N] and the kernels that add such sums in segment order finish the
 // product.  The chain of an output element is the same as in every other kernel: 16x16x32
 // MFMAs in ascending k from zero over its segment.
-template <int NT16, int WAVES, int NS, int EPI>
+template <int NT16, int MT16, int WAVES, int NS, int EPI>
 __global__ void __launch_bounds__(WAVES * 64, 2)      // two waves a SIMD: 256 registers each
 gemm_rows_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ w, const void* __restrict__ bias,
                  int bias_is_f32, void* __restrict__ out, int out_stride, int M, int N, int K, int mode,
@@ -1322,7 +1322,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   constexpr bool GLU = EPI == EPI_GLU;
   // every wave fetches XI blocks of X a step (where the waves do not divide the blocks, some
   // twice: the same bytes to the same place), so that every wave counts the same loads
-  constexpr int MT16 = 4, XB = MT16 * 2, XI = (XB + WAVES - 1) / WAVES, WI = NT16 * 2, LOADS = XI + WI;
+  constexpr int XB = MT16 * 2, XI = (XB + WAVES - 1) / WAVES, WI = NT16 * 2, LOADS = XI + WI;
   static_assert(EPI == EPI_PLAIN || (EPI == EPI_GLU && NT16 == 2), "plain tiles, or gate and up tiles of the same columns");
   static_assert((NS - 2) * LOADS < 64, "the counter of loads in flight has six bits");
   extern __shared__ __align__(16) unsigned char x_ring[];      // [NS][XB][1 KB]
@@ -1386,18 +1386,25 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
   };
   // one step: behind the barrier its X is in LDS for every wave and nobody reads the step before
   // any more (the bare barrier: the fence of __syncthreads would wait for every load under way)
+  // (the second half of the step's k is read while the first is multiplied)
   auto multiply = [&](int d) {
-    u32x4 xf[XB];
-    read_frags<XB, 1024>(xf, ring0 + d * (XB * 1024) + lane * 16);
+    u32x4 xf[2][MT16];
+    read_frags<MT16, 2048>(xf[0], ring0 + d * (XB * 1024) + lane * 16);
+    read_frags<MT16, 2048>(xf[1], ring0 + d * (XB * 1024) + 1024 + lane * 16);
+    wait_lgkmcnt<MT16>();
+    use_frags<MT16>(xf[0]);
+#pragma unroll
+    for (int i = 0; i < NT16; ++i)
+#pragma unroll
+      for (int j = 0; j < MT16; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[d][i][0]), as_frag(xf[0][j]), acc[i][j], 0, 0, 0);
     wait_lgkmcnt<0>();
-    use_frags<XB>(xf);
+    use_frags<MT16>(xf[1]);
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int i = 0; i < NT16; ++i)
 #pragma unroll
-      for (int i = 0; i < NT16; ++i)
-#pragma unroll
-        for (int j = 0; j < MT16; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[d][i][h]), as_frag(xf[j * 2 + h]), acc[i][j], 0, 0, 0);
+      for (int j = 0; j < MT16; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(wf[d][i][1]), as_frag(xf[1][j]), acc[i][j], 0, 0, 0);
   };
   static_assert(NS >= 4 && NS <= 8, "the ring of steps");
 #pragma unroll
@@ -1452,14 +1459,31 @@ gemm_rows_kernel(const bf16_t* __restrict__ x, int x_stride, const bf16_t* __res
                                     RopeAhead<MT16>());
 }
 
-#define ROWS_NS 8
+// The ring of steps: eight for up to 64 rows; with 128 rows a step's X is 16 KB and the sums take
+// twice the registers, so four steps (two row tiles a wave: 12 KB of W in flight a wave) or six.
+template <int NT16, int MT16>
+struct RowsRing {
+  static constexpr int NS = MT16 <= 4 ? 8 : NT16 == 2 ? 4 : 6;
+};
 
-template <int NT16, int WAVES, int EPI>
+template <int NT16, int MT16, int WAVES, int EPI>
 static int launch_rows_of(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                           int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs, float* partial, int units) {
-  constexpr int lds_bytes = ROWS_NS * 8 * 1024;
-  AXK_INSTANCE(INST_GEMM_ROWS, NT16, WAVES, EPI);
-  gemm_rows_kernel<NT16, WAVES, ROWS_NS, EPI><<<dim3(ceil_div(units, WAVES), segs), WAVES * 64, lds_bytes, stream>>>(
+  constexpr int NS = RowsRing<NT16, MT16>::NS, lds_bytes = NS * MT16 * 2 * 1024;
+  static_assert(lds_bytes <= 160 * 1024, "the ring does not fit the LDS of a CU");
+  auto kernel = &gemm_rows_kernel<NT16, MT16, WAVES, NS, EPI>;
+  static bool configured = lds_bytes <= 64 * 1024;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       lds_bytes);
+    if (e != hipSuccess) {
+      axk_set_error("gemm_rows: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+      return -2;
+    }
+    configured = true;
+  }
+  AXK_INSTANCE(INST_GEMM_ROWS, NT16, MT16, WAVES, EPI);
+  kernel<<<dim3(ceil_div(units, WAVES), segs), WAVES * 64, lds_bytes, stream>>>(
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, segs > 1 ? partial : nullptr, units);
   AXK_LAUNCH_CHECK("gemm_rows");
   return 0;
@@ -1467,23 +1491,26 @@ static int launch_rows_of(const bf16_t* x, int x_stride, const bf16_t* w, const 
 
 // A CU streams at its own pace however many blocks it holds, so the waves of a block are as many
 // as it takes to give each of the chip's 256 CUs one block (at most eight: two a SIMD).
-template <int NT16, int EPI>
+template <int NT16, int MT16, int EPI>
 static int launch_rows(const bf16_t* x, int x_stride, const bf16_t* w, const void* bias, int bias_is_f32, void* out,
                        int out_stride, int m, int n, int k, int mode, hipStream_t stream, int segs, float* partial,
                        const SplitNorm* norm, const RopeStore* rope) {
   const int units = EPI == EPI_GLU ? n / 16 : ceil_div(ceil_div(n, 16), NT16);
+  constexpr int LEAST = MT16 <= 4 ? 2 : 3;      // 128 rows with two waves: each would fetch half of X and spill
   int waves = ceil_div(units * segs, 256);
-  waves = waves < 2 ? 2 : waves > 8 ? 8 : waves;
+  waves = waves < LEAST ? LEAST : waves > 8 ? 8 : waves;
 #define ARGS_ROWS x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, stream, segs, partial, units
   int rc = -1;
   switch (waves) {
-    case 2: rc = launch_rows_of<NT16, 2, EPI>(ARGS_ROWS); break;
-    case 3: rc = launch_rows_of<NT16, 3, EPI>(ARGS_ROWS); break;
-    case 4: rc = launch_rows_of<NT16, 4, EPI>(ARGS_ROWS); break;
-    case 5: rc = launch_rows_of<NT16, 5, EPI>(ARGS_ROWS); break;
-    case 6: rc = launch_rows_of<NT16, 6, EPI>(ARGS_ROWS); break;
-    case 7: rc = launch_rows_of<NT16, 7, EPI>(ARGS_ROWS); break;
-    default: rc = launch_rows_of<NT16, 8, EPI>(ARGS_ROWS); break;
+    case 2:
+      if constexpr (LEAST <= 2) rc = launch_rows_of<NT16, MT16, 2, EPI>(ARGS_ROWS);
+      break;
+    case 3: rc = launch_rows_of<NT16, MT16, 3, EPI>(ARGS_ROWS); break;
+    case 4: rc = launch_rows_of<NT16, MT16, 4, EPI>(ARGS_ROWS); break;
+    case 5: rc = launch_rows_of<NT16, MT16, 5, EPI>(ARGS_ROWS); break;
+    case 6: rc = launch_rows_of<NT16, MT16, 6, EPI>(ARGS_ROWS); break;
+    case 7: rc = launch_rows_of<NT16, MT16, 7, EPI>(ARGS_ROWS); break;
+    default: rc = launch_rows_of<NT16, MT16, 8, EPI>(ARGS_ROWS); break;
   }
 #undef ARGS_ROWS
   if (rc != 0) return rc;
@@ -1698,9 +1725,15 @@ static int gemm_mfma_pass(const bf16_t* x, int x_stride, const bf16_t* w, const 
   const bool glu = mode == MODE_SWIGLU;
   if (m <= 64) {
     // W streamed, X shared through LDS; a block a segment.  Two row tiles a wave where the matrix is large.
-    if (glu) return launch_rows<2, EPI_GLU>(ARGS, segs, ws, nullptr, nullptr);
-    if (n >= 32 * 512) return launch_rows<2, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
-    return launch_rows<1, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
+    if (glu) return launch_rows<2, 4, EPI_GLU>(ARGS, segs, ws, nullptr, nullptr);
+    if (n >= 32 * 512) return launch_rows<2, 4, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
+    return launch_rows<1, 4, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
+  }
+  if (m <= 128) {
+    // the same with 128 rows of X a step: still bound by reading W (a tile kernel's blocks are too few here)
+    if (glu) return launch_rows<2, 8, EPI_GLU>(ARGS, segs, ws, nullptr, nullptr);
+    if (n >= 32 * 512) return launch_rows<2, 8, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
+    return launch_rows<1, 8, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
   }
   if (m <= 256) {
     if (glu) return launch_tile<128, 128, 2, 2, true>(ARGS, segs, ws);

@@ -20,7 +20,7 @@ enum {
   INST_GEMM_TILE,            // BM, BN, waves m, waves n, gated, BK, stages, segments in registers
   INST_GEMM_STREAM,          // row tiles, tiles of X rows, segments, epilogue
   INST_GEMM_NORMED,          // tile pairs a wave, segments, epilogue, rows of X in LDS, float4 a lane
-  INST_GEMM_ROWS,            // row tiles, waves, epilogue
+  INST_GEMM_ROWS,            // row tiles of W a wave, tiles of 16 rows of X, waves, epilogue
   INST_GEMM_SPLIT_REDUCE,    // 0 plain, 1 with the norm, 2 with the rotary store
   INST_ATTENTION_ROWS,       // bfloat16 build, waves a (token, head)
   INST_ATTENTION_PREFILL,    // head_dim, query heads a block, pages of 64 positions or more

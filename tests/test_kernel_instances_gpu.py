@@ -294,39 +294,64 @@ CASES = [
     (BF, ["gemm_normed<1,4,2,8,20>"], check_normed_qkv, (8, 40, 8, 128, 5120, 64)),           # a 14B layer's
     # 17 to 64 rows: W streamed, X shared through LDS; as many waves a block as give each CU a block.
     # With several segments the sums go through the workspace (gemm_split_reduce<0>).
-    (BF, ["gemm_rows<1,2,0>"], check_gemm, (BF, 17, 100, 128, MODE_STORE, True)),
-    (BF, ["gemm_rows<1,3,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 33, 4100, 512, MODE_STORE_F32, True)),
-    (BF, ["gemm_rows<1,4,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 64, 3584, 1024, MODE_ADD_F32)),
-    (BF, ["gemm_rows<1,5,0>"], check_gemm, (BF, 40, 4100, 1024, MODE_STORE)),
-    (BF, ["gemm_rows<1,6,0>"], check_gemm, (BF, 20, 5600, 1024, MODE_STORE_F32)),
-    (BF, ["gemm_rows<1,7,0>"], check_gemm, (BF, 64, 6400, 1024, MODE_ADD_F32, True)),
-    (BF, ["gemm_rows<1,8,0>"], check_gemm, (BF, 48, 9600, 1024, MODE_STORE)),
-    (BF, ["gemm_rows<2,2,0>"], check_gemm, (BF, 17, 16384, 256, MODE_STORE_F32)),
-    (BF, ["gemm_rows<2,3,0>"], check_gemm, (BF, 64, 16400, 256, MODE_STORE_F32, True)),
-    (BF, ["gemm_rows<2,4,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 32, 16384, 512, MODE_STORE_F32)),
-    (BF, ["gemm_rows<2,5,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 17, 16400, 3584, MODE_STORE_F32)),
-    (BF, ["gemm_rows<2,6,0>"], check_gemm, (BF, 64, 20500, 512, MODE_STORE_F32)),
-    (BF, ["gemm_rows<2,7,0>"], check_gemm, (BF, 33, 50000, 256, MODE_STORE_F32)),
-    (BF, ["gemm_rows<2,8,0>"], check_gemm, (BF, 64, 152064, 3584, MODE_STORE_F32)),          # the head of a real model
-    (BF, ["gemm_rows<2,2,1>"], check_gemm, (BF, 40, 96, 64, MODE_SWIGLU)),
-    (BF, ["gemm_rows<2,3,1>"], check_gemm, (BF, 17, 8208, 64, MODE_SWIGLU)),
-    (BF, ["gemm_rows<2,4,1>", "gemm_split_reduce<0>"], check_gemm, (BF, 64, 3584, 1024, MODE_SWIGLU)),
-    (BF, ["gemm_rows<2,5,1>"], check_gemm, (BF, 64, 18944, 3584, MODE_SWIGLU)),              # a 7B layer's
-    (BF, ["gemm_rows<2,6,1>"], check_gemm, (BF, 33, 5600, 1024, MODE_SWIGLU)),
-    (BF, ["gemm_rows<2,7,1>"], check_gemm, (BF, 20, 24592, 64, MODE_SWIGLU)),
-    (BF, ["gemm_rows<2,8,1>"], check_gemm, (BF, 64, 28688, 64, MODE_SWIGLU)),
-    (BF, ["gemm_rows<1,2,0>", "gemm_split_reduce<3>"], check_gemm, (BF, 48, 130, 1024, MODE_STORE_F32, True)),   # N % 4 != 0
-    (BF, ["gemm_rows<1,4,0>", "gemm_split_reduce<1>"], check_then_norm, (64, 3584, 1024)),
-    (BF, ["gemm_rows<1,5,0>", "gemm_split_reduce<2>"], check_qkv_rope, (64, 28, 4, 128, 3584, 64)),
-    # more than 64 rows: tiles of the output through LDS
-    (BF, ["gemm_tile<128,128,2,2,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 100, 132, 2048, MODE_STORE, True)),
+    (BF, ["gemm_rows<1,4,2,0>"], check_gemm, (BF, 17, 100, 128, MODE_STORE, True)),
+    (BF, ["gemm_rows<1,4,3,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 33, 4100, 512, MODE_STORE_F32, True)),
+    (BF, ["gemm_rows<1,4,4,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 64, 3584, 1024, MODE_ADD_F32)),
+    (BF, ["gemm_rows<1,4,5,0>"], check_gemm, (BF, 40, 4100, 1024, MODE_STORE)),
+    (BF, ["gemm_rows<1,4,6,0>"], check_gemm, (BF, 20, 5600, 1024, MODE_STORE_F32)),
+    (BF, ["gemm_rows<1,4,7,0>"], check_gemm, (BF, 64, 6400, 1024, MODE_ADD_F32, True)),
+    (BF, ["gemm_rows<1,4,8,0>"], check_gemm, (BF, 48, 9600, 1024, MODE_STORE)),
+    (BF, ["gemm_rows<2,4,2,0>"], check_gemm, (BF, 17, 16384, 256, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,4,3,0>"], check_gemm, (BF, 64, 16400, 256, MODE_STORE_F32, True)),
+    (BF, ["gemm_rows<2,4,4,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 32, 16384, 512, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,4,5,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 17, 16400, 3584, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,4,6,0>"], check_gemm, (BF, 64, 20500, 512, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,4,7,0>"], check_gemm, (BF, 33, 50000, 256, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,4,8,0>"], check_gemm, (BF, 64, 152064, 3584, MODE_STORE_F32)),          # the head of a real model
+    (BF, ["gemm_rows<2,4,2,1>"], check_gemm, (BF, 40, 96, 64, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,4,3,1>"], check_gemm, (BF, 17, 8208, 64, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,4,4,1>", "gemm_split_reduce<0>"], check_gemm, (BF, 64, 3584, 1024, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,4,5,1>"], check_gemm, (BF, 64, 18944, 3584, MODE_SWIGLU)),              # a 7B layer's
+    (BF, ["gemm_rows<2,4,6,1>"], check_gemm, (BF, 33, 5600, 1024, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,4,7,1>"], check_gemm, (BF, 20, 24592, 64, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,4,8,1>"], check_gemm, (BF, 64, 28688, 64, MODE_SWIGLU)),
+    (BF, ["gemm_rows<1,4,2,0>", "gemm_split_reduce<3>"], check_gemm, (BF, 48, 130, 1024, MODE_STORE_F32, True)),   # N % 4 != 0
+    (BF, ["gemm_rows<1,4,4,0>", "gemm_split_reduce<1>"], check_then_norm, (64, 3584, 1024)),
+    (BF, ["gemm_rows<1,4,5,0>", "gemm_split_reduce<2>"], check_qkv_rope, (64, 28, 4, 128, 3584, 64)),
+    # 65 to 128 rows: the same kernel with eight tiles of 16 rows of X a step
+    (BF, ["gemm_rows<1,8,3,0>"], check_gemm, (BF, 65, 100, 128, MODE_STORE, True)),
+    (BF, ["gemm_rows<1,8,3,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 97, 4100, 512, MODE_STORE_F32, True)),
+    (BF, ["gemm_rows<1,8,4,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 128, 3584, 1024, MODE_ADD_F32)),
+    (BF, ["gemm_rows<1,8,5,0>"], check_gemm, (BF, 100, 4100, 1024, MODE_STORE)),
+    (BF, ["gemm_rows<1,8,6,0>"], check_gemm, (BF, 80, 5600, 1024, MODE_STORE_F32)),
+    (BF, ["gemm_rows<1,8,7,0>"], check_gemm, (BF, 128, 6400, 1024, MODE_ADD_F32, True)),
+    (BF, ["gemm_rows<1,8,8,0>"], check_gemm, (BF, 112, 9600, 1024, MODE_STORE)),
+    (BF, ["gemm_rows<2,8,3,0>"], check_gemm, (BF, 65, 16384, 256, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,8,3,0>"], check_gemm, (BF, 128, 16400, 256, MODE_STORE_F32, True)),
+    (BF, ["gemm_rows<2,8,4,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 96, 16384, 512, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,8,5,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 66, 16400, 3584, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,8,6,0>"], check_gemm, (BF, 128, 20500, 512, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,8,7,0>"], check_gemm, (BF, 97, 50000, 256, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,8,8,0>"], check_gemm, (BF, 127, 152064, 3584, MODE_STORE_F32)),
+    (BF, ["gemm_rows<2,8,3,1>"], check_gemm, (BF, 100, 96, 64, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,8,3,1>"], check_gemm, (BF, 65, 8208, 64, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,8,4,1>", "gemm_split_reduce<0>"], check_gemm, (BF, 128, 3584, 1024, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,8,5,1>"], check_gemm, (BF, 128, 18944, 3584, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,8,6,1>"], check_gemm, (BF, 97, 5600, 1024, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,8,7,1>"], check_gemm, (BF, 80, 24592, 64, MODE_SWIGLU)),
+    (BF, ["gemm_rows<2,8,8,1>"], check_gemm, (BF, 128, 28688, 64, MODE_SWIGLU)),
+    (BF, ["gemm_rows<1,8,3,0>", "gemm_split_reduce<3>"], check_gemm, (BF, 112, 130, 1024, MODE_STORE_F32, True)),   # N % 4 != 0
+    (BF, ["gemm_rows<1,8,4,0>", "gemm_split_reduce<1>"], check_then_norm, (128, 3584, 1024)),
+    (BF, ["gemm_rows<1,8,5,0>", "gemm_split_reduce<2>"], check_qkv_rope, (128, 28, 4, 128, 3584, 64)),
+    # more than 128 rows: tiles of the output through LDS
+    (BF, ["gemm_tile<128,128,2,2,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 140, 132, 2048, MODE_STORE, True)),
     (BF, ["gemm_tile<128,128,2,2,0>", "gemm_split_reduce<3>"], check_gemm, (BF, 200, 130, 1024, MODE_ADD_F32)),
     (BF, ["gemm_tile<128,128,2,2,1>", "gemm_split_reduce<0>"], check_gemm, (BF, 130, 96, 2048, MODE_SWIGLU)),
     (BF, ["gemm_tile<256,192,4,2,0>"], check_gemm, (BF, 2048, 4608, 192, MODE_STORE, True)),
     (BF, ["gemm_tile<256,256,4,2,0>"], check_gemm, (BF, 1100, 9300, 128, MODE_STORE_F32)),
     (BF, ["gemm_tile<256,256,4,2,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 2049, 3584, 3584, MODE_ADD_F32)),
     (BF, ["gemm_tile<256,256,4,2,1>"], check_gemm, (BF, 2048, 2608, 64, MODE_SWIGLU)),
-    (BF, ["gemm_tile<128,128,2,2,0>", "gemm_split_reduce<1>"], check_then_norm, (100, 256, 1024)),
+    (BF, ["gemm_tile<128,128,2,2,0>", "gemm_split_reduce<1>"], check_then_norm, (150, 256, 1024)),
     (BF, ["gemm_tile<256,256,4,2,0>", "gemm_split_reduce<2>"], check_qkv_rope, (2048, 28, 4, 128, 3584, 64)),
     # attention on the matrix cores: (head size, query heads a block, pages of 64 positions or more)
     # and (head size, waves a block) (one wave a block in the decoding kernel up to 2,560 blocks of
