@@ -39,31 +39,26 @@ gemm_fma_kernel(const elem_t* __restrict__ x, int x_stride, const elem_t* __rest
       if (GLU) acc_up[i][j] = 0.0f;
     }
 
-  // loader: each thread brings 4 consecutive k of one row
+  // loader: each thread brings 4 consecutive k of one row, a step ahead of the products
   const int lrow = tid >> 2, lk = (tid & 3) * 4;
+  float pw[4], pu[4], px[4];
+  auto fetch = [&](int k0) {
+    const int n = n0 + lrow, m = m0 + lrow;
+    const int left = max(0, min(4, K - (k0 + lk)));
+    load4_guarded(w + (size_t)n * K + k0 + lk, n < N ? left : 0, vec_w, pw);
+    if (GLU) load4_guarded(w + (size_t)(N + n) * K + k0 + lk, n < N ? left : 0, vec_w, pu);
+    if (lrow < BM) load4_guarded(x + (size_t)m * x_stride + k0 + lk, m < M ? left : 0, vec_x, px);
+  };
+  fetch(0);
   for (int k0 = 0; k0 < K; k0 += FMA_BK) {
-    {
-      float v[4];
-      const int n = n0 + lrow;
-      const int valid = n < N ? min(4, K - (k0 + lk)) : 0;
-      load4_guarded(w + (size_t)n * K + k0 + lk, valid > 0 ? valid : 0, vec_w, v);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) ws[lk + i][lrow] = v[i];
-      if (GLU) {
-        load4_guarded(w + (size_t)(N + n) * K + k0 + lk, valid > 0 ? valid : 0, vec_w, v);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) us[lk + i][lrow] = v[i];
-      }
-    }
-    if (lrow < BM) {
-      float v[4];
-      const int m = m0 + lrow;
-      const int valid = m < M ? min(4, K - (k0 + lk)) : 0;
-      load4_guarded(x + (size_t)m * x_stride + k0 + lk, valid > 0 ? valid : 0, vec_x, v);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) xs[lk + i][lrow] = v[i];
+    for (int i = 0; i < 4; ++i) {
+      ws[lk + i][lrow] = pw[i];
+      if (GLU) us[lk + i][lrow] = pu[i];
+      if (lrow < BM) xs[lk + i][lrow] = px[i];
     }
     __syncthreads();
+    if (k0 + FMA_BK < K) fetch(k0 + FMA_BK);
 #pragma unroll
     for (int kk = 0; kk < FMA_BK; ++kk) {
       float a[RM], b[4];
