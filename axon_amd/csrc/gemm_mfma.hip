@@ -540,7 +540,7 @@ static int launch_tile(const bf16_t* x, int x_stride, const bf16_t* w, const voi
   // a block a segment (gridDim.y), the sums through `partial`
   const int splits = segs;
   const int m_blocks = ceil_div(m, BM), n_blocks = ceil_div(n, GLU ? BN / 2 : BN);
-  AXK_INSTANCE(INST_GEMM_TILE, BM, BN, WAVES_M, WAVES_N, GLU);
+  AXK_INSTANCE(INST_GEMM_TILE, BM, BN, WAVES_M, WAVES_N, GLU, STAGES);
   kernel<<<dim3(m_blocks * n_blocks, splits), WAVES_M * WAVES_N * 64, lds_bytes, stream>>>(
       x, x_stride, w, bias, bias_is_f32, out, out_stride, m, n, k, mode, m_blocks, n_blocks, splits > 1 ? partial : nullptr);
   AXK_LAUNCH_CHECK("gemm_tile");
@@ -1735,10 +1735,6 @@ static int gemm_mfma_pass(const bf16_t* x, int x_stride, const bf16_t* w, const 
     if (n >= 32 * 512) return launch_rows<2, 8, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
     return launch_rows<1, 8, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
   }
-  if (m <= 256) {
-    if (glu) return launch_tile<128, 128, 2, 2, true>(ARGS, segs, ws);
-    return launch_tile<128, 128, 2, 2, false>(ARGS, segs, ws, norm, rope_after);
-  }
   // 256 x 256 tiles (8 waves) where they fill the chip: one round of at least 140 blocks (on 256
   // CUs), or several rounds of which the last is not mostly idle; else 128 x 128 tiles, four times
   // as many blocks at twice the traffic from L2 per product.  Thresholds are measured ones.
@@ -1746,6 +1742,19 @@ static int gemm_mfma_pass(const bf16_t* x, int x_stride, const bf16_t* w, const 
   const long big = (long)ceil_div(m, 256) * ceil_div(n, n_per_block) * segs;
   const long rounds = (big + 255) / 256;
   const bool use_big = big <= 256 ? big >= 140 : big * 10 >= rounds * 256 * 7;
+  if (m <= 256 && !(glu && use_big)) {
+    // So few rows still wait for W more than for the matrix cores.  Where the 128 x 128 tiles are no
+    // more blocks than CUs, a block has its CU's LDS to itself: four stages instead of two, three
+    // steps of loads in flight (the down projection of a 7B layer at 256 rows 79 -> 64 us); with
+    // more blocks two of them share a CU and cover each other's waits (four stages there: slower).
+    const bool deep = (long)ceil_div(m, 128) * ceil_div(n, glu ? 64 : 128) * segs <= 256;
+    if (glu) {
+      if (deep) return launch_tile<128, 128, 2, 2, true, 64, 4>(ARGS, segs, ws);
+      return launch_tile<128, 128, 2, 2, true>(ARGS, segs, ws);
+    }
+    if (deep) return launch_tile<128, 128, 2, 2, false, 64, 4>(ARGS, segs, ws, norm, rope_after);
+    return launch_tile<128, 128, 2, 2, false>(ARGS, segs, ws, norm, rope_after);
+  }
   if (glu) {
     if (use_big) return launch_tile<256, 256, 4, 2, true>(ARGS, segs, ws);
     return launch_tile<128, 128, 2, 2, true>(ARGS, segs, ws);

@@ -17,7 +17,7 @@
 
 enum {
   INST_GEMM_FMA = 0,
-  INST_GEMM_TILE,            // BM, BN, waves m, waves n, gated, BK, stages, segments in registers
+  INST_GEMM_TILE,            // BM, BN, waves m, waves n, gated, stages
   INST_GEMM_STREAM,          // row tiles, tiles of X rows, segments, epilogue
   INST_GEMM_NORMED,          // tile pairs a wave, segments, epilogue, rows of X in LDS, float4 a lane
   INST_GEMM_ROWS,            // row tiles of W a wave, tiles of 16 rows of X, waves, epilogue

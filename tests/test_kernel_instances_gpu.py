@@ -344,15 +344,22 @@ CASES = [
     (BF, ["gemm_rows<1,8,4,0>", "gemm_split_reduce<1>"], check_then_norm, (128, 3584, 1024)),
     (BF, ["gemm_rows<1,8,5,0>", "gemm_split_reduce<2>"], check_qkv_rope, (128, 28, 4, 128, 3584, 64)),
     # more than 128 rows: tiles of the output through LDS
-    (BF, ["gemm_tile<128,128,2,2,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 140, 132, 2048, MODE_STORE, True)),
-    (BF, ["gemm_tile<128,128,2,2,0>", "gemm_split_reduce<3>"], check_gemm, (BF, 200, 130, 1024, MODE_ADD_F32)),
-    (BF, ["gemm_tile<128,128,2,2,1>", "gemm_split_reduce<0>"], check_gemm, (BF, 130, 96, 2048, MODE_SWIGLU)),
-    (BF, ["gemm_tile<256,192,4,2,0>"], check_gemm, (BF, 2048, 4608, 192, MODE_STORE, True)),
-    (BF, ["gemm_tile<256,256,4,2,0>"], check_gemm, (BF, 1100, 9300, 128, MODE_STORE_F32)),
-    (BF, ["gemm_tile<256,256,4,2,0>", "gemm_split_reduce<0>"], check_gemm, (BF, 2049, 3584, 3584, MODE_ADD_F32)),
-    (BF, ["gemm_tile<256,256,4,2,1>"], check_gemm, (BF, 2048, 2608, 64, MODE_SWIGLU)),
-    (BF, ["gemm_tile<128,128,2,2,0>", "gemm_split_reduce<1>"], check_then_norm, (150, 256, 1024)),
-    (BF, ["gemm_tile<256,256,4,2,0>", "gemm_split_reduce<2>"], check_qkv_rope, (2048, 28, 4, 128, 3584, 64)),
+    # (129 to 256 rows in no more blocks than CUs: four stages)
+    (BF, ["gemm_tile<128,128,2,2,0,4>", "gemm_split_reduce<0>"], check_gemm, (BF, 140, 132, 2048, MODE_STORE, True)),
+    (BF, ["gemm_tile<128,128,2,2,0,4>", "gemm_split_reduce<3>"], check_gemm, (BF, 200, 130, 1024, MODE_ADD_F32)),
+    (BF, ["gemm_tile<128,128,2,2,1,4>", "gemm_split_reduce<0>"], check_gemm, (BF, 130, 96, 2048, MODE_SWIGLU)),
+    (BF, ["gemm_tile<128,128,2,2,0,4>", "gemm_split_reduce<0>"], check_gemm, (BF, 256, 3584, 18944, MODE_ADD_F32)),  # a 7B layer's
+    (BF, ["gemm_tile<128,128,2,2,0,2>", "gemm_split_reduce<0>"], check_gemm, (BF, 200, 4608, 3584, MODE_STORE, True)),
+    (BF, ["gemm_tile<128,128,2,2,0,2>", "gemm_split_reduce<3>"], check_gemm, (BF, 300, 130, 1024, MODE_ADD_F32)),
+    (BF, ["gemm_tile<128,128,2,2,1,2>", "gemm_split_reduce<0>"], check_gemm, (BF, 300, 96, 2048, MODE_SWIGLU)),
+    (BF, ["gemm_tile<128,128,2,2,1,2>"], check_gemm, (BF, 200, 8320, 256, MODE_SWIGLU)),
+    (BF, ["gemm_tile<256,192,4,2,0,2>"], check_gemm, (BF, 2048, 4608, 192, MODE_STORE, True)),
+    (BF, ["gemm_tile<256,256,4,2,0,2>"], check_gemm, (BF, 1100, 9300, 128, MODE_STORE_F32)),
+    (BF, ["gemm_tile<256,256,4,2,0,2>", "gemm_split_reduce<0>"], check_gemm, (BF, 2049, 3584, 3584, MODE_ADD_F32)),
+    (BF, ["gemm_tile<256,256,4,2,1,2>"], check_gemm, (BF, 2048, 2608, 64, MODE_SWIGLU)),
+    (BF, ["gemm_tile<128,128,2,2,0,4>", "gemm_split_reduce<1>"], check_then_norm, (150, 256, 1024)),
+    (BF, ["gemm_tile<256,256,4,2,1,2>"], check_gemm, (BF, 200, 18944, 3584, MODE_SWIGLU)),              # a 7B layer's at 200 rows
+    (BF, ["gemm_tile<256,256,4,2,0,2>", "gemm_split_reduce<2>"], check_qkv_rope, (2048, 28, 4, 128, 3584, 64)),
     # attention on the matrix cores: (head size, query heads a block, pages of 64 positions or more)
     # and (head size, waves a block) (one wave a block in the decoding kernel up to 2,560 blocks of
     # positions, four beyond; two heads a block in the prompt kernel from 200 such blocks on: the long
