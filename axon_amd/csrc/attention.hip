@@ -189,7 +189,7 @@ attention_rows_kernel(const elem_t* __restrict__ q, int q_stride, const elem_t* 
       }
       M = mn;
     }
-    if (WAVES > 1) __syncthreads();   // the next round writes `part` again
+    if (WAVES > 1) __syncthreads();   // the loop's next turn writes `part` again
   }
 
   if (wave != 0) return;

@@ -119,7 +119,7 @@ def test_attention_over_the_paged_cache(dtype, nh, nkv, hd, page, T, window):
                 1.0 / math.sqrt(hd))
     assert torch.equal(one[0], out[T - 1])
     # pages of another size, one that goes through LDS in whole loads if this one does not (a
-    # multiple of 4 positions does) and the other way round: the same bits
+    # multiple of 4 positions does) and vice versa: the same bits
     other = page + 1 if page % 4 == 0 else 4 * page
     kc2, vc2, table2 = paged_cache(kr, vr, other, dtype)
     out2 = torch.empty_like(out)
