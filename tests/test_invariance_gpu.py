@@ -126,6 +126,42 @@ def test_a_replayed_graph_gives_the_bits_of_the_step_launched_kernel_by_kernel(n
         assert torch.equal(with_graph, without)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["D", "E"])
+def test_a_decoding_row_has_the_same_bits_among_two_hundred_rows_as_among_few(name, dtype, model_dirs):
+    """Two hundred requests decode a token each: all in one step, in steps of 100, 70 and 30, and in
+    steps of 17, 1, 64, 65 and 53 rows, so that every product takes each of its kernels (up to 16
+    rows, up to 64, up to 128, more).  A request's logits and cache rows are the same bits."""
+    d = model_dirs(name, "float32" if dtype == "float32" else "bfloat16")
+    page = TINY[name]["page_size"]
+    n = 200
+    lengths = [3 + (7 * i) % 23 for i in range(n)]
+    prompts = prompts_for(name, lengths, seed=5)
+    pages = sum(-(-(length + 1) // page) for length in lengths) + 8
+
+    def decode(groups):
+        eng = engine_for(d, dtype, page, pages, max_seqs=n, max_batch_tokens=4096)
+        for first in range(0, n, 50):                               # the prompts, fifty requests a step
+            eng.step([StepEntry(f"r{i}", prompts[i][:-1], []) for i in range(first, first + 50)])
+        rows, at = {}, 0
+        for size in groups:
+            ids = list(range(at, at + size))
+            logits = eng.step([StepEntry(f"r{i}", prompts[i][-1:], [0]) for i in ids])
+            for j, i in enumerate(ids):
+                rows[i] = logits[j].clone()
+            at += size
+        assert at == n
+        return rows, [cache_rows(eng, f"r{i}") for i in (0, 16, 17, 99, 100, 199)]
+
+    whole, whole_cache = decode([n])
+    for groups in ([100, 70, 30], [17, 1, 64, 65, 53]):
+        got, got_cache = decode(groups)
+        for i in range(n):
+            assert torch.equal(got[i], whole[i]), f"request {i} in steps of {groups}"
+        for a, b in zip(got_cache, whole_cache):
+            assert torch.equal(a, b)
+
+
 def grade(ref: torch.Tensor, got: torch.Tensor):
     """max |difference| relative to the logits' range, top-1 agreement, mean KL(ref || got)."""
     ref, got = ref.double(), got.double()
