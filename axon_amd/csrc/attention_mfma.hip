@@ -880,10 +880,11 @@ extern "C" int axk_attention_prefill(const void* q, int q_stride, const void* k_
   }
 #define LAUNCH(HD, HPB) \
   if (page_size >= ATT_BLOCK) LAUNCH_PAGED(HD, HPB, 1) else LAUNCH_PAGED(HD, HPB, 0)
-  // two query heads of a kv head a block (they share each K and V block in LDS) where that still
-  // gives the chip's 256 CUs about a block each; else one head a block
-  const int blocks_of_pairs = n_tiles * n_kv_heads * ((group + 1) / 2);
-  if (group >= 2 && blocks_of_pairs >= 200) {
+  // one query head a block while such blocks find a CU each (256 of them); beyond that two query
+  // heads of a kv head a block, which share each K and V block in LDS and whose waves fill each
+  // other's waits (7B sizes: 2,304 tokens 88 against 101 us with one head, 2,560 tokens 123 against
+  // 109 us with two; 14B sizes at 2,048 tokens 101 against 88 us)
+  if (group >= 2 && (long)n_tiles * n_heads > 256) {
     if (head_dim == 64) LAUNCH(64, 2) else LAUNCH(128, 2)
   } else {
     if (head_dim == 64) LAUNCH(64, 1) else LAUNCH(128, 1)

@@ -362,8 +362,8 @@ CASES = [
     (BF, ["gemm_tile<256,256,4,2,0,2>", "gemm_split_reduce<2>"], check_qkv_rope, (2048, 28, 4, 128, 3584, 64)),
     # attention on the matrix cores: (head size, query heads a block, pages of 64 positions or more)
     # and (head size, waves a block) (one wave a block in the decoding kernel up to 2,560 blocks of
-    # positions, four beyond; two heads a block in the prompt kernel from 200 such blocks on: the long
-    # prompts of real models)
+    # positions, four beyond; two heads a block in the prompt kernel where tiles x heads are more
+    # than 256: the long prompts of real models)
     (BF, ["attention_prefill<64,1,0>", "attention_decode<64,1>"], check_attention_mfma, (4, 2, 64, 16, 200, 0)),
     (BF, ["attention_prefill<64,1,1>"], check_attention_mfma, (4, 2, 64, 64, 200, 0)),
     (BF, ["attention_prefill<128,1,1>", "attention_decode<128,1>"], check_attention_mfma, (7, 1, 128, 64, 333, 90)),
