@@ -1735,19 +1735,21 @@ static int gemm_mfma_pass(const bf16_t* x, int x_stride, const bf16_t* w, const 
     if (n >= 32 * 512) return launch_rows<2, 8, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
     return launch_rows<1, 8, EPI_PLAIN>(ARGS, segs, ws, norm, rope_after);
   }
-  // 256 x 256 tiles (8 waves) where they fill the chip: one round of at least 140 blocks (on 256
-  // CUs), or several rounds of which the last is not mostly idle; else 128 x 128 tiles, four times
-  // as many blocks at twice the traffic from L2 per product.  Thresholds are measured ones.
-  const int n_per_block = glu ? 128 : 256;
-  const long big = (long)ceil_div(m, 256) * ceil_div(n, n_per_block) * segs;
-  const long rounds = (big + 255) / 256;
-  const bool use_big = big <= 256 ? big >= 140 : big * 10 >= rounds * 256 * 7;
-  if (m <= 256 && !(glu && use_big)) {
-    // So few rows still wait for W more than for the matrix cores.  Where the 128 x 128 tiles are no
+  // 256 x 256 tiles (8 waves, a block a CU) or 128 x 128 tiles (4 waves, two blocks a CU, four
+  // times as many blocks at twice the traffic from L2 per product): whichever takes the chip's 256
+  // CUs fewer rounds, a round of the small tiles counted as 0.65 of a round of the large ones
+  // (measured on the four products of the 7B and 14B layers at 200 to 2,048 rows: the rule picks
+  // the faster tile in 66 of 70 cases and loses 7 % at most in the others).
+  const long big = (long)ceil_div(m, 256) * ceil_div(n, glu ? 128 : 256) * segs;
+  const long small = (long)ceil_div(m, 128) * ceil_div(n, glu ? 64 : 128) * segs;
+  const long rounds_big = (big + 255) / 256, rounds_small = (small + 511) / 512;
+  const bool use_big = rounds_big * 100 <= rounds_small * 65;
+  if (!use_big) {
+    // Up to 256 rows still wait for W more than for the matrix cores.  Where the small tiles are no
     // more blocks than CUs, a block has its CU's LDS to itself: four stages instead of two, three
     // steps of loads in flight (the down projection of a 7B layer at 256 rows 79 -> 64 us); with
     // more blocks two of them share a CU and cover each other's waits (four stages there: slower).
-    const bool deep = (long)ceil_div(m, 128) * ceil_div(n, glu ? 64 : 128) * segs <= 256;
+    const bool deep = m <= 256 && small <= 256;
     if (glu) {
       if (deep) return launch_tile<128, 128, 2, 2, true, 64, 4>(ARGS, segs, ws);
       return launch_tile<128, 128, 2, 2, true>(ARGS, segs, ws);
@@ -1755,17 +1757,13 @@ static int gemm_mfma_pass(const bf16_t* x, int x_stride, const bf16_t* w, const 
     if (deep) return launch_tile<128, 128, 2, 2, false, 64, 4>(ARGS, segs, ws, norm, rope_after);
     return launch_tile<128, 128, 2, 2, false>(ARGS, segs, ws, norm, rope_after);
   }
-  if (glu) {
-    if (use_big) return launch_tile<256, 256, 4, 2, true>(ARGS, segs, ws);
-    return launch_tile<128, 128, 2, 2, true>(ARGS, segs, ws);
-  }
+  if (glu) return launch_tile<256, 256, 4, 2, true>(ARGS, segs, ws);
   // one round of 256 x 256 tiles that leaves a quarter of the CUs idle, and N in whole tiles of
   // 192 columns that still fit one round: the narrower tile (measured 1.1 times the cost per
   // product, three quarters of the products per block).
-  if (use_big && segs == 1 && big <= 192 && n % 192 == 0 && (long)ceil_div(m, 256) * (n / 192) <= 256)
+  if (segs == 1 && big <= 192 && n % 192 == 0 && (long)ceil_div(m, 256) * (n / 192) <= 256)
     return launch_tile<256, 192, 4, 2, false>(ARGS, segs, ws, norm);
-  if (use_big) return launch_tile<256, 256, 4, 2, false>(ARGS, segs, ws, norm, rope_after);
-  return launch_tile<128, 128, 2, 2, false>(ARGS, segs, ws, norm, rope_after);
+  return launch_tile<256, 256, 4, 2, false>(ARGS, segs, ws, norm, rope_after);
 #undef ARGS
 }
 
