@@ -28,6 +28,8 @@
 // position-contiguous: [page][kv head][dim][slot]).
 #include <math.h>
 
+#include <type_traits>
+
 #include "api.h"
 #include "common.h"
 #include "instances.h"
@@ -769,7 +771,8 @@ __global__ void __launch_bounds__(HD)
 attention_combine_kernel(const float* __restrict__ partial, const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ token_index, bf16_t* __restrict__ out, int max_chunks, int n_heads,
                          int window) {
-  __shared__ float block_max[HD], block_sum[HD], old_factor[HD], new_factor[HD], wave_max[HD / 64];
+  __shared__ float block_max[HD], block_sum[HD], wave_max[HD / 64];
+  __shared__ __align__(16) float old_factor[HD], new_factor[HD], scaled_sum[HD];   // a, b, and l_b b, of the group's blocks
   const int t = token_index ? token_index[blockIdx.x] : blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
@@ -807,24 +810,38 @@ attention_combine_kernel(const float* __restrict__ partial, const int32_t* __res
         attention_fold(before, unused, mine, 0.0f, fa, fb);
         old_factor[d] = fa;
         new_factor[d] = fb;
+        scaled_sum[d] = __fmul_rn(block_sum[d], fb);
       }
     }
     __syncthreads();
+    // the fold is a chain, the loads are not: thirty-two blocks' values under way at a time where
+    // that many are left, then sixteen; the blocks' factors come from LDS four at a time
     int i = 0;
-    for (; i + 15 < n; i += 16) {              // sixteen blocks' values under way at a time
-      float ob[16];
+    auto fold_batch = [&](auto count) {
+      constexpr int COUNT = decltype(count)::value;
+      for (; i + COUNT - 1 < n; i += COUNT) {
+        float ob[COUNT];
 #pragma unroll
-      for (int j = 0; j < 16; ++j) ob[j] = src[(size_t)(g0 + i + j) * (HD + 2) + d];
+        for (int j = 0; j < COUNT; ++j) ob[j] = src[(size_t)(g0 + i + j) * (HD + 2) + d];
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const float fa = old_factor[i + j], fb = new_factor[i + j];
-        l = __builtin_fmaf(l, fa, __fmul_rn(block_sum[i + j], fb));
-        attention_fold_into(o, fa, ob[j], fb);
+        for (int q = 0; q < COUNT / 4; ++q) {
+          const float4 fa = *reinterpret_cast<const float4*>(&old_factor[i + 4 * q]);
+          const float4 fb = *reinterpret_cast<const float4*>(&new_factor[i + 4 * q]);
+          const float4 ls = *reinterpret_cast<const float4*>(&scaled_sum[i + 4 * q]);
+          const float a4[4] = {fa.x, fa.y, fa.z, fa.w}, b4[4] = {fb.x, fb.y, fb.z, fb.w}, l4[4] = {ls.x, ls.y, ls.z, ls.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            l = __builtin_fmaf(l, a4[e], l4[e]);
+            attention_fold_into(o, a4[e], ob[4 * q + e], b4[e]);
+          }
+        }
       }
-    }
+    };
+    fold_batch(std::integral_constant<int, 32>());
+    fold_batch(std::integral_constant<int, 16>());
     for (; i < n; ++i) {
       const float fa = old_factor[i], fb = new_factor[i];
-      l = __builtin_fmaf(l, fa, __fmul_rn(block_sum[i], fb));
+      l = __builtin_fmaf(l, fa, scaled_sum[i]);
       attention_fold_into(o, fa, src[(size_t)(g0 + i) * (HD + 2) + d], fb);
     }
     for (int w = 0; w < HD / 64; ++w) m = fmaxf(m, wave_max[w]);     // blocks past n count as -inf
