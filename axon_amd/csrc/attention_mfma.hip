@@ -88,10 +88,13 @@ __device__ __forceinline__ int page_offset(int p, int page_size) { return p & (p
 
 // The page a lane's piece of load instruction `instr` lies in (looked up ahead of the load that
 // uses it).  Positions past `hi` (never written for this request): any valid row.
+// (K: an instruction's 4 or 8 rows lie in one page, pages holding at least 8 positions, and rows
+// past `hi` read row `hi`, which lies in the page of the instruction's first row or before every
+// row of it: the page is the wave's, looked up once, and the address a scalar base plus an offset.)
 template <int HD>
 __device__ __forceinline__ int att_k_page(int instr, int lane, int p0, int hi, const int32_t* table_row, int page_size) {
-  const int row = instr * AttStage<HD>::K_ROWS_PER_INSTR + lane / AttStage<HD>::KCH;
-  return table_row[page_index(min(p0 + row, hi), page_size)];
+  const int row0 = instr * AttStage<HD>::K_ROWS_PER_INSTR;
+  return table_row[page_index(min(p0 + row0, hi), page_size)];
 }
 
 template <int HD>
@@ -456,7 +459,7 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
   // them, so that no load waits for a table entry behind the loads issued just before it.
   // ONE_PAGE (pages of 64 positions or more): a block lies in one page, known to the whole wave,
   // and the addresses are a scalar base plus a lane's 32-bit offset.
-  int k_page[K_INSTR], v_page[V_INSTR];
+  int k_page[K_INSTR], v_page[1];
   auto lookup_k = [&](int b) {
     const int p0 = first_block + b * ATT_BLOCK;
     if (ONE_PAGE) {
@@ -472,8 +475,10 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
       v_page[0] = table_row[page_index(p0, page_size)];
       return;
     }
-#pragma unroll
-    for (int n = 0; n < V_INSTR; ++n) v_page[n] = att_v_page<HD>(n * NW + block_wave, lane, p0, hi, table_row, page_size);
+    // the 8 positions a lane brings depend on the instruction through its parity alone (the
+    // permutation of a V^T row's slots), and a wave's instructions are NW apart: one page for all
+    static_assert(NW % 2 == 0, "a wave's load instructions have one parity");
+    v_page[0] = att_v_page<HD>(block_wave, lane, p0, hi, table_row, page_size);
   };
   auto issue_k = [&](int b) {
     unsigned char* stage = smem + (b & 1) * S::BYTES;
@@ -488,8 +493,7 @@ attention_prefill_tile(unsigned char* smem, int t0, int count, const bf16_t* __r
     const int p0 = first_block + b * ATT_BLOCK;
 #pragma unroll
     for (int n = 0; n < V_INSTR; ++n)
-      att_issue_v<HD>(stage, n * NW + block_wave, lane, ONE_PAGE ? v_page[0] : v_page[n], p0, hi, v_head, page_stride,
-                      page_size);
+      att_issue_v<HD>(stage, n * NW + block_wave, lane, v_page[0], p0, hi, v_head, page_stride, page_size);
   };
 
   float o_acc[DT][16];              // (plain registers: the fold below names each as an instruction's operand)
