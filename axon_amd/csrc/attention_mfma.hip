@@ -218,11 +218,12 @@ __device__ __forceinline__ void attention_weights(f32x16 (&s_acc)[2], int p0, bo
         s_acc[pt][e] = seen ? s_acc[pt][e] : -INFINITY;
       }
   }
-  float mloc = -INFINITY;
+  float mpt[2] = {-INFINITY, -INFINITY};      // a chain a tile: the maximum does not depend on the order
 #pragma unroll
   for (int pt = 0; pt < 2; ++pt)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) mloc = fmaxf(mloc, s_acc[pt][e]);
+    for (int e = 0; e < 16; ++e) mpt[pt] = fmaxf(mpt[pt], s_acc[pt][e]);
+  float mloc = fmaxf(mpt[0], mpt[1]);
   mloc = fmaxf(mloc, __shfl_xor(mloc, 32, AXON_WAVE));
   m_b = __fmul_rn(mloc, c);
   const float mref = m_b == -INFINITY ? 0.0f : m_b;     // a column that sees nothing of this block
